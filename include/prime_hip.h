@@ -1,0 +1,117 @@
+/*
+ * prime_hip.h - C ABI of libprime_hip.so: the int8 (uint8 code + 256-entry fp32 lookup)
+ * pseudo-gradient compression path on MI355X (gfx950).
+ *
+ * Every entry point enqueues HIP kernels on `stream` (a hipStream_t passed as void*; NULL is
+ * the default stream) and returns without synchronising.  All pointers are device pointers
+ * unless a comment says otherwise.  The library never allocates or frees memory: the caller
+ * owns inputs, outputs and the workspace.  Return value: 0 on success, a positive hipError_t
+ * on a HIP failure, a negative PRIME_E* on a rejected argument; prime_hip_last_error() gives
+ * the text for the calling thread.
+ *
+ * Reference interfaces these entry points stand in for (paths relative to the reference
+ * checkout) are cited per function.  n_bins is 256 and zero_point 128 throughout
+ * (src/zeroband/C/csrc/compression.cpp:5,107) unless passed explicitly.
+ */
+#ifndef PRIME_HIP_H
+#define PRIME_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PRIME_HIP_ABI_VERSION 1
+
+#define PRIME_EINVAL (-1)   /* null pointer, negative size, bad n_bins ... */
+#define PRIME_EWORKSPACE (-2) /* workspace missing, too small or not initialised */
+
+typedef void* prime_stream_t; /* hipStream_t */
+
+/* What the statistics pass leaves on the device for the quantizer (32 bytes). */
+typedef struct prime_qparams {
+    float scale;      /* float(6 * std / 256), compression.cpp:116,119 */
+    float inv_scale;  /* 1.0f / scale, compression.cpp:16 */
+    double sum;       /* sum of x   (fp64) */
+    double sumsq;     /* sum of x*x (fp64) */
+    int64_t n;
+} prime_qparams;
+
+int prime_hip_abi_version(void);
+const char* prime_hip_last_error(void);
+
+/* Tuning knobs ("blocks_per_cu", "hist_mode", "reverse_second_pass", ...); returns 0 if known. */
+int prime_hip_set_option(const char* name, int value);
+int prime_hip_get_option(const char* name, int* value);
+
+/* Workspace: a fixed-size block of ordinary device memory (hipMalloc / torch allocator;
+ * not fine-grained or host memory: hardware fp64 atomics are used on it).  It holds
+ * per-block partial sums, the grid-level ticket and the 256-bin accumulators.  Initialise it
+ * once with prime_workspace_init (a fill kernel, safe under stream capture); every entry
+ * point leaves it ready for the next call.  Two calls that share a workspace must be
+ * ordered on one stream. */
+int64_t prime_workspace_bytes(void);
+int prime_workspace_init(void* ws, int64_t ws_bytes, prime_stream_t stream);
+
+/* Sum and sum of squares in fp64 plus the quantization scale, written to *out (device).
+ * Stands in for `tensor.norm()` and the scale formula of uniform_8bit_quantize,
+ * src/zeroband/C/csrc/compression.cpp:113-116. */
+int prime_stats_f32(const float* x, int64_t n, prime_qparams* out, void* ws, prime_stream_t stream);
+
+/* codes[i] = clamp(int32(round(x[i] * (1.0f / scale))) + zero_point, 0, 255), round half away
+ * from zero.  Stands in for quantize_per_tensor_multithreaded, compression.cpp:9-43
+ * (pybind name quantize_per_tensor_uint8, compression.cpp:146-154). */
+int prime_quantize_u8(const float* x, int64_t n, float scale, int32_t zero_point, uint8_t* codes,
+                      prime_stream_t stream);
+
+/* lut[b] = mean of x[i] over codes[i] == b, 0.0f for an empty bin, b < n_bins; codes >= n_bins
+ * are skipped.  Stands in for average_buckets_multithread, compression.cpp:45-104 (pybind name
+ * average_buckets, compression.cpp:130-138).  lut has n_bins entries; n_bins >= 1.
+ * counts (optional, 256 x uint64) receives the bin populations of bins < min(n_bins, 256). */
+int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64_t n_bins, float* lut,
+                          uint64_t* counts, void* ws, prime_stream_t stream);
+
+/* Quantize with a caller-supplied scale and build the lookup table in the same pass
+ * (compression.cpp:119 + :122 with the scale of :116 given).  lut has 256 entries. */
+int prime_quantize_lookup_u8(const float* x, int64_t n, float scale, uint8_t* codes, float* lut,
+                             void* ws, prime_stream_t stream);
+
+/* The whole of uniform_8bit_quantize, compression.cpp:106-125: statistics pass, then the fused
+ * quantize + lookup pass.  qparams_out (optional, device) receives scale and sums. */
+int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float* lut,
+                                prime_qparams* qparams_out, void* ws, prime_stream_t stream);
+
+/* Many tensors in one launch: tensor t is x[offsets[t] .. offsets[t+1]) of a flat buffer, the
+ * layout of the per-layer views of Diloco's flat pseudo-gradient buffer
+ * (src/zeroband/diloco.py:147-201), each handled as uniform_8bit_quantize handles one tensor.
+ * offsets: count+1 int64 on the device.  codes uses the same offsets; luts is count x 256;
+ * qparams_out (optional) is count entries.  Meant for small tensors: one workgroup each. */
+int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, int64_t count,
+                                        uint8_t* codes, float* luts, prime_qparams* qparams_out,
+                                        prime_stream_t stream);
+
+/* out[i] = lut[codes[i]]: fast_index_set_omp<float>, src/zeroband/C/csrc/collectives.cpp:16-22. */
+int prime_dequant_set(float* out, const float* lut, const uint8_t* codes, int64_t n,
+                      prime_stream_t stream);
+
+/* out[i] += lut[codes[i]]: fast_index_add_omp<float>, collectives.cpp:8-14. */
+int prime_dequant_add(float* out, const float* lut, const uint8_t* codes, int64_t n,
+                      prime_stream_t stream);
+
+/* One hop of the ring's reduce-scatter as ring_allreduce runs it on a received chunk,
+ * collectives.cpp:124-138: acc[i] += lut_in[codes_in[i]] (fast_index_add_omp), then
+ * (codes_out, lut_out) = uniform_8bit_quantize(acc).  The sum of squares of the updated acc is
+ * taken in the accumulate pass, so acc is read twice and written once. */
+int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut_in, int64_t n,
+                           uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out,
+                           void* ws, prime_stream_t stream);
+
+/* A plain device copy of n bytes (16-byte vectors): the yardstick the profiler's byte
+ * counters are scaled against.  No counterpart in the reference. */
+int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PRIME_HIP_H */

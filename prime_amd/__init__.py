@@ -1,0 +1,13 @@
+"""prime_amd: the int8 pseudo-gradient compression path of prime (ZeroBand) on MI355X.
+
+Layout
+    csrc/            HIP kernels and the C ABI (libprime_hip.so; include/prime_hip.h)
+    _lib.py          ctypes binding of the C ABI
+    ops.py           torch.library ops over it
+    C/compression.py, C/collectives.py, collectives.py, config.py
+                     the reference's module and function names for this path
+    ring.py          the ring's per-hop compute for W simulated ranks on one GPU
+"""
+from .config import Compression  # noqa: F401
+
+__all__ = ["Compression"]

@@ -1,0 +1,258 @@
+"""``torch.library`` registration of the compression ops over the C ABI.
+
+Schemas mirror the Python signatures of the reference's wrappers
+(src/zeroband/C/compression.py:11,22,34) plus the ops the ring needs
+(src/zeroband/C/csrc/collectives.cpp:8-22,124-138):
+
+    prime::uniform_8bit_quantize(Tensor tensor, bool inplace=True) -> (Tensor, Tensor)
+    prime::average_buckets(Tensor tensor, Tensor quant_weight, int n_bins) -> Tensor
+    prime::quantize_per_tensor_uint8(Tensor tensor, float scale, int zero_point) -> Tensor
+    prime::dequantize(Tensor codes, Tensor lut) -> Tensor
+    prime::dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()
+    prime::ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
+    prime::uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)
+    prime::uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)
+
+Kernels exist for ROCm tensors only.  A CPU tensor reaches no kernel and the dispatcher
+raises: there is deliberately no CPU path here.
+
+torch is used for device memory (outputs come from its caching allocator) and for the
+current stream; all arithmetic happens in libprime_hip.so.
+"""
+from __future__ import annotations
+
+from typing import Dict, Tuple
+
+import torch
+
+from . import _lib
+
+N_BINS = 256      # src/zeroband/C/csrc/compression.cpp:5
+ZERO_POINT = 128  # compression.cpp:107
+
+_LIB = torch.library.Library("prime", "DEF")
+_LIB.define("uniform_8bit_quantize(Tensor tensor, bool inplace=True) -> (Tensor, Tensor)")
+_LIB.define("average_buckets(Tensor tensor, Tensor quant_weight, int n_bins) -> Tensor")
+_LIB.define("quantize_per_tensor_uint8(Tensor tensor, float scale, int zero_point) -> Tensor")
+_LIB.define("dequantize(Tensor codes, Tensor lut) -> Tensor")
+_LIB.define("dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()")
+_LIB.define("ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
+_LIB.define("uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)")
+_LIB.define("uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)")
+
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def workspace(device: torch.device) -> torch.Tensor:
+    """The per-(device, stream) scratch block the multi-workgroup kernels share.  Work on one
+    stream is ordered, so one block per stream is enough."""
+    lib = _lib.load()
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    key = (idx, _stream(device))
+    ws = _workspaces.get(key)
+    if ws is None:
+        nbytes = int(lib.prime_workspace_bytes())
+        with torch.cuda.device(idx):
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=torch.device("cuda", idx))
+            _lib.check(lib.prime_workspace_init(ws.data_ptr(), nbytes, key[1]), "prime_workspace_init")
+        _workspaces[key] = ws
+    return ws
+
+
+def _need_f32(t: torch.Tensor, name: str) -> None:
+    # the reference reads data_ptr<float>(): any other dtype is a c10::Error -> RuntimeError
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"{name}: expected scalar type Float but found {t.dtype}")
+
+
+def _need_u8(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.uint8:
+        raise RuntimeError(f"{name}: expected scalar type Byte but found {t.dtype}")
+
+
+def _need_lut(lut: torch.Tensor, name: str) -> torch.Tensor:
+    _need_f32(lut, name)
+    if lut.numel() < N_BINS:
+        raise RuntimeError(f"{name}: lookup table needs {N_BINS} entries, got {lut.numel()}")
+    return lut.contiguous()
+
+
+def _uniform_8bit_quantize(tensor: torch.Tensor, inplace: bool = True):
+    codes, lut, _ = _uniform_8bit_quantize_stats(tensor)
+    return codes, lut
+
+
+def _uniform_8bit_quantize_stats(tensor: torch.Tensor):
+    """(codes, lut, qparams): qparams is the 32-byte ``prime_qparams`` record as 4 float64
+    words; view it with ``unpack_qparams``."""
+    _need_f32(tensor, "uniform_8bit_quantize")
+    lib = _lib.load()
+    x = tensor.contiguous()
+    dev = x.device
+    with torch.cuda.device(dev):
+        codes = torch.empty(x.shape, dtype=torch.uint8, device=dev)
+        lut = torch.empty(N_BINS, dtype=torch.float32, device=dev)
+        qp = torch.empty(4, dtype=torch.float64, device=dev)
+        ws = workspace(dev)
+        _lib.check(
+            lib.prime_uniform_8bit_quantize(x.data_ptr(), x.numel(), codes.data_ptr(), lut.data_ptr(), qp.data_ptr(),
+                                            ws.data_ptr(), _stream(dev)),
+            "prime_uniform_8bit_quantize")
+    return codes, lut, qp
+
+
+def _average_buckets(tensor: torch.Tensor, quant_weight: torch.Tensor, n_bins: int) -> torch.Tensor:
+    _need_f32(tensor, "average_buckets")
+    _need_u8(quant_weight, "average_buckets")
+    if tensor.numel() != quant_weight.numel():
+        raise RuntimeError("average_buckets: tensor and quant_weight differ in numel")
+    lib = _lib.load()
+    x = tensor.contiguous()
+    q = quant_weight.contiguous()
+    dev = x.device
+    with torch.cuda.device(dev):
+        lut = torch.empty(int(n_bins), dtype=torch.float32, device=dev)
+        ws = workspace(dev)
+        _lib.check(
+            lib.prime_average_buckets(x.data_ptr(), q.data_ptr(), x.numel(), int(n_bins), lut.data_ptr(), None,
+                                      ws.data_ptr(), _stream(dev)),
+            "prime_average_buckets")
+    return lut
+
+
+def _quantize_per_tensor_uint8(tensor: torch.Tensor, scale: float, zero_point: int) -> torch.Tensor:
+    _need_f32(tensor, "quantize_per_tensor_uint8")
+    lib = _lib.load()
+    x = tensor.contiguous()
+    dev = x.device
+    with torch.cuda.device(dev):
+        codes = torch.empty(x.shape, dtype=torch.uint8, device=dev)
+        _lib.check(
+            lib.prime_quantize_u8(x.data_ptr(), x.numel(), float(scale), int(zero_point), codes.data_ptr(), _stream(dev)),
+            "prime_quantize_u8")
+    return codes
+
+
+def _dequantize(codes: torch.Tensor, lut: torch.Tensor) -> torch.Tensor:
+    _need_u8(codes, "dequantize")
+    out = torch.empty(codes.shape, dtype=torch.float32, device=codes.device)
+    _dequantize_(out, codes, lut, False)
+    return out
+
+
+def _dequantize_(out: torch.Tensor, codes: torch.Tensor, lut: torch.Tensor, accumulate: bool) -> None:
+    _need_f32(out, "dequantize_")
+    _need_u8(codes, "dequantize_")
+    lut = _need_lut(lut, "dequantize_")
+    if not out.is_contiguous():
+        raise RuntimeError("dequantize_: out must be contiguous (it is written in place)")
+    if out.numel() != codes.numel():
+        raise RuntimeError("dequantize_: out and codes differ in numel")
+    lib = _lib.load()
+    c = codes.contiguous()
+    dev = out.device
+    with torch.cuda.device(dev):
+        fn = lib.prime_dequant_add if accumulate else lib.prime_dequant_set
+        _lib.check(fn(out.data_ptr(), lut.data_ptr(), c.data_ptr(), out.numel(), _stream(dev)), "prime_dequant")
+
+
+def _ring_reduce_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor):
+    _need_f32(acc, "ring_reduce_step")
+    _need_u8(codes_in, "ring_reduce_step")
+    lut_in = _need_lut(lut_in, "ring_reduce_step")
+    if not acc.is_contiguous():
+        raise RuntimeError("ring_reduce_step: acc must be contiguous (it is updated in place)")
+    if acc.numel() != codes_in.numel():
+        raise RuntimeError("ring_reduce_step: acc and codes_in differ in numel")
+    lib = _lib.load()
+    c = codes_in.contiguous()
+    dev = acc.device
+    with torch.cuda.device(dev):
+        codes = torch.empty(acc.shape, dtype=torch.uint8, device=dev)
+        lut = torch.empty(N_BINS, dtype=torch.float32, device=dev)
+        ws = workspace(dev)
+        _lib.check(
+            lib.prime_ring_reduce_step(acc.data_ptr(), c.data_ptr(), lut_in.data_ptr(), acc.numel(), codes.data_ptr(),
+                                       lut.data_ptr(), None, ws.data_ptr(), _stream(dev)),
+            "prime_ring_reduce_step")
+    return codes, lut
+
+
+def _uniform_8bit_quantize_batched(flat: torch.Tensor, offsets: torch.Tensor):
+    """Every slice flat[offsets[t]:offsets[t+1]] quantized on its own, one launch.
+    Returns (codes like flat, luts [count, 256], qparams [count, 4] float64 words)."""
+    _need_f32(flat, "uniform_8bit_quantize_batched")
+    if offsets.dtype != torch.int64 or offsets.dim() != 1 or offsets.numel() < 1:
+        raise RuntimeError("uniform_8bit_quantize_batched: offsets must be a 1-D int64 tensor of count+1 entries")
+    if not flat.is_contiguous():
+        raise RuntimeError("uniform_8bit_quantize_batched: flat must be contiguous")
+    lib = _lib.load()
+    dev = flat.device
+    count = offsets.numel() - 1
+    off = offsets.to(dev).contiguous()
+    with torch.cuda.device(dev):
+        codes = torch.empty(flat.shape, dtype=torch.uint8, device=dev)
+        luts = torch.empty((count, N_BINS), dtype=torch.float32, device=dev)
+        qps = torch.empty((count, 4), dtype=torch.float64, device=dev)
+        _lib.check(
+            lib.prime_uniform_8bit_quantize_batched(flat.data_ptr(), off.data_ptr(), count, codes.data_ptr(),
+                                                    luts.data_ptr(), qps.data_ptr(), _stream(dev)),
+            "prime_uniform_8bit_quantize_batched")
+    return codes, luts, qps
+
+
+_LIB.impl("uniform_8bit_quantize", _uniform_8bit_quantize, "CUDA")
+_LIB.impl("average_buckets", _average_buckets, "CUDA")
+_LIB.impl("quantize_per_tensor_uint8", _quantize_per_tensor_uint8, "CUDA")
+_LIB.impl("dequantize", _dequantize, "CUDA")
+_LIB.impl("dequantize_", _dequantize_, "CUDA")
+_LIB.impl("ring_reduce_step", _ring_reduce_step, "CUDA")
+_LIB.impl("uniform_8bit_quantize_stats", _uniform_8bit_quantize_stats, "CUDA")
+_LIB.impl("uniform_8bit_quantize_batched", _uniform_8bit_quantize_batched, "CUDA")
+
+
+# shape-only implementations so the ops can be traced
+@torch.library.register_fake("prime::uniform_8bit_quantize")
+def _(tensor, inplace=True):
+    return tensor.new_empty(tensor.shape, dtype=torch.uint8), tensor.new_empty(N_BINS, dtype=torch.float32)
+
+
+@torch.library.register_fake("prime::average_buckets")
+def _(tensor, quant_weight, n_bins):
+    return tensor.new_empty(n_bins, dtype=torch.float32)
+
+
+@torch.library.register_fake("prime::quantize_per_tensor_uint8")
+def _(tensor, scale, zero_point):
+    return tensor.new_empty(tensor.shape, dtype=torch.uint8)
+
+
+@torch.library.register_fake("prime::dequantize")
+def _(codes, lut):
+    return codes.new_empty(codes.shape, dtype=torch.float32)
+
+
+@torch.library.register_fake("prime::ring_reduce_step")
+def _(acc, codes_in, lut_in):
+    return acc.new_empty(acc.shape, dtype=torch.uint8), acc.new_empty(N_BINS, dtype=torch.float32)
+
+
+def unpack_qparams(qp: torch.Tensor) -> dict:
+    """Host view of one ``prime_qparams`` record (synchronises)."""
+    raw = qp.detach().cpu().contiguous().view(torch.uint8).numpy().tobytes()
+    rec = _lib.QParams.from_buffer_copy(raw[: _lib.QPARAMS_BYTES])
+    return {"scale": rec.scale, "inv_scale": rec.inv_scale, "sum": rec.sum, "sumsq": rec.sumsq, "n": rec.n}
+
+
+uniform_8bit_quantize = torch.ops.prime.uniform_8bit_quantize
+average_buckets = torch.ops.prime.average_buckets
+quantize_per_tensor_uint8 = torch.ops.prime.quantize_per_tensor_uint8
+dequantize = torch.ops.prime.dequantize
+dequantize_ = torch.ops.prime.dequantize_
+ring_reduce_step = torch.ops.prime.ring_reduce_step
+uniform_8bit_quantize_stats = torch.ops.prime.uniform_8bit_quantize_stats
+uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched

@@ -1,0 +1,103 @@
+"""The ring all-reduce's compute, run on one GPU for W simulated ranks.
+
+The reference's ``ring_allreduce`` (src/zeroband/C/csrc/collectives.cpp:76-230; readable twin
+src/zeroband/collectives.py:53-192) splits each rank's tensor into 2 W chunks and passes
+uint8 codes plus a 256-entry lookup round the ring.  What a rank computes per received
+message is fixed by the schedule and independent of the transport:
+
+  reduce-scatter   chunk += lut[codes]; (codes, lut) = uniform_8bit_quantize(chunk)   :124-138
+  own chunks       [chunk /= W]; chunk = lut[codes] of its own quantization          :155-173
+  all-gather       chunk = lut[codes]; re-quantize before forwarding                 :194-215
+
+Here every "rank" is a tensor on the same device and a send is a hand-over of the
+(codes, lut) pair; the kernels are the ones a real ring over RCCL or TCP would run.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence, Tuple
+
+import torch
+
+from . import ops
+
+BUFFER_COUNT = 2   # collectives.cpp:6
+
+
+def ring_hops(chunks: Sequence[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One chunk's trip through the reduce-scatter phase: ``chunks[r]`` is what the r-th rank
+    on the path holds.  chunks[0] is quantized; each later rank accumulates the received
+    codes into its chunk (in place) and requantizes.  Returns the last (codes, lut)."""
+    codes, lut = ops.uniform_8bit_quantize(chunks[0], False)
+    for acc in chunks[1:]:
+        codes, lut = ops.ring_reduce_step(acc, codes, lut)
+    return codes, lut
+
+
+def _check_ring_inputs(tensors: Sequence[torch.Tensor]) -> int:
+    if len(tensors) == 0:
+        raise ValueError("at least one rank is needed")
+    n = tensors[0].numel()
+    for t in tensors:
+        if t.dtype != torch.float32:
+            raise RuntimeError(f"expected scalar type Float but found {t.dtype}")
+        if t.numel() != n or t.device != tensors[0].device:
+            raise ValueError("all simulated ranks must hold tensors of one size on one device")
+        if not t.is_contiguous():
+            raise RuntimeError("ring all-reduce works in place and needs contiguous tensors")
+    if n % (BUFFER_COUNT * len(tensors)) != 0:
+        # the Python twin asserts this (src/zeroband/collectives.py:83)
+        raise ValueError("Tensor size must be divisible by world size")
+    return n
+
+
+def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False) -> None:
+    """The whole of ``ring_allreduce`` for ``len(tensors)`` ranks, in place, in lock step.
+
+    A message posted at step s is consumed at step s + 2 (BUFFER_COUNT receive slots,
+    collectives.cpp:118-122), which lock-stepping the ranks reproduces exactly."""
+    W = len(tensors)
+    n = _check_ring_inputs(tensors)
+    nb = BUFFER_COUNT * W
+    csz = n // nb
+    flats = [t.view(-1) for t in tensors]
+
+    def chunk(r: int, c: int) -> torch.Tensor:
+        return flats[r][c * csz:(c + 1) * csz]
+
+    for phase in (1, 2):
+        inbox: List[dict] = [dict() for _ in range(W)]
+        for step in range(1, nb + 1):
+            posted = []
+            for r in range(W):
+                if phase == 1:
+                    c = (r * BUFFER_COUNT - step) % nb                      # collectives.cpp:116
+                else:
+                    c = (r * BUFFER_COUNT + BUFFER_COUNT - step) % nb       # :192
+                ch = chunk(r, c)
+                msg = inbox[r].pop(step - BUFFER_COUNT, None)
+                sending = step <= (W - 1) * BUFFER_COUNT                    # :136 / :212
+                if msg is not None and phase == 1 and sending:
+                    codes, lut = ops.ring_reduce_step(ch, msg[0], msg[1])   # :128-138 fused
+                    posted.append(((r + 1) % W, step, codes, lut))
+                    continue
+                if msg is not None:
+                    ops.dequantize_(ch, msg[0], msg[1], phase == 1)         # :128-133 / :204-209
+                if sending:
+                    codes, lut = ops.uniform_8bit_quantize(ch, False)       # :138 / :215
+                    posted.append(((r + 1) % W, step, codes, lut))
+            for dst, st, codes, lut in posted:
+                inbox[dst][st] = (codes, lut)
+        if phase == 1:
+            for r in range(W):
+                for i in range(BUFFER_COUNT):
+                    ch = chunk(r, i + r * BUFFER_COUNT)
+                    if avg:
+                        ch.div_(W)                                          # :155-159
+                    codes, lut = ops.uniform_8bit_quantize(ch, True)        # :162
+                    ops.dequantize_(ch, codes, lut, False)                  # :167-172
+
+
+def ring_allreduce_single(tensor: torch.Tensor, avg: bool = False) -> None:
+    """``ring_allreduce`` on a group of one rank: no message is sent, but both of the rank's
+    chunks still take the lossy quantize / dequantize round trip (collectives.cpp:161-173)."""
+    ring_allreduce_simulated([tensor.view(-1)], avg=avg)
