@@ -17,13 +17,13 @@
 //                               fp64 closed form; compiled reference
 //   oracle_uniform_8bit_quantize closed forms (constant tensor -> code 171, zero tensor, n = 1),
 //                               golden fixtures written by the compiled reference
-//   oracle_norm_literal         bit-for-bit against libtorch's at::norm (observed accumulation
-//                               order: 8 fp32 lanes, fused multiply-add, lanes summed 0..7, sqrtf);
+//   oracle_norm_literal         bit-for-bit against libtorch's at::norm over sizes 1..70 and larger
+//                               (observed order: 8 fp32 FMA lanes, lanes summed 0..7, tail, sqrtf);
 //                               the order used by the reference's pinned torch 2.5.1 cannot be
 //                               checked offline: "parity unpinned" for that version only
 //   oracle_index_add / _set     numpy lut[codes] bitwise
 //
-// Build: see oracle/Makefile (g++ -O3, the reference's only flag, src/zeroband/C/compression.py:8).
+// Build: see oracle/build.py (g++ -O3, the reference's only flag, src/zeroband/C/compression.py:8).
 
 #include <algorithm>
 #include <cmath>
@@ -140,9 +140,11 @@ void oracle_average_buckets_f64(const float* x, const uint8_t* codes, int64_t n,
 }
 
 // The value `tensor.norm()` (compression.cpp:113) returns for a contiguous fp32 CPU tensor
-// in libtorch 2.10: eight fp32 lanes, lane j accumulating elements j, j+8, ... with a fused
-// multiply-add, lanes then added 0..7, the n % 8 tail added with separate multiply and add,
-// and a float square root.
+// in libtorch 2.10 on x86-64, found by matching it bit for bit: eight fp32 lanes, lane j
+// accumulating elements j, j+8, ... with a fused multiply-add; lanes added 0..7; then the
+// n % 8 tail in order, a group of four as rounded products added one by one (the compiler's
+// in-order vectorisation of the scalar tail loop) and the last n % 4 elements by fused
+// multiply-add; and a float square root.
 float oracle_norm_literal(const float* x, int64_t n) {
     float lane[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     const int64_t m = n - (n % 8);
@@ -150,10 +152,15 @@ float oracle_norm_literal(const float* x, int64_t n) {
         for (int j = 0; j < 8; ++j) lane[j] = std::fma(x[i + j], x[i + j], lane[j]);
     float s = lane[0];
     for (int j = 1; j < 8; ++j) s += lane[j];
-    for (int64_t i = m; i < n; ++i) {
-        volatile float sq = x[i] * x[i];   // keep the product rounded: no contraction here
-        s += sq;
+    int64_t i = m;
+    if (n - i >= 4) {
+        for (int k = 0; k < 4; ++k) {
+            volatile float sq = x[i + k] * x[i + k];   // product rounded on its own: no contraction
+            s += sq;
+        }
+        i += 4;
     }
+    for (; i < n; ++i) s = std::fma(x[i], x[i], s);
     return std::sqrt(s);
 }
 

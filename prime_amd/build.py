@@ -27,12 +27,16 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose: bool = True) -> Path:
-    cmd = ["hipcc", *HIPCC_FLAGS, *map(str, SOURCES), "-o", str(LIB_PATH)]
+def build(verbose: bool = True, defines: dict | None = None, out: Path | None = None) -> Path:
+    """Compile the library.  ``defines`` overrides the PRIME_* tuning macros of the source and
+    ``out`` redirects the output (for tuning sweeps that keep several variants side by side)."""
+    out = Path(out) if out else LIB_PATH
+    extra = [f"-D{k}={v}" for k, v in (defines or {}).items()]
+    cmd = ["hipcc", *HIPCC_FLAGS, *extra, *map(str, SOURCES), "-o", str(out)]
     if verbose:
         print("+", " ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    return LIB_PATH
+    return out
 
 
 if __name__ == "__main__":

@@ -2,7 +2,8 @@
 // compression path: fp64 statistics, uint8 quantization, 256-bin lookup build, lookup
 // dequantization and the ring's accumulate + requantize step.  All kernels are HBM-bound
 // streams: 16-byte loads per lane, 256-thread workgroups that loop over tiles, histogram
-// traffic kept in LDS and merged once per workgroup.
+// traffic kept in LDS.  Grid-level reductions are two-stage: every workgroup stores its
+// partial result, a small second kernel adds the partials in a fixed order.
 //
 // Arithmetic follows the reference's CPU ops (paths relative to the reference checkout):
 //   src/zeroband/C/csrc/compression.cpp:9-43    quantize      -> quantize_code()
@@ -20,31 +21,102 @@
 
 namespace {
 
+// Build-time tuning.
+#ifndef PRIME_UNROLL
+#define PRIME_UNROLL 4                   // 16-byte loads in flight per lane
+#endif
+#ifndef PRIME_NT_LOAD
+#define PRIME_NT_LOAD 0                  // non-temporal hint on streamed loads
+#endif
+#ifndef PRIME_NT_STORE
+#define PRIME_NT_STORE 0                 // non-temporal hint on streamed stores
+#endif
+
 constexpr int kThreads = 256;            // 4 wavefronts of 64
 constexpr int kWaves = kThreads / 64;
 constexpr int kBins = 256;               // compression.cpp:5
 constexpr int kZeroPoint = 128;          // compression.cpp:107
-constexpr int kMaxGrid = 4096;           // partial-sum slots in the workspace
-constexpr int kUnroll = 4;               // 16-byte loads in flight per lane
+constexpr int kMaxGrid = 2048;           // per-workgroup partial slots in the workspace
+constexpr int kUnroll = PRIME_UNROLL;
+constexpr int kFinalThreads = 1024;      // workgroup size of the second-stage kernels
+constexpr int kLutBinsPerBlock = 4;      // bins one second-stage workgroup reduces (64 bytes per partial)
+constexpr int64_t kMaxElems = int64_t(1) << 40;   // per-workgroup counts are 32-bit
 
-struct Workspace {
-    uint32_t ticket;                     // grid-level "last workgroup" counter, 0 between calls
-    uint32_t pad[3];
-    prime_qparams qp;                    // scale of the tensor in flight
-    double hist_sum[kBins];              // 0 between calls
-    unsigned long long hist_cnt[kBins];  // 0 between calls
-    double part_sum[kMaxGrid];
-    double part_sq[kMaxGrid];
+struct BinAcc {
+    double sum;
+    unsigned long long cnt;
 };
 
-typedef float f4a __attribute__((ext_vector_type(4)));                 // 16-byte aligned
-typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));     // element aligned only
-typedef uint32_t u32a;
-typedef uint32_t u32u __attribute__((aligned(1)));
+// Every kernel stores its per-workgroup partial results here with plain stores; the kernel
+// boundary makes them visible to the second stage.  Nothing has to be zero between calls.
+struct Workspace {
+    prime_qparams qp;                    // scale of the tensor in flight
+    double part_sum[kMaxGrid];
+    double part_sq[kMaxGrid];
+    BinAcc hist[kMaxGrid][kBins];        // 4 KiB per workgroup
+};
 
-template <bool ALIGNED> struct Vec;
-template <> struct Vec<true> { using f4 = f4a; using u32 = u32a; };
-template <> struct Vec<false> { using f4 = f4u; using u32 = u32u; };
+typedef float f4a __attribute__((ext_vector_type(4)));   // 16-byte aligned
+
+// Under-aligned views for buffers that are only element aligned (a chunk or a view that
+// starts at an odd element).  They are distinct struct types, so the alignment survives
+// template deduction; the compiler picks accesses that are legal for that alignment.
+struct __attribute__((packed, aligned(4))) F4U { float x, y, z, w; };
+struct __attribute__((packed)) U32U { uint32_t v; };
+
+// Streamed accesses, 4 floats / 4 codes at vector index i.  ALIGNED means the float buffer is
+// 16-byte aligned and the code buffer 4-byte aligned.
+template <bool ALIGNED> struct Mem;
+
+template <> struct Mem<true> {
+    static __device__ __forceinline__ f4a ldf4(const float* p, int64_t i) {
+        const f4a* q = reinterpret_cast<const f4a*>(p) + i;
+#if PRIME_NT_LOAD
+        return __builtin_nontemporal_load(q);
+#else
+        return *q;
+#endif
+    }
+    static __device__ __forceinline__ void stf4(float* p, int64_t i, f4a v, bool streaming) {
+        f4a* q = reinterpret_cast<f4a*>(p) + i;
+#if PRIME_NT_STORE
+        if (streaming) { __builtin_nontemporal_store(v, q); return; }
+#endif
+        *q = v;
+    }
+    static __device__ __forceinline__ uint32_t ldu32(const uint8_t* p, int64_t i) {
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(p) + i;
+#if PRIME_NT_LOAD
+        return __builtin_nontemporal_load(q);
+#else
+        return *q;
+#endif
+    }
+    static __device__ __forceinline__ void stu32(uint8_t* p, int64_t i, uint32_t v) {
+        uint32_t* q = reinterpret_cast<uint32_t*>(p) + i;
+#if PRIME_NT_STORE
+        __builtin_nontemporal_store(v, q);
+#else
+        *q = v;
+#endif
+    }
+};
+
+template <> struct Mem<false> {
+    static __device__ __forceinline__ f4a ldf4(const float* p, int64_t i) {
+        const F4U t = reinterpret_cast<const F4U*>(p)[i];
+        return f4a{t.x, t.y, t.z, t.w};
+    }
+    static __device__ __forceinline__ void stf4(float* p, int64_t i, f4a v, bool) {
+        reinterpret_cast<F4U*>(p)[i] = F4U{v.x, v.y, v.z, v.w};
+    }
+    static __device__ __forceinline__ uint32_t ldu32(const uint8_t* p, int64_t i) {
+        return reinterpret_cast<const U32U*>(p)[i].v;
+    }
+    static __device__ __forceinline__ void stu32(uint8_t* p, int64_t i, uint32_t v) {
+        reinterpret_cast<U32U*>(p)[i] = U32U{v};
+    }
+};
 
 __device__ __forceinline__ double wave_sum(double v) {
 #pragma unroll
@@ -77,14 +149,11 @@ __device__ __forceinline__ void finalize_qparams(double sum, double sumsq, int64
     qp->n = n;
 }
 
-// Workgroup reduction of (sum, sumsq), one partial per workgroup, and a second stage run by
-// whichever workgroup takes the last ticket.  The second stage adds the partials in a fixed
-// order, so the scale does not depend on scheduling.
-__device__ __forceinline__ void block_stats_finish(double s, double q, int64_t n, Workspace* ws,
-                                                   prime_qparams* out) {
+// Workgroup reduction of (sum, sumsq) in a fixed order; the workgroup's partial goes to the
+// workspace for stats_finalize_kernel.
+__device__ __forceinline__ void block_stats_store(double s, double q, Workspace* ws) {
     __shared__ double sh_s[kWaves];
     __shared__ double sh_q[kWaves];
-    __shared__ int sh_last;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     s = wave_sum(s);
     q = wave_sum(q);
@@ -96,30 +165,33 @@ __device__ __forceinline__ void block_stats_finish(double s, double q, int64_t n
         for (int w = 1; w < kWaves; ++w) { S += sh_s[w]; Q += sh_q[w]; }
         ws->part_sum[blockIdx.x] = S;
         ws->part_sq[blockIdx.x] = Q;
-        __threadfence();
-        const unsigned t = __hip_atomic_fetch_add(&ws->ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        sh_last = (t == gridDim.x - 1);
     }
-    __syncthreads();
-    if (!sh_last) return;
-    __threadfence();
+}
+
+// Second stage of the statistics: one workgroup adds the partials (tree of fixed shape) and
+// derives the scale.
+__global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace* ws, int nparts, int64_t n,
+                                                                        prime_qparams* out) {
+    __shared__ double sh_s[kFinalThreads / 64];
+    __shared__ double sh_q[kFinalThreads / 64];
     double a = 0.0, b = 0.0;
-    for (int i = threadIdx.x; i < static_cast<int>(gridDim.x); i += kThreads) {
+    for (int i = threadIdx.x; i < nparts; i += kFinalThreads) {
         a += ws->part_sum[i];
         b += ws->part_sq[i];
     }
     a = wave_sum(a);
     b = wave_sum(b);
-    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (lane == 0) { sh_s[wave] = a; sh_q[wave] = b; }
     __syncthreads();
     if (threadIdx.x == 0) {
         double S = sh_s[0], Q = sh_q[0];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) { S += sh_s[w]; Q += sh_q[w]; }
-        finalize_qparams(S, Q, n, &ws->qp);
-        if (out) *out = ws->qp;
-        ws->ticket = 0;
+        for (int w = 1; w < kFinalThreads / 64; ++w) { S += sh_s[w]; Q += sh_q[w]; }
+        prime_qparams qp;
+        finalize_qparams(S, Q, n, &qp);
+        ws->qp = qp;
+        if (out) *out = qp;
     }
 }
 
@@ -133,10 +205,8 @@ __device__ __forceinline__ void stats_add4(const f4a v, double& s, double& q) {
 
 // K1: sum and sum of squares in fp64.  4 bytes per element.
 template <bool ALIGNED>
-__global__ __launch_bounds__(kThreads) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws,
-                                                         prime_qparams* out) {
-    using f4 = typename Vec<ALIGNED>::f4;
-    const f4* __restrict__ x4 = reinterpret_cast<const f4*>(x);
+__global__ __launch_bounds__(kThreads) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
+    using M = Mem<ALIGNED>;
     const int64_t nvec = n >> 2;
     const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
@@ -145,30 +215,31 @@ __global__ __launch_bounds__(kThreads) void stats_kernel(const float* __restrict
         const int64_t i0 = base + threadIdx.x;
         if (base + tile <= nvec) {
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) v[j] = x4[i0 + j * kThreads];
+            for (int j = 0; j < kUnroll; ++j) v[j] = M::ldf4(x, i0 + j * kThreads);
         } else {
 #pragma unroll
             for (int j = 0; j < kUnroll; ++j) {
                 const int64_t i = i0 + j * kThreads;
-                v[j] = i < nvec ? static_cast<f4a>(x4[i]) : f4a{0.f, 0.f, 0.f, 0.f};
+                v[j] = i < nvec ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
             }
         }
-        stats_add4(v[0], s0, q0);
-        stats_add4(v[1], s1, q1);
-        stats_add4(v[2], s0, q0);
-        stats_add4(v[3], s1, q1);
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            if (j & 1) stats_add4(v[j], s1, q1); else stats_add4(v[j], s0, q0);
+        }
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const double v = x[(nvec << 2) + threadIdx.x];
         s0 += v;
         q0 = fma(v, v, q0);
     }
-    block_stats_finish(s0 + s1, q0 + q1, n, ws, out);
+    block_stats_store(s0 + s1, q0 + q1, ws);
 }
 
 // LDS histogram: R copies of each bin, chosen by lane, so that lanes of one wavefront that
 // hit the same bin mostly hit different addresses (and banks).  Sums are fp64, counts u32
-// (a workgroup never sees 2^32 elements: the grid is sized so that it cannot).
+// (a workgroup never sees 2^32 elements: n is capped at 2^40 and the grid is at least one
+// workgroup per compute unit once n is that large).
 template <int R>
 struct LdsHist {
     double sum[kBins * R];
@@ -187,19 +258,15 @@ __device__ __forceinline__ void hist_add(LdsHist<R>& h, int code, float x) {
     __hip_atomic_fetch_add(&h.cnt[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-// Merge a workgroup's histogram into the workspace accumulators (one fp64 and one u64
-// hardware atomic per non-empty bin).
+// Store the workgroup's histogram (copies added in a fixed order) as its partial: one
+// 16-byte store per lane, 4 KiB contiguous per workgroup.
 template <int R>
-__device__ __forceinline__ void hist_flush(LdsHist<R>& h, Workspace* ws) {
+__device__ __forceinline__ void hist_store(LdsHist<R>& h, Workspace* ws) {
     const int b = threadIdx.x;   // kThreads == kBins
-    double s = 0.0;
-    unsigned long long c = 0;
+    BinAcc acc{0.0, 0ull};
 #pragma unroll
-    for (int r = 0; r < R; ++r) { s += h.sum[b * R + r]; c += h.cnt[b * R + r]; }
-    if (c) {
-        unsafeAtomicAdd(&ws->hist_sum[b], s);
-        __hip_atomic_fetch_add(&ws->hist_cnt[b], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    for (int r = 0; r < R; ++r) { acc.sum += h.sum[b * R + r]; acc.cnt += h.cnt[b * R + r]; }
+    ws->hist[blockIdx.x][b] = acc;
 }
 
 // K2 (+K3 when HIST): quantize to uint8, 4 codes packed per 32-bit store, and the 256-bin
@@ -208,16 +275,13 @@ template <bool ALIGNED, bool HIST, int R>
 __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
                                                             const prime_qparams* __restrict__ qp, int zero_point,
                                                             uint8_t* __restrict__ codes, Workspace* ws, int reverse) {
-    using f4 = typename Vec<ALIGNED>::f4;
-    using u32 = typename Vec<ALIGNED>::u32;
+    using M = Mem<ALIGNED>;
     __shared__ LdsHist<HIST ? R : 1> hist;
     if (HIST) {
         hist_zero(hist);
         __syncthreads();
     }
     const float inv = qp ? qp->inv_scale : 1.0f / scale_val;
-    const f4* __restrict__ x4 = reinterpret_cast<const f4*>(x);
-    u32* __restrict__ c4 = reinterpret_cast<u32*>(codes);
     const int64_t nvec = n >> 2;
     const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
     const int64_t ntiles = (nvec + tile - 1) / tile;
@@ -228,12 +292,12 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
         const bool full = base + tile <= nvec;
         if (full) {
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) v[j] = x4[i0 + j * kThreads];
+            for (int j = 0; j < kUnroll; ++j) v[j] = M::ldf4(x, i0 + j * kThreads);
         } else {
 #pragma unroll
             for (int j = 0; j < kUnroll; ++j) {
                 const int64_t i = i0 + j * kThreads;
-                v[j] = i < nvec ? static_cast<f4a>(x4[i]) : f4a{0.f, 0.f, 0.f, 0.f};
+                v[j] = i < nvec ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
             }
         }
 #pragma unroll
@@ -244,8 +308,8 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
                 const int b = quantize_code(v[j].y, inv, zero_point);
                 const int c = quantize_code(v[j].z, inv, zero_point);
                 const int d = quantize_code(v[j].w, inv, zero_point);
-                c4[i] = static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) |
-                        (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24);
+                M::stu32(codes, i, static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) |
+                                       (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24));
                 if (HIST) {
                     hist_add(hist, a, v[j].x);
                     hist_add(hist, b, v[j].y);
@@ -264,7 +328,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
     }
     if (HIST) {
         __syncthreads();
-        hist_flush(hist, ws);
+        hist_store(hist, ws);
     }
 }
 
@@ -272,23 +336,33 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
 template <bool ALIGNED, int R>
 __global__ __launch_bounds__(kThreads) void hist_kernel(const float* __restrict__ x, const uint8_t* __restrict__ codes,
                                                         int64_t n, int n_bins, Workspace* ws) {
-    using f4 = typename Vec<ALIGNED>::f4;
-    using u32 = typename Vec<ALIGNED>::u32;
+    using M = Mem<ALIGNED>;
     __shared__ LdsHist<R> hist;
     hist_zero(hist);
     __syncthreads();
-    const f4* __restrict__ x4 = reinterpret_cast<const f4*>(x);
-    const u32* __restrict__ c4 = reinterpret_cast<const u32*>(codes);
     const int64_t nvec = n >> 2;
-    for (int64_t i = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x; i < nvec;
-         i += static_cast<int64_t>(gridDim.x) * kThreads) {
-        const f4a v = x4[i];
-        const uint32_t c = c4[i];
-        const int a = c & 255, b = (c >> 8) & 255, cc = (c >> 16) & 255, d = c >> 24;
-        if (a < n_bins) hist_add(hist, a, v.x);     // compression.cpp:70
-        if (b < n_bins) hist_add(hist, b, v.y);
-        if (cc < n_bins) hist_add(hist, cc, v.z);
-        if (d < n_bins) hist_add(hist, d, v.w);
+    const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
+    for (int64_t base = blockIdx.x * tile; base < nvec; base += static_cast<int64_t>(gridDim.x) * tile) {
+        f4a v[kUnroll];
+        uint32_t c[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = base + threadIdx.x + j * kThreads;
+            const bool ok = i < nvec;
+            v[j] = ok ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            c[j] = ok ? M::ldu32(codes, i) : 0xffffffffu;
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = base + threadIdx.x + j * kThreads;
+            if (i < nvec) {
+                const int a = c[j] & 255, b = (c[j] >> 8) & 255, cc = (c[j] >> 16) & 255, d = c[j] >> 24;
+                if (a < n_bins) hist_add(hist, a, v[j].x);     // compression.cpp:70
+                if (b < n_bins) hist_add(hist, b, v[j].y);
+                if (cc < n_bins) hist_add(hist, cc, v[j].z);
+                if (d < n_bins) hist_add(hist, d, v[j].w);
+            }
+        }
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
@@ -296,25 +370,54 @@ __global__ __launch_bounds__(kThreads) void hist_kernel(const float* __restrict_
         if (a < n_bins) hist_add(hist, a, x[i]);
     }
     __syncthreads();
-    hist_flush(hist, ws);
+    hist_store(hist, ws);
 }
 
-// Turn the workspace accumulators into the lookup table and clear them for the next call.
-// Mean = fp64 sum / count, rounded to float once; an empty bin gives 0.0f (compression.cpp:100).
-__global__ __launch_bounds__(kThreads) void lut_finalize_kernel(Workspace* ws, float* __restrict__ lut, int64_t n_bins,
-                                                                unsigned long long* __restrict__ counts) {
-    for (int64_t b = threadIdx.x; b < n_bins; b += kThreads) {
-        float m = 0.0f;
-        if (b < kBins) {
-            const double s = ws->hist_sum[b];
-            const unsigned long long c = ws->hist_cnt[b];
-            if (c) m = static_cast<float>(s / static_cast<double>(c));
-            if (counts) counts[b] = c;
-        }
-        lut[b] = m;
+// Second stage of the lookup build.  Workgroup j owns bins 4j .. 4j+3 (64 contiguous bytes
+// of every partial): lane (row, bin) adds partials row, row + 256, ... in order, the 256
+// rows are then added by a tree of fixed shape.  Mean = fp64 sum / count rounded to float
+// once; an empty bin gives 0.0f (compression.cpp:100).  Entries >= 256 of a longer table
+// are 0.0f.
+__global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Workspace* __restrict__ ws, int nparts,
+                                                                      float* __restrict__ lut, int64_t n_bins,
+                                                                      unsigned long long* __restrict__ counts) {
+    constexpr int kRows = kFinalThreads / kLutBinsPerBlock;
+    __shared__ double sh_sum[kFinalThreads];
+    __shared__ unsigned long long sh_cnt[kFinalThreads];
+    const int bl = threadIdx.x % kLutBinsPerBlock;
+    const int row = threadIdx.x / kLutBinsPerBlock;
+    const int bin = blockIdx.x * kLutBinsPerBlock + bl;
+    double s = 0.0;
+    unsigned long long c = 0;
+    for (int p = row; p < nparts; p += kRows) {
+        const BinAcc a = ws->hist[p][bin];
+        s += a.sum;
+        c += a.cnt;
     }
-    ws->hist_sum[threadIdx.x] = 0.0;
-    ws->hist_cnt[threadIdx.x] = 0ull;
+    sh_sum[threadIdx.x] = s;
+    sh_cnt[threadIdx.x] = c;
+    __syncthreads();
+    for (int half = kRows / 2; half > 0; half >>= 1) {
+        if (row < half) {
+            sh_sum[threadIdx.x] += sh_sum[threadIdx.x + half * kLutBinsPerBlock];
+            sh_cnt[threadIdx.x] += sh_cnt[threadIdx.x + half * kLutBinsPerBlock];
+        }
+        __syncthreads();
+    }
+    if (row == 0 && bin < n_bins) {
+        const unsigned long long cc = sh_cnt[threadIdx.x];
+        lut[bin] = cc ? static_cast<float>(sh_sum[threadIdx.x] / static_cast<double>(cc)) : 0.0f;
+        if (counts) counts[bin] = cc;
+    }
+    if (blockIdx.x == 0)
+        for (int64_t b = kBins + threadIdx.x; b < n_bins; b += kFinalThreads) lut[b] = 0.0f;
+}
+
+__global__ void lut_zero_kernel(float* __restrict__ lut, int64_t n_bins, unsigned long long* __restrict__ counts) {
+    for (int64_t b = threadIdx.x; b < n_bins; b += blockDim.x) {
+        lut[b] = 0.0f;
+        if (counts && b < kBins) counts[b] = 0ull;
+    }
 }
 
 // K5 / K4 pass A: out = lut[codes] (collectives.cpp:16-22) or out += lut[codes] (:8-14),
@@ -322,15 +425,11 @@ __global__ __launch_bounds__(kThreads) void lut_finalize_kernel(Workspace* ws, f
 // values are taken in the same pass (the next quantization's scale).
 template <bool ADD, bool STATS, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut,
-                                                           const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
-                                                           prime_qparams* qp_out) {
-    using f4 = typename Vec<ALIGNED>::f4;
-    using u32 = typename Vec<ALIGNED>::u32;
+                                                           const uint8_t* __restrict__ codes, int64_t n, Workspace* ws) {
+    using M = Mem<ALIGNED>;
     __shared__ float s_lut[kBins];
     s_lut[threadIdx.x] = lut[threadIdx.x];
     __syncthreads();
-    f4* __restrict__ o4 = reinterpret_cast<f4*>(out);
-    const u32* __restrict__ c4 = reinterpret_cast<const u32*>(codes);
     const int64_t nvec = n >> 2;
     const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
@@ -343,8 +442,8 @@ __global__ __launch_bounds__(kThreads) void dequant_kernel(float* __restrict__ o
         for (int j = 0; j < kUnroll; ++j) {
             const int64_t i = i0 + j * kThreads;
             const bool ok = full || i < nvec;
-            c[j] = ok ? static_cast<uint32_t>(c4[i]) : 0u;
-            if (ADD) a[j] = ok ? static_cast<f4a>(o4[i]) : f4a{0.f, 0.f, 0.f, 0.f};
+            c[j] = ok ? M::ldu32(codes, i) : 0u;
+            if (ADD) a[j] = ok ? M::ldf4(out, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
@@ -356,7 +455,7 @@ __global__ __launch_bounds__(kThreads) void dequant_kernel(float* __restrict__ o
             v.w = s_lut[c[j] >> 24];
             if (ADD) v += a[j];
             if (full || i < nvec) {
-                o4[i] = v;
+                M::stf4(out, i, v, !STATS);   // with STATS the quantize pass reads it again: no streaming hint
                 if (STATS) {
                     if (j & 1) stats_add4(v, s1, q1); else stats_add4(v, s0, q0);
                 }
@@ -374,7 +473,7 @@ __global__ __launch_bounds__(kThreads) void dequant_kernel(float* __restrict__ o
             q0 = fma(d, d, q0);
         }
     }
-    if (STATS) block_stats_finish(s0 + s1, q0 + q1, n, ws, qp_out);
+    if (STATS) block_stats_store(s0 + s1, q0 + q1, ws);
 }
 
 // Small tensors: one workgroup per tensor of a flat buffer does the whole of
@@ -430,9 +529,20 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
 }
 
 __global__ __launch_bounds__(kThreads) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
-    for (int64_t i = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x; i < nvec;
-         i += static_cast<int64_t>(gridDim.x) * kThreads)
-        dst[i] = src[i];
+    const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
+    for (int64_t base = blockIdx.x * tile; base < nvec; base += static_cast<int64_t>(gridDim.x) * tile) {
+        f4a v[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = base + threadIdx.x + j * kThreads;
+            if (i < nvec) v[j] = Mem<true>::ldf4(reinterpret_cast<const float*>(src), i);
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = base + threadIdx.x + j * kThreads;
+            if (i < nvec) Mem<true>::stf4(reinterpret_cast<float*>(dst), i, v[j], true);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -469,9 +579,11 @@ int cu_count() {
     return cus[dev];
 }
 
-// Workgroups for a kernel whose workgroups each loop over tiles of `tile_elems` elements.
-int grid_for(int64_t n, int64_t tile_elems) {
-    int64_t tiles = (n + tile_elems - 1) / tile_elems;
+constexpr int64_t kTileElems = static_cast<int64_t>(kThreads) * kUnroll * 4;
+
+// Workgroups for a kernel whose workgroups each loop over tiles of kTileElems elements.
+int grid_for(int64_t n) {
+    int64_t tiles = (n + kTileElems - 1) / kTileElems;
     if (tiles < 1) tiles = 1;
     int64_t cap = static_cast<int64_t>(cu_count()) * g_opt.blocks_per_cu;
     if (cap > kMaxGrid) cap = kMaxGrid;
@@ -480,20 +592,24 @@ int grid_for(int64_t n, int64_t tile_elems) {
 
 inline bool aligned_to(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-constexpr int64_t kTileElems = static_cast<int64_t>(kThreads) * kUnroll * 4;
-
 int launch_check(const char* where) {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? 0 : hip_fail(e, where);
 }
 
+int run_stats_finalize(Workspace* ws, int nparts, int64_t n, prime_qparams* out, hipStream_t st) {
+    hipLaunchKernelGGL(stats_finalize_kernel, dim3(1), dim3(kFinalThreads), 0, st, ws, nparts, n, out);
+    return launch_check("stats_finalize_kernel");
+}
+
 int run_stats(const float* x, int64_t n, prime_qparams* out, Workspace* ws, hipStream_t st) {
-    const int grid = grid_for(n, kTileElems);
+    const int grid = grid_for(n);
     if (aligned_to(x, 16))
-        hipLaunchKernelGGL(stats_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, n, ws, out);
+        hipLaunchKernelGGL(stats_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, n, ws);
     else
-        hipLaunchKernelGGL(stats_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, n, ws, out);
-    return launch_check("stats_kernel");
+        hipLaunchKernelGGL(stats_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+    if (int rc = launch_check("stats_kernel")) return rc;
+    return run_stats_finalize(ws, grid, n, out, st);
 }
 
 template <bool HIST, int R>
@@ -505,9 +621,10 @@ void launch_quantize_r(bool al, int grid, hipStream_t st, const float* x, int64_
         hipLaunchKernelGGL((quantize_kernel<false, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, qp, zp, codes, ws, reverse);
 }
 
+// Returns the grid size through *grid_out: the number of histogram partials written.
 int run_quantize(const float* x, int64_t n, float scale, const prime_qparams* qp, int zp, uint8_t* codes, Workspace* ws,
-                 bool hist, int reverse, hipStream_t st) {
-    const int grid = grid_for(n, kTileElems);
+                 bool hist, int reverse, hipStream_t st, int* grid_out) {
+    const int grid = grid_for(n);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
     if (!hist) {
         launch_quantize_r<false, 1>(al, grid, st, x, n, scale, qp, zp, codes, ws, reverse);
@@ -519,25 +636,32 @@ int run_quantize(const float* x, int64_t n, float scale, const prime_qparams* qp
             default: launch_quantize_r<true, 4>(al, grid, st, x, n, scale, qp, zp, codes, ws, reverse); break;
         }
     }
+    if (grid_out) *grid_out = grid;
     return launch_check("quantize_kernel");
 }
 
-int run_lut_finalize(Workspace* ws, float* lut, int64_t n_bins, uint64_t* counts, hipStream_t st) {
-    hipLaunchKernelGGL(lut_finalize_kernel, dim3(1), dim3(kThreads), 0, st, ws, lut, n_bins,
+int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins, uint64_t* counts, hipStream_t st) {
+    if (nparts == 0) {
+        hipLaunchKernelGGL(lut_zero_kernel, dim3(1), dim3(kThreads), 0, st, lut, n_bins, reinterpret_cast<unsigned long long*>(counts));
+        return launch_check("lut_zero_kernel");
+    }
+    hipLaunchKernelGGL(lut_finalize_kernel, dim3(kBins / kLutBinsPerBlock), dim3(kFinalThreads), 0, st, ws, nparts, lut, n_bins,
                        reinterpret_cast<unsigned long long*>(counts));
     return launch_check("lut_finalize_kernel");
 }
 
 template <bool ADD, bool STATS>
-int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, prime_qparams* qp_out,
-                hipStream_t st) {
-    const int grid = grid_for(n, kTileElems);
+int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out) {
+    const int grid = grid_for(n);
     if (aligned_to(out, 16) && aligned_to(codes, 4))
-        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, true>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws, qp_out);
+        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, true>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
     else
-        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, false>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws, qp_out);
+        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, false>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
+    if (grid_out) *grid_out = grid;
     return launch_check("dequant_kernel");
 }
+
+bool bad_n(int64_t n) { return n < 0 || n > kMaxElems; }
 
 }  // namespace
 
@@ -568,6 +692,7 @@ int prime_hip_get_option(const char* name, int* value) {
     if (!strcmp(name, "blocks_per_cu")) *value = g_opt.blocks_per_cu;
     else if (!strcmp(name, "hist_replicas")) *value = g_opt.hist_replicas;
     else if (!strcmp(name, "reverse_second_pass")) *value = g_opt.reverse_second_pass;
+    else if (!strcmp(name, "unroll")) *value = kUnroll;
     else return fail(PRIME_EINVAL, "unknown option");
     return 0;
 }
@@ -578,33 +703,35 @@ int prime_workspace_init(void* ws, int64_t ws_bytes, prime_stream_t stream) {
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     if (ws_bytes < static_cast<int64_t>(sizeof(Workspace))) return fail(PRIME_EWORKSPACE, "workspace too small");
     if (!aligned_to(ws, 16)) return fail(PRIME_EWORKSPACE, "workspace must be 16-byte aligned");
-    const int64_t words = static_cast<int64_t>(sizeof(Workspace) / 4);
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(32), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
-                       static_cast<uint32_t*>(ws), words);
+    // Only the scale record is ever read before it is written by the same call sequence;
+    // clear it so that a stray read is defined.
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint32_t*>(ws), static_cast<int64_t>(sizeof(prime_qparams) / 4));
     return launch_check("fill_zero_kernel");
 }
 
 int prime_stats_f32(const float* x, int64_t n, prime_qparams* out, void* ws, prime_stream_t stream) {
-    if (n < 0 || (!x && n > 0) || !out) return fail(PRIME_EINVAL, "prime_stats_f32: bad argument");
+    if (bad_n(n) || (!x && n > 0) || !out) return fail(PRIME_EINVAL, "prime_stats_f32: bad argument");
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     return run_stats(x, n, out, static_cast<Workspace*>(ws), static_cast<hipStream_t>(stream));
 }
 
 int prime_quantize_u8(const float* x, int64_t n, float scale, int32_t zero_point, uint8_t* codes, prime_stream_t stream) {
-    if (n < 0 || (n > 0 && (!x || !codes))) return fail(PRIME_EINVAL, "prime_quantize_u8: bad argument");
+    if (bad_n(n) || (n > 0 && (!x || !codes))) return fail(PRIME_EINVAL, "prime_quantize_u8: bad argument");
     if (n == 0) return 0;
-    return run_quantize(x, n, scale, nullptr, zero_point, codes, nullptr, false, 0, static_cast<hipStream_t>(stream));
+    return run_quantize(x, n, scale, nullptr, zero_point, codes, nullptr, false, 0, static_cast<hipStream_t>(stream), nullptr);
 }
 
 int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64_t n_bins, float* lut, uint64_t* counts,
                           void* ws, prime_stream_t stream) {
-    if (n < 0 || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_average_buckets: bad argument");
+    if (bad_n(n) || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_average_buckets: bad argument");
     if (n_bins < 1 || n_bins > (1 << 24)) return fail(PRIME_EINVAL, "prime_average_buckets: n_bins out of range");
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     hipStream_t st = static_cast<hipStream_t>(stream);
     Workspace* w = static_cast<Workspace*>(ws);
+    int grid = 0;
     if (n > 0) {
-        const int grid = grid_for(n, static_cast<int64_t>(kThreads) * 4 * 4);
+        grid = grid_for(n);
         const int nb = static_cast<int>(n_bins < kBins ? n_bins : kBins);
         if (aligned_to(x, 16) && aligned_to(codes, 4))
             hipLaunchKernelGGL((hist_kernel<true, 4>), dim3(grid), dim3(kThreads), 0, st, x, codes, n, nb, w);
@@ -612,30 +739,32 @@ int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64
             hipLaunchKernelGGL((hist_kernel<false, 4>), dim3(grid), dim3(kThreads), 0, st, x, codes, n, nb, w);
         if (int rc = launch_check("hist_kernel")) return rc;
     }
-    return run_lut_finalize(w, lut, n_bins, counts, st);
+    return run_lut_finalize(w, grid, lut, n_bins, counts, st);
 }
 
 int prime_quantize_lookup_u8(const float* x, int64_t n, float scale, uint8_t* codes, float* lut, void* ws,
                              prime_stream_t stream) {
-    if (n < 0 || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_quantize_lookup_u8: bad argument");
+    if (bad_n(n) || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_quantize_lookup_u8: bad argument");
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     hipStream_t st = static_cast<hipStream_t>(stream);
     Workspace* w = static_cast<Workspace*>(ws);
+    int grid = 0;
     if (n > 0)
-        if (int rc = run_quantize(x, n, scale, nullptr, kZeroPoint, codes, w, true, 0, st)) return rc;
-    return run_lut_finalize(w, lut, kBins, nullptr, st);
+        if (int rc = run_quantize(x, n, scale, nullptr, kZeroPoint, codes, w, true, 0, st, &grid)) return rc;
+    return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
 }
 
 int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out, void* ws,
                                 prime_stream_t stream) {
-    if (n < 0 || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize: bad argument");
+    if (bad_n(n) || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize: bad argument");
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     hipStream_t st = static_cast<hipStream_t>(stream);
     Workspace* w = static_cast<Workspace*>(ws);
     if (int rc = run_stats(x, n, qparams_out, w, st)) return rc;
+    int grid = 0;
     if (n > 0)
-        if (int rc = run_quantize(x, n, 0.0f, &w->qp, kZeroPoint, codes, w, true, g_opt.reverse_second_pass, st)) return rc;
-    return run_lut_finalize(w, lut, kBins, nullptr, st);
+        if (int rc = run_quantize(x, n, 0.0f, &w->qp, kZeroPoint, codes, w, true, g_opt.reverse_second_pass, st, &grid)) return rc;
+    return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
 }
 
 int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, int64_t count, uint8_t* codes, float* luts,
@@ -649,31 +778,33 @@ int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, 
 }
 
 int prime_dequant_set(float* out, const float* lut, const uint8_t* codes, int64_t n, prime_stream_t stream) {
-    if (n < 0 || (n > 0 && (!out || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_dequant_set: bad argument");
+    if (bad_n(n) || (n > 0 && (!out || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_dequant_set: bad argument");
     if (n == 0) return 0;
-    return run_dequant<false, false>(out, lut, codes, n, nullptr, nullptr, static_cast<hipStream_t>(stream));
+    return run_dequant<false, false>(out, lut, codes, n, nullptr, static_cast<hipStream_t>(stream), nullptr);
 }
 
 int prime_dequant_add(float* out, const float* lut, const uint8_t* codes, int64_t n, prime_stream_t stream) {
-    if (n < 0 || (n > 0 && (!out || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_dequant_add: bad argument");
+    if (bad_n(n) || (n > 0 && (!out || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_dequant_add: bad argument");
     if (n == 0) return 0;
-    return run_dequant<true, false>(out, lut, codes, n, nullptr, nullptr, static_cast<hipStream_t>(stream));
+    return run_dequant<true, false>(out, lut, codes, n, nullptr, static_cast<hipStream_t>(stream), nullptr);
 }
 
 int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out,
                            float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
-    if (n < 0 || (n > 0 && (!acc || !codes_in || !codes_out)) || !lut_in || !lut_out)
+    if (bad_n(n) || (n > 0 && (!acc || !codes_in || !codes_out)) || !lut_in || !lut_out)
         return fail(PRIME_EINVAL, "prime_ring_reduce_step: bad argument");
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     hipStream_t st = static_cast<hipStream_t>(stream);
     Workspace* w = static_cast<Workspace*>(ws);
     if (n == 0) {
         if (int rc = run_stats(acc, 0, qparams_out, w, st)) return rc;
-        return run_lut_finalize(w, lut_out, kBins, nullptr, st);
+        return run_lut_finalize(w, 0, lut_out, kBins, nullptr, st);
     }
-    if (int rc = run_dequant<true, true>(acc, lut_in, codes_in, n, w, qparams_out, st)) return rc;
-    if (int rc = run_quantize(acc, n, 0.0f, &w->qp, kZeroPoint, codes_out, w, true, g_opt.reverse_second_pass, st)) return rc;
-    return run_lut_finalize(w, lut_out, kBins, nullptr, st);
+    int grid = 0;
+    if (int rc = run_dequant<true, true>(acc, lut_in, codes_in, n, w, st, &grid)) return rc;
+    if (int rc = run_stats_finalize(w, grid, n, qparams_out, st)) return rc;
+    if (int rc = run_quantize(acc, n, 0.0f, &w->qp, kZeroPoint, codes_out, w, true, g_opt.reverse_second_pass, st, &grid)) return rc;
+    return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
 }
 
 int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t stream) {
@@ -682,7 +813,7 @@ int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t
         return fail(PRIME_EINVAL, "prime_copy_bytes: size and pointers must be multiples of 16");
     if (n_bytes == 0) return 0;
     const int64_t nvec = n_bytes >> 4;
-    const int grid = grid_for(nvec, kThreads);
+    const int grid = grid_for(nvec * 4);
     hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<f4a*>(dst), static_cast<const f4a*>(src), nvec);
     return launch_check("copy_kernel");

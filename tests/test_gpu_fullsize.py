@@ -1,0 +1,77 @@
+"""Full-size runs (2^28 elements; 2^26-element ring chunks) checked through properties that
+do not need the CPU oracle: torch on the GPU is used as a plain calculator here."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import Abi, announce
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def abi(dev):
+    return Abi(dev)
+
+
+def test_uniform_8bit_quantize_2p28_properties(abi):
+    n = 1 << 28
+    g = torch.Generator(device=abi.dev).manual_seed(0)
+    x = torch.randn(n, device=abi.dev, generator=g) * 1e-3
+    announce("2^28 uniform")
+    codes, lut, qp = abi.uniform(x)
+    torch.cuda.synchronize()
+    q = abi.qparams(qp)
+    # scale: the reference's formula on an fp64 sum of squares
+    sumsq = float((x.double() ** 2).sum())
+    want = np.float32(6.0 * (float(np.float32(np.sqrt(sumsq))) / np.sqrt(n - 1)) / 256.0)
+    assert abs(q["sumsq"] - sumsq) <= 1e-12 * sumsq
+    assert abs(float(q["scale"]) - float(want)) <= 1e-6 * float(want)
+    assert abs(q["sum"] - float(x.double().sum())) <= 1e-12 * float(x.double().abs().sum())
+    # codes: the same arithmetic spelled with torch ops (multiply, round half away, clamp)
+    inv = torch.tensor(1.0, dtype=torch.float32) / torch.tensor(float(q["scale"]), dtype=torch.float32)
+    p = x * float(inv)
+    r = torch.where(p >= 0, torch.floor(p + 0.5), torch.ceil(p - 0.5))
+    r = torch.where((p - torch.trunc(p)).abs() == 0.5, torch.trunc(p) + torch.sign(p), torch.round(p))
+    want_codes = (r.clamp(-128, 127) + 128).to(torch.uint8)
+    assert torch.equal(codes, want_codes)
+    del p, r, want_codes
+    # lookup: counts add up, count-weighted means give back the sum, bins are ordered
+    cnt = torch.bincount(codes.view(-1).int(), minlength=256).double()
+    assert int(cnt.sum()) == n
+    sums = torch.zeros(256, dtype=torch.float64, device=abi.dev).index_add_(0, codes.long(), x.double())
+    mean = torch.where(cnt > 0, sums / cnt.clamp(min=1), torch.zeros_like(sums))
+    err = (lut.double() - mean).abs() / torch.maximum(mean.abs(), torch.tensor(float(q["scale"]), device=abi.dev, dtype=torch.float64))
+    assert float(err.max()) <= 1e-6
+    assert abs(float((cnt * lut.double()).sum()) - float(x.double().sum())) <= 1e-6 * float(x.double().abs().sum())
+    filled = lut[cnt > 0]
+    assert bool((filled[1:] > filled[:-1]).all())
+    # dequantize: a gather, and within one bin width of the input for unclipped elements
+    out = torch.empty_like(x)
+    abi.dequant(out, lut, codes, add=False)
+    assert torch.equal(out, lut[codes.long()])
+    inside = (codes > 0) & (codes < 255)
+    assert float((out - x)[inside].abs().max()) <= float(q["scale"])
+
+
+def test_ring_reduce_step_2p26_chunks(abi):
+    # BASELINE config 3 shape: 2^26-element chunks; three ranks' worth to bound memory and time
+    n = 1 << 26
+    g = torch.Generator(device=abi.dev).manual_seed(1)
+    x0 = torch.randn(n, device=abi.dev, generator=g) * 1e-3
+    announce("2^26 ring: quantize rank 0")
+    codes, lut, _ = abi.uniform(x0)
+    for r in (1, 2):
+        acc = torch.randn(n, device=abi.dev, generator=g) * 1e-3
+        want = acc + lut[codes.long()]
+        announce(f"2^26 ring hop {r}")
+        codes, lut, qp = abi.ring_step(acc, codes, lut)
+        torch.cuda.synchronize()
+        assert torch.equal(acc, want)
+        q = abi.qparams(qp)
+        sumsq = float((want.double() ** 2).sum())
+        assert abs(q["sumsq"] - sumsq) <= 1e-12 * sumsq
+        cnt = torch.bincount(codes.int(), minlength=256)
+        assert int(cnt.sum()) == n
+        inside = (codes > 0) & (codes < 255)
+        assert float((lut[codes.long()] - want)[inside].abs().max()) <= float(q["scale"])

@@ -1,0 +1,360 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on the BASELINE
+configurations at sizes the oracle finishes in seconds.
+
+Bars: uint8 codes, dequantized values and accumulators bit-exact; scale equal to the float
+the reference's formula gives on an exact sum of squares (and within 1e-6 relative of the
+golden, libtorch-accumulated value at small n); lookup entries within 1e-6 relative of the
+fp64 bin mean, with one bin width as the floor for bins whose mean is near zero.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from tests.conftest import lut_rel_err
+from tests.golden.make_fixtures import CASES, case_input
+from tests.gpu_util import Abi, announce
+
+pytestmark = pytest.mark.gpu
+
+LUT_TOL = 1e-6
+
+
+@pytest.fixture(scope="module")
+def abi(dev):
+    return Abi(dev)
+
+
+def check_uniform(abi, oracle, x: np.ndarray, label: str):
+    """uniform_8bit_quantize on the GPU against the oracle for one tensor; returns GPU outputs."""
+    announce(f"{label} n={x.size}")
+    xt = abi.to_dev(x)
+    codes, lut, qp = abi.uniform(xt)
+    torch.cuda.synchronize()
+    q = abi.qparams(qp)
+    gc, gl = codes.cpu().numpy(), lut.cpu().numpy()
+    s, sq = oracle.stats_f64(x)
+    assert q["n"] == x.size
+    assert abs(q["sum"] - s) <= 1e-12 * max(np.abs(x).astype(np.float64).sum(), 1e-300), label
+    assert abs(q["sumsq"] - sq) <= 1e-12 * max(sq, 1e-300), label
+    want_scale = oracle.scale_exact(x)
+    assert np.array_equal(np.array([q["scale"]]), np.array([want_scale]), equal_nan=True), (label, q["scale"], want_scale)
+    oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
+    assert np.array_equal(gc, oc), (label, int((gc != oc).sum()))
+    mean, _ = oracle.average_buckets_f64(x, gc)
+    floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+    assert lut_rel_err(gl, mean, floor) <= LUT_TOL, label
+    return xt, codes, lut, q
+
+
+def test_cfg1_round_trip_2p24(abi, oracle):
+    # BASELINE config 1: 2^24 elements, N(0, 1e-3), seed 0; quantize then dequantize
+    x = (np.random.default_rng(0).standard_normal(1 << 24) * 1e-3).astype(np.float32)
+    xt, codes, lut, q = check_uniform(abi, oracle, x, "cfg1")
+    out = torch.empty_like(xt)
+    abi.dequant(out, lut, codes, add=False)
+    gl, gc = lut.cpu().numpy(), codes.cpu().numpy()
+    assert np.array_equal(out.cpu().numpy(), gl[gc])
+    inside = (gc > 0) & (gc < 255)
+    assert np.abs(out.cpu().numpy()[inside] - x[inside]).max() <= q["scale"]
+    # the literal reference scale (libtorch's fp32 accumulation) injected: codes equal to the
+    # reference's at any n
+    lit = float(oracle.scale_literal(x))
+    announce(f"cfg1 literal scale {lit!r} vs exact {float(q['scale'])!r} ratio-1 = {lit / float(q['scale']) - 1:.3e}")
+    c2, l2 = abi.quantize_lookup(xt, lit)
+    oc, ol, _ = oracle.uniform_8bit_quantize(x, "literal")
+    assert np.array_equal(c2.cpu().numpy(), oc)
+    mean, _ = oracle.average_buckets_f64(x, oc)
+    assert lut_rel_err(l2.cpu().numpy(), mean, lit) <= LUT_TOL
+    if oracle.ref_available():
+        rc, _ = oracle.ref().uniform_8bit_quantize(torch.from_numpy(x.copy()), True)
+        assert np.array_equal(c2.cpu().numpy(), rc.numpy())
+
+
+def test_cfg2_llama_1b_layer_bucket(abi, oracle):
+    # BASELINE config 2: one per-layer bucket, 4*2048*2048 + 3*2048*5632 elements, Student-t(3) * 1e-4
+    n = 4 * 2048 * 2048 + 3 * 2048 * 5632
+    assert n == 51_380_224
+    x = (np.random.default_rng(0).standard_t(3, n) * 1e-4).astype(np.float32)
+    _, codes, _, _ = check_uniform(abi, oracle, x, "cfg2 layer 0")
+    gc = codes.cpu().numpy()
+    assert (gc == 0).mean() > 1e-3 and (gc == 255).mean() > 1e-3      # heavy tails fill the clip bins
+
+
+def test_cfg3_ring_hops_w8(abi, oracle):
+    # BASELINE config 3 at chunk 2^20: W = 8 ranks, hop by hop with identical inputs on both sides
+    W, n = 8, 1 << 20
+    chunks = [(np.random.default_rng(r).standard_normal(n) * 1e-3).astype(np.float32) for r in range(W)]
+    xt, codes, lut, q = check_uniform(abi, oracle, chunks[0], "cfg3 rank 0")
+    total_scale = float(q["scale"])
+    inside = (codes.cpu().numpy() > 0) & (codes.cpu().numpy() < 255)
+    for r in range(1, W):
+        announce(f"cfg3 hop {r}")
+        acc = abi.to_dev(chunks[r])
+        c_in, l_in = codes.cpu().numpy(), lut.cpu().numpy()
+        codes, lut, qp = abi.ring_step(acc, codes, lut)
+        torch.cuda.synchronize()
+        want_acc = chunks[r].copy()
+        oracle.index_add(want_acc, l_in, c_in)                       # collectives.cpp:128-133
+        got_acc = acc.cpu().numpy()
+        assert np.array_equal(got_acc, want_acc), r
+        q = abi.qparams(qp)
+        assert q["scale"] == oracle.scale_exact(want_acc)
+        oc, _, _ = oracle.uniform_8bit_quantize(want_acc, "given", scale=float(q["scale"]))
+        gc = codes.cpu().numpy()
+        assert np.array_equal(gc, oc), r
+        mean, _ = oracle.average_buckets_f64(want_acc, gc)
+        assert lut_rel_err(lut.cpu().numpy(), mean, float(q["scale"])) <= LUT_TOL
+        # the accumulator holds this rank's data plus the (lossy) running sum
+        chunks[r] = want_acc
+        if r < W - 1:
+            total_scale += float(q["scale"])
+            inside &= (gc > 0) & (gc < 255)
+    exact = np.sum(np.stack([(np.random.default_rng(r).standard_normal(n) * 1e-3).astype(np.float32) for r in range(W)])
+                   .astype(np.float64), axis=0)
+    assert np.abs(chunks[W - 1][inside] - exact[inside]).max() <= total_scale
+
+
+def test_cfg4_fsdp_shard_bucket_with_outliers(abi, oracle):
+    # BASELINE config 4: 1.25e9 elements in 42 buckets of 29,761,904, the last one 32 longer;
+    # N(0, 5e-4) with 0.01 % of entries at +-50 sigma.  The last bucket is checked in full.
+    n = 29_761_904 + 32
+    assert 41 * 29_761_904 + n == 1_250_000_000
+    rng = np.random.default_rng(41)
+    x = (rng.standard_normal(n) * 5e-4).astype(np.float32)
+    k = n // 10000
+    pos = rng.choice(n, k, replace=False)
+    x[pos] = np.where(rng.random(k) < 0.5, -1.0, 1.0).astype(np.float32) * np.float32(50 * 5e-4)
+    xt, codes, lut, q = check_uniform(abi, oracle, x, "cfg4 bucket 41")
+    gc = codes.cpu().numpy()
+    assert set(np.unique(gc[pos])) == {0, 255}
+    out = torch.empty_like(xt)
+    abi.dequant(out, lut, codes, add=False)
+    assert np.array_equal(out.cpu().numpy(), lut.cpu().numpy()[gc])
+
+
+def test_cfg5_two_thousand_small_tensors_batched(abi, oracle):
+    # BASELINE config 5: 2,000 tensors of sizes U[1, 65536], N(1, 1e-2), one launch
+    rng = np.random.default_rng(5)
+    sizes = rng.integers(1, 65536, 2000, endpoint=True)
+    off = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    flat = (1 + rng.standard_normal(off[-1]) * 1e-2).astype(np.float32)
+    announce(f"cfg5 batched total={off[-1]}")
+    ft, ot = abi.to_dev(flat), abi.to_dev(off)
+    codes, luts, qps = abi.batched(ft, ot)
+    torch.cuda.synchronize()
+    gc, gl, gq = codes.cpu().numpy(), luts.cpu().numpy(), qps.cpu()
+    for t in range(2000):
+        xs = flat[off[t]:off[t + 1]]
+        q = abi.qparams(gq[t])
+        want = oracle.scale_exact(xs)
+        assert np.array_equal(np.array([q["scale"]]), np.array([want]), equal_nan=True), (t, xs.size)
+        oc, _, _ = oracle.uniform_8bit_quantize(xs, "given", scale=float(q["scale"]))
+        assert np.array_equal(gc[off[t]:off[t + 1]], oc), (t, xs.size)
+        mean, _ = oracle.average_buckets_f64(xs, oc)
+        floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+        assert lut_rel_err(gl[t], mean, floor) <= LUT_TOL, (t, xs.size)
+    # the one-tensor entry point gives the same codes as the batched one
+    for t in (0, 1, 7, 500, 1999):
+        announce(f"cfg5 single tensor {t} n={sizes[t]}")
+        c1, l1, _ = abi.uniform(ft[off[t]:off[t + 1]])
+        assert np.array_equal(c1.cpu().numpy(), gc[off[t]:off[t + 1]])
+        assert np.allclose(l1.cpu().numpy(), gl[t], rtol=1e-6, atol=0)
+
+
+def test_cfg5_edge_tensors(abi, oracle):
+    n = 1 << 20
+    # constant, non-zero: every code is round(256/6 * sqrt((n-1)/n)) + 128 = 171
+    xt, codes, lut, q = check_uniform(abi, oracle, np.full(n, 0.25, np.float32), "cfg5 constant")
+    assert (codes.cpu().numpy() == 171).all() and lut.cpu().numpy()[171] == np.float32(0.25)
+    assert np.count_nonzero(lut.cpu().numpy()) == 1
+    # all zero: scale 0, x * inf = NaN -> code 0, lookup all zero
+    xt, codes, lut, q = check_uniform(abi, oracle, np.zeros(n, np.float32), "cfg5 zeros")
+    assert q["scale"] == 0 and not codes.cpu().numpy().any() and not lut.cpu().numpy().any()
+    # half exact zeros
+    rng = np.random.default_rng(50)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    x[rng.random(n) < 0.5] = 0.0
+    xt, codes, lut, q = check_uniform(abi, oracle, x, "cfg5 half zeros")
+    assert (codes.cpu().numpy() == 128).mean() > 0.5
+    # non-aligned tail
+    x = (np.random.default_rng(51).standard_normal((1 << 24) + 7) * 1e-3).astype(np.float32)
+    xt, codes, lut, q = check_uniform(abi, oracle, x, "cfg5 2^24+7")
+    out = torch.empty_like(xt)
+    abi.dequant(out, lut, codes, add=False)
+    assert np.array_equal(out.cpu().numpy(), lut.cpu().numpy()[codes.cpu().numpy()])
+
+
+@pytest.mark.parametrize("n", [0, 1, 2, 3, 5, 63, 64, 65, 255, 1023, 1024, 1025, 4099, 65543, 262147])
+def test_small_and_ragged_sizes(abi, oracle, n):
+    rng = np.random.default_rng(1000 + n)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    if n == 0:
+        announce("empty tensor")
+        xt = torch.empty(0, dtype=torch.float32, device=abi.dev)
+        codes, lut, qp = abi.uniform(xt)
+        torch.cuda.synchronize()
+        assert codes.numel() == 0 and not lut.cpu().numpy().any()
+        return
+    xt, codes, lut, q = check_uniform(abi, oracle, x, "ragged")
+    acc0 = rng.standard_normal(n).astype(np.float32)
+    acc = abi.to_dev(acc0)
+    abi.dequant(acc, lut, codes, add=True)
+    want = acc0.copy()
+    oracle.index_add(want, lut.cpu().numpy(), codes.cpu().numpy())
+    assert np.array_equal(acc.cpu().numpy(), want)
+
+
+def test_single_zero_element_gives_nan_scale_and_code_zero(abi, oracle):
+    xt, codes, lut, q = check_uniform(abi, oracle, np.zeros(1, np.float32), "n=1 zero")
+    assert np.isnan(q["scale"]) and codes.cpu().numpy()[0] == 0
+    xt, codes, lut, q = check_uniform(abi, oracle, np.array([0.7], np.float32), "n=1")
+    assert np.isinf(q["scale"]) and codes.cpu().numpy()[0] == 128 and lut.cpu().numpy()[128] == np.float32(0.7)
+
+
+@pytest.mark.parametrize("shift", [1, 2, 3])
+def test_buffers_that_are_only_element_aligned(abi, oracle, shift):
+    # views that start at an odd element: the 16-byte fast path must not be taken
+    n = 100003
+    rng = np.random.default_rng(shift)
+    base = (rng.standard_normal(n + 8) * 1e-3).astype(np.float32)
+    bt = abi.to_dev(base)
+    xv = bt[shift:shift + n]
+    x = base[shift:shift + n]
+    announce(f"misaligned x shift={shift}")
+    codes, lut, qp = abi.uniform(xv)
+    q = abi.qparams(qp)
+    assert q["scale"] == oracle.scale_exact(x)
+    oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
+    assert np.array_equal(codes.cpu().numpy(), oc)
+    # codes buffer misaligned as well
+    cbuf = torch.zeros(n + 8, dtype=torch.uint8, device=abi.dev)
+    cv = cbuf[shift:shift + n]
+    abi.quantize(xv, float(q["scale"]), 128, codes=cv)
+    assert np.array_equal(cv.cpu().numpy(), oc)
+    assert not cbuf[:shift].cpu().numpy().any() and not cbuf[shift + n:].cpu().numpy().any()
+    # dequantize into / accumulate onto a misaligned output, misaligned codes
+    obuf = torch.zeros(n + 8, dtype=torch.float32, device=abi.dev)
+    ov = obuf[shift:shift + n]
+    abi.dequant(ov, lut, cv, add=False)
+    gl = lut.cpu().numpy()
+    assert np.array_equal(ov.cpu().numpy(), gl[oc])
+    abi.dequant(ov, lut, cv, add=True)
+    assert np.array_equal(ov.cpu().numpy(), gl[oc] + gl[oc])
+    assert not obuf[:shift].cpu().numpy().any() and not obuf[shift + n:].cpu().numpy().any()
+    # ring step on a misaligned accumulator
+    acc0 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    abuf = torch.zeros(n + 8, dtype=torch.float32, device=abi.dev)
+    av = abuf[shift:shift + n]
+    av.copy_(abi.to_dev(acc0))
+    c2, l2, qp2 = abi.ring_step(av, cv, lut)
+    want = acc0.copy()
+    oracle.index_add(want, gl, oc)
+    assert np.array_equal(av.cpu().numpy(), want)
+    q2 = abi.qparams(qp2)
+    oc2, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q2["scale"]))
+    assert q2["scale"] == oracle.scale_exact(want) and np.array_equal(c2.cpu().numpy(), oc2)
+
+
+def test_quantize_special_values_and_denormals(abi, oracle):
+    announce("specials")
+    sp = np.array([np.nan, np.inf, -np.inf, 3e38, -3e38, 2147483520.0, 2147483648.0, -2147483648.0, 2147483392.0,
+                   0.5, -0.5, 1.5, 2.5, -2.5, 126.5, 127.5, -128.5, -127.5, 1e-40, -1e-40, 0.49999997, -0.49999997],
+                  np.float32)
+    for scale, zp in [(1.0, 128), (1.0, 0), (0.5, 200), (3.0, -5)]:
+        got = abi.quantize(abi.to_dev(sp), scale, zp).cpu().numpy()
+        assert np.array_equal(got, oracle.quantize_per_tensor_uint8(sp, scale, zp)), (scale, zp)
+    den = np.array([1e-39, -1e-39, 3e-39, 5e-39, 1.2e-38, -7e-39], np.float32)
+    got = abi.quantize(abi.to_dev(den), 3e-39, 128).cpu().numpy()
+    assert np.array_equal(got, oracle.quantize_per_tensor_uint8(den, 3e-39, 128))
+    assert len(set(got)) > 3       # denormal inputs and a denormal scale are not flushed
+
+
+def test_quantize_brute_force_around_every_boundary(abi, oracle):
+    announce("boundaries")
+    scale = np.float32(2.3418523e-05)
+    xs = []
+    for k in range(-130, 130):
+        v = np.float32((k + 0.5) * float(scale))
+        for _ in range(40):
+            v = np.nextafter(v, np.float32(-np.inf), dtype=np.float32)
+        for _ in range(80):
+            xs.append(v)
+            v = np.nextafter(v, np.float32(np.inf), dtype=np.float32)
+    x = np.array(xs, np.float32)
+    got = abi.quantize(abi.to_dev(x), float(scale), 128).cpu().numpy()
+    assert np.array_equal(got, oracle.quantize_per_tensor_uint8(x, float(scale), 128))
+
+
+def test_reference_test_vector_saturates(abi):
+    # tests/test_c/test_compression.py:46-48
+    announce("ones*10 / 0.01")
+    x = torch.ones(10_000_000, device=abi.dev) * 10
+    assert bool((abi.quantize(x, 0.01, 128) == 255).all())
+
+
+def test_average_buckets_with_foreign_codes(abi, oracle):
+    rng = np.random.default_rng(66)
+    n = 10_000_000                                     # the reference test's N (tests/test_c/test_compression.py:8)
+    x = (rng.standard_normal(n) * 10).astype(np.float32)
+    codes = rng.integers(0, 255, n).astype(np.uint8)
+    announce("average_buckets 1e7")
+    xt, ct = abi.to_dev(x), abi.to_dev(codes)
+    lut, cnt = abi.average_buckets(xt, ct, 256)
+    mean, c64 = oracle.average_buckets_f64(x, codes)
+    assert np.array_equal(cnt.cpu().numpy(), c64)
+    assert lut_rel_err(lut.cpu().numpy(), mean, 1e-3) <= LUT_TOL
+    assert lut.cpu().numpy()[255] == 0.0
+    # fewer bins: codes >= n_bins are skipped; more bins: the extra entries are zero
+    lut8, _ = abi.average_buckets(xt, ct, 8)
+    assert lut8.shape == (8,) and np.array_equal(lut8.cpu().numpy(), lut.cpu().numpy()[:8])
+    lut300, _ = abi.average_buckets(xt, ct, 300)
+    assert np.array_equal(lut300.cpu().numpy()[:256], lut.cpu().numpy()) and not lut300.cpu().numpy()[256:].any()
+    # integer-valued data: sums are exact in any order, so the table is bit-exact
+    xi = rng.integers(-50, 50, 1 << 20).astype(np.float32)
+    ci = rng.integers(0, 256, 1 << 20).astype(np.uint8)
+    li, _ = abi.average_buckets(abi.to_dev(xi), abi.to_dev(ci), 256)
+    mi, _ = oracle.average_buckets_f64(xi, ci)
+    assert np.array_equal(li.cpu().numpy(), mi.astype(np.float32))
+
+
+@pytest.mark.parametrize("name", CASES)
+def test_golden_fixtures_of_the_compiled_reference(abi, oracle, golden, name):
+    key = name.replace(":", "_")
+    x = case_input(name)
+    ref_scale = float(golden[f"{key}/scale"][0])
+    announce(f"golden {name}")
+    xt = abi.to_dev(x)
+    if np.isfinite(ref_scale) and ref_scale > 0:
+        # the reference's own scale injected: codes are the reference's, bit for bit
+        codes, lut = abi.quantize_lookup(xt, ref_scale)
+        assert np.array_equal(codes.cpu().numpy(), golden[f"{key}/codes"])
+        # its lookup carries fp32, thread-order noise: agree to that, and to 1e-6 with fp64
+        assert lut_rel_err(lut.cpu().numpy(), golden[f"{key}/lut"].astype(np.float64), ref_scale) < 2e-5
+        mean, _ = oracle.average_buckets_f64(x, golden[f"{key}/codes"])
+        assert lut_rel_err(lut.cpu().numpy(), mean, ref_scale) <= LUT_TOL
+    # end to end with the GPU's own scale
+    codes, lut, qp = abi.uniform(xt)
+    q = abi.qparams(qp)
+    if np.isfinite(ref_scale) and ref_scale > 0:
+        assert abs(float(q["scale"]) - ref_scale) <= 1e-6 * ref_scale
+        diff = codes.cpu().numpy() != golden[f"{key}/codes"]
+        if float(q["scale"]) == ref_scale:
+            assert not diff.any()
+        else:
+            # a scale one ulp away may move elements that sit on a bin boundary, by one code
+            assert diff.mean() <= 1e-4
+            d = codes.cpu().numpy().astype(int)[diff] - golden[f"{key}/codes"].astype(int)[diff]
+            assert (np.abs(d) == 1).all()
+    else:
+        assert np.array_equal(np.array([q["scale"]]), golden[f"{key}/scale"], equal_nan=True)
+        assert np.array_equal(codes.cpu().numpy(), golden[f"{key}/codes"])
+
+
+def test_results_do_not_depend_on_scheduling(abi):
+    announce("determinism")
+    x = torch.randn(3_000_001, device=abi.dev) * 1e-3
+    c1, l1, q1 = abi.uniform(x)
+    c2, l2, q2 = abi.uniform(x)
+    assert torch.equal(c1, c2) and torch.equal(l1, l2) and torch.equal(q1, q2)

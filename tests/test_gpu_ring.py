@@ -1,0 +1,121 @@
+"""The ring all-reduce schedule on W simulated ranks (one GPU), through the host-side mirror
+of the reference interface: ``all_reduce(Compression.UINT8, tensor, op, group)``."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.distributed as dist
+
+from tests.gpu_util import announce
+
+pytestmark = pytest.mark.gpu
+
+N = 1_000_000      # tests/test_c/test_collectives.py:13
+
+
+def _inputs(W, n, seed):
+    rng = np.random.default_rng(seed)
+    return [(rng.standard_normal(n) * 10).astype(np.float32) for _ in range(W)]      # test_collectives.py:39
+
+
+@pytest.mark.parametrize("W", [2, 4])
+def test_ring_allreduce_matches_cpu_ring_like_the_reference_test(dev, oracle, W):
+    # the reference's acceptance test (tests/test_c/test_collectives.py:14-57): the C ring and the
+    # Python ring must land equally far from the exact all-reduce,
+    # |norm(a - c) - norm(b - c)| / sqrt(N) < 0.5
+    from prime_amd.C.collectives import SimulatedRing
+    from prime_amd.collectives import Compression, all_reduce
+
+    n = N - N % (2 * W)
+    xs = _inputs(W, n, W)
+    exact = np.sum(np.stack(xs).astype(np.float64), axis=0)
+    cpu = [x.copy() for x in xs]
+    oracle.ring_allreduce_sim(cpu, avg=False)
+    announce(f"ring W={W}")
+    gpu = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    all_reduce(Compression.UINT8, gpu[0], dist.ReduceOp.SUM, SimulatedRing(gpu))
+    torch.cuda.synchronize()
+    for r in range(W):
+        a = gpu[r].cpu().numpy()
+        err_new = np.linalg.norm(a - exact)
+        err_old = np.linalg.norm(cpu[r] - exact)
+        assert abs(err_new - err_old) / math.sqrt(n) < 0.5
+        # far tighter in fact: both are a fraction of one bin of the summed data
+        assert abs(err_new - err_old) / math.sqrt(n) < 0.02
+        assert err_new / math.sqrt(n) < 1.5 * (6 * 10 * math.sqrt(W) / 256) * math.sqrt(W - 1)
+
+
+def test_ring_first_hop_is_bit_exact_against_cpu_ring(dev, oracle):
+    # with W = 2 each chunk makes one hop; codes sent on step 1 are a pure function of the input
+    from prime_amd import ring
+
+    W, n = 2, 4 * 65536
+    xs = _inputs(W, n, 9)
+    gpu = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    announce("ring first hop")
+    csz = n // (2 * W)
+    c = (0 * 2 - 1) % (2 * W)                       # rank 0, step 1 (collectives.cpp:116)
+    chunk = gpu[0][c * csz:(c + 1) * csz]
+    from tests.gpu_util import Abi
+
+    abi = Abi(dev)
+    codes, lut, qp = abi.uniform(chunk)
+    q = abi.qparams(qp)
+    oc, _, _ = oracle.uniform_8bit_quantize(xs[0][c * csz:(c + 1) * csz], "given", scale=float(q["scale"]))
+    assert q["scale"] == oracle.scale_exact(xs[0][c * csz:(c + 1) * csz])
+    assert np.array_equal(codes.cpu().numpy(), oc)
+    ring.ring_allreduce_simulated(gpu)              # and the whole schedule runs
+
+
+def test_ring_avg_and_single_rank(dev, oracle):
+    from prime_amd.C.collectives import SimulatedRing, ring_allreduce
+
+    W, n = 4, 8 * 4096
+    xs = _inputs(W, n, 3)
+    gpu = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    announce("ring AVG")
+    ring_allreduce(gpu[1], dist.ReduceOp.AVG, SimulatedRing(gpu))
+    exact = np.mean(np.stack(xs).astype(np.float64), axis=0)
+    for t in gpu:
+        assert np.linalg.norm(t.cpu().numpy() - exact) / math.sqrt(n) < 6 * 10 / 256
+    # one rank: no message, but the rank's two chunks take the quantize / dequantize round trip
+    x = xs[0]
+    t = torch.from_numpy(x.copy()).to(dev)
+    announce("ring W=1")
+    ring_allreduce(t, dist.ReduceOp.SUM, SimulatedRing([t]))
+    want = [x.copy()]
+    oracle.ring_allreduce_sim(want)
+    got = t.cpu().numpy()
+    assert len(np.unique(got[: n // 2])) <= 256 and len(np.unique(got[n // 2:])) <= 256
+    assert np.allclose(got, want[0], rtol=2e-6, atol=1e-6)
+    codes_a = oracle.uniform_8bit_quantize(x[: n // 2], "exact")[0]
+    # dequantized values map one-to-one onto the oracle's codes
+    assert len(np.unique(codes_a)) == len(np.unique(got[: n // 2]))
+
+
+def test_ops_layer_checks_on_device_tensors(dev):
+    from prime_amd.C import compression as C
+    from prime_amd import ops
+
+    x = torch.randn(1000, device=dev)
+    with pytest.raises(RuntimeError, match="Float"):
+        C.uniform_8bit_quantize(x.double())
+    with pytest.raises(RuntimeError, match="Byte"):
+        C.average_buckets(x, torch.zeros(1000, dtype=torch.int32, device=dev), 256)
+    with pytest.raises(RuntimeError, match="numel"):
+        C.average_buckets(x, torch.zeros(10, dtype=torch.uint8, device=dev), 256)
+    codes, lut = C.uniform_8bit_quantize(x.view(10, 100))
+    assert codes.shape == (10, 100) and codes.dtype == torch.uint8 and lut.shape == (256,)
+    # a non-contiguous input is read in logical order, never modified
+    xt = torch.randn(64, 32, device=dev)
+    before = xt.clone()
+    c1, l1 = C.uniform_8bit_quantize(xt.t(), True)
+    c2, l2 = C.uniform_8bit_quantize(xt.t().contiguous(), True)
+    assert torch.equal(c1, c2) and torch.equal(l1, l2) and torch.equal(xt, before)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ops.dequantize_(torch.zeros(64, 32, device=dev).t(), c1, l1, False)
+    q = C.quantize_per_tensor_uint8(torch.ones(1000, device=dev) * 10, 0.01, 128)
+    assert bool((q == 255).all())
+    d = ops.dequantize(c1, l1)
+    assert torch.equal(d, l1[c1.long()])

@@ -1,0 +1,107 @@
+"""Host-side mirror of the reference interface: names, signatures, error behaviour (CPU only)."""
+import inspect
+
+import pytest
+import torch
+import torch.distributed as dist
+
+
+def test_compression_enum_values():
+    # src/zeroband/config.py:10-12
+    from prime_amd.config import Compression
+
+    assert Compression.NO.value == "no" and Compression.UINT8.value == "uint8"
+    assert Compression("uint8") is Compression.UINT8
+
+
+def test_python_signatures_match_the_reference_wrappers():
+    # src/zeroband/C/compression.py:11,22,34 and src/zeroband/C/collectives.py:23-27, collectives.py:31-36
+    from prime_amd.C import collectives as Cc
+    from prime_amd.C import compression as C
+    from prime_amd import collectives
+
+    assert str(inspect.signature(C.uniform_8bit_quantize)) == \
+        "(tensor: torch.Tensor, inplace: bool = True) -> Tuple[torch.Tensor, torch.Tensor]"
+    assert list(inspect.signature(C.average_buckets).parameters) == ["tensor", "quant_weight", "n_bins"]
+    assert list(inspect.signature(C.quantize_per_tensor_uint8).parameters) == ["tensor", "scale", "zero_point"]
+    p = inspect.signature(Cc.ring_allreduce).parameters
+    assert list(p) == ["tensor", "op", "group"] and p["op"].default == dist.ReduceOp.SUM and p["group"].default is None
+    p = inspect.signature(collectives.all_reduce).parameters
+    assert list(p) == ["compression", "tensor", "op", "group"]
+
+
+def test_op_schemas():
+    import prime_amd.ops  # noqa: F401
+
+    want = {
+        "uniform_8bit_quantize": "prime::uniform_8bit_quantize(Tensor tensor, bool inplace=True) -> (Tensor, Tensor)",
+        "average_buckets": "prime::average_buckets(Tensor tensor, Tensor quant_weight, int n_bins) -> Tensor",
+        "quantize_per_tensor_uint8": "prime::quantize_per_tensor_uint8(Tensor tensor, float scale, int zero_point) -> Tensor",
+        "dequantize": "prime::dequantize(Tensor codes, Tensor lut) -> Tensor",
+        "ring_reduce_step": "prime::ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)",
+    }
+    for name, schema in want.items():
+        assert str(getattr(torch.ops.prime, name).default._schema) == schema
+
+
+def test_cpu_tensors_reach_no_kernel():
+    # the product has no CPU path: the dispatcher must refuse, not fall back
+    from prime_amd.C import compression as C
+
+    with pytest.raises(NotImplementedError):
+        C.uniform_8bit_quantize(torch.randn(16))
+    with pytest.raises(NotImplementedError):
+        C.quantize_per_tensor_uint8(torch.randn(16), 0.1, 128)
+    with pytest.raises(NotImplementedError):
+        C.average_buckets(torch.randn(16), torch.zeros(16, dtype=torch.uint8), 256)
+
+
+def test_fake_tensors_give_shapes():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    import prime_amd.ops  # noqa: F401
+
+    with FakeTensorMode():
+        x = torch.empty(3, 5)
+        codes, lut = torch.ops.prime.uniform_8bit_quantize(x)
+        assert codes.shape == (3, 5) and codes.dtype == torch.uint8 and lut.shape == (256,) and lut.dtype == torch.float32
+
+
+def test_ring_allreduce_rejects_other_reduce_ops():
+    # collectives.cpp:83
+    from prime_amd.C.collectives import ring_allreduce
+
+    with pytest.raises(RuntimeError, match="Only SUM and AVG"):
+        ring_allreduce(torch.zeros(8), dist.ReduceOp.MAX, None)
+
+
+def test_fake_process_group_is_a_no_op():
+    # src/zeroband/C/collectives.py:32-33
+    from torch.testing._internal.distributed.fake_pg import FakeProcessGroup
+    from prime_amd.collectives import Compression, all_reduce
+
+    pg = FakeProcessGroup.__new__(FakeProcessGroup)
+    x = torch.arange(8, dtype=torch.float32)
+    all_reduce(Compression.UINT8, x, dist.ReduceOp.SUM, pg)
+    assert torch.equal(x, torch.arange(8, dtype=torch.float32))
+
+
+def test_simulated_ring_input_checks():
+    from prime_amd.C.collectives import SimulatedRing, ring_allreduce
+
+    a, b = torch.zeros(10), torch.zeros(10)
+    with pytest.raises(ValueError, match="divisible"):
+        ring_allreduce(a, dist.ReduceOp.SUM, SimulatedRing([a, b]))      # 10 % (2*2) != 0
+    with pytest.raises(ValueError, match="not one of"):
+        ring_allreduce(torch.zeros(8), dist.ReduceOp.SUM, SimulatedRing([torch.zeros(8), torch.zeros(8)]))
+    d = a.double()
+    with pytest.raises(RuntimeError, match="Float"):
+        ring_allreduce(d, dist.ReduceOp.SUM, SimulatedRing([d]))
+
+
+def test_missing_library_is_an_error(monkeypatch, tmp_path):
+    from prime_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libprime_hip.so")
+    with pytest.raises(_lib.PrimeHipError, match="no CPU fallback"):
+        _lib.load()
