@@ -1,0 +1,276 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 pseudo-gradient compression path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one pass of the hot path over the workload of BASELINE config 2: the 22
+per-layer pseudo-gradient buckets of a 1B Llama-style model (51,380,224 fp32 elements each,
+Student-t(3) * 1e-4), each run through uniform_8bit_quantize (statistics pass, then the
+fused quantize + 256-bin lookup build).  Inputs are generated on the GPU with a seeded torch
+generator (seed = layer index) and are resident in HBM before the timed region.
+
+The single JSON line printed at the end carries
+  value          algorithmic GB/s of quantize+lookup (9 bytes per element: x read twice, codes
+                 written once) over the whole step, wall clock between two synchronisations
+  roofline       the dominant kernel (quantize + histogram, 5 bytes per element) priced against
+                 the 8 TB/s HBM peak from per-launch HIP-event times taken in a second pass over
+                 the same workload
+  ring_step      BASELINE config 3: W = 8 chunks of 2^26 elements; quantize chunk 0, then 7 hops of
+                 dequantize-add + requantize (14 bytes per element per hop)
+  tensor_2p28    uniform_8bit_quantize on one 2^28-element tensor, the size the target is quoted on
+  cpu_baseline   the reference's own compression.cpp (compiled into oracle/_ref) on this box's
+                 host cores, on a bounded sample (one bucket, a few repetitions)
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
+BUCKET_ELEMS = 4 * 2048 * 2048 + 3 * 2048 * 5632    # 51,380,224
+N_LAYERS = 22
+RING_W = 8
+RING_CHUNK = 1 << 26
+
+
+def student_t3(n, device, seed, scale):
+    """Student-t with 3 degrees of freedom: z / sqrt(chi2_3 / 3), seeded per bucket."""
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    z = torch.randn(n, device=device, generator=g)
+    chi = torch.zeros(n, device=device)
+    for _ in range(3):
+        w = torch.randn(n, device=device, generator=g)
+        chi.addcmul_(w, w)
+    z.div_(chi.div_(3.0).sqrt_()).mul_(scale)
+    return z
+
+
+def cpu_baseline(sample_elems: int, reps: int) -> dict:
+    """The reference's CPU op on this host: kind "reference" when oracle/_ref is present (the
+    reference's compression.cpp compiled unchanged), else the restatement ("port")."""
+    import numpy as np
+    import torch
+    from oracle import oracle as O
+
+    x = (np.random.default_rng(0).standard_t(3, sample_elems) * 1e-4).astype(np.float32)
+    threads = O.hardware_threads()
+    if O.ref_available():
+        R = O.ref()
+        xt = torch.from_numpy(x)
+        fn = lambda: R.uniform_8bit_quantize(xt, True)          # noqa: E731
+        kind = "reference"
+    else:
+        fn = lambda: O.uniform_8bit_quantize(x, "literal")      # noqa: E731
+        kind = "port"
+    fn()
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    return {
+        "value": round(9.0 * sample_elems / t / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": kind,
+        "sample": f"uniform_8bit_quantize on one {sample_elems}-element Student-t(3)*1e-4 bucket, median of {reps} runs "
+                  f"after one warm-up, {threads} threads (hardware_concurrency, as compression.cpp:7), "
+                  f"{os.cpu_count()} logical CPUs visible",
+        "elements_per_s": round(sample_elems / t, 1),
+        "ms_per_bucket": round(t * 1e3, 3),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the ring and 2^28 legs")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import torch
+    from prime_amd import _lib
+
+    lib = _lib.load()          # raises if libprime_hip.so is not built: there is no fallback
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    st = torch.cuda.current_stream(dev).cuda_stream
+    ws = torch.empty(int(lib.prime_workspace_bytes()), dtype=torch.uint8, device=dev)
+    _lib.check(lib.prime_workspace_init(ws.data_ptr(), ws.numel(), st), "workspace_init")
+
+    def uniform(x, codes, lut, qp):
+        _lib.check(lib.prime_uniform_8bit_quantize(x.data_ptr(), x.numel(), codes.data_ptr(), lut.data_ptr(), qp.data_ptr(),
+                                                   ws.data_ptr(), st), "uniform_8bit_quantize")
+
+    def ring_step(acc, codes_in, lut_in, codes_out, lut_out):
+        _lib.check(lib.prime_ring_reduce_step(acc.data_ptr(), codes_in.data_ptr(), lut_in.data_ptr(), acc.numel(),
+                                              codes_out.data_ptr(), lut_out.data_ptr(), None, ws.data_ptr(), st), "ring_step")
+
+    def timed(step_fn, steps, warmup):
+        for _ in range(warmup):
+            step_fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step_fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    # ---- config 2: 22 layer buckets, quantize + lookup per bucket -------------------------------
+    buckets = [student_t3(BUCKET_ELEMS, dev, layer, 1e-4) for layer in range(N_LAYERS)]
+    codes = [torch.empty(BUCKET_ELEMS, dtype=torch.uint8, device=dev) for _ in range(N_LAYERS)]
+    luts = torch.empty((N_LAYERS, 256), dtype=torch.float32, device=dev)
+    qps = torch.empty((N_LAYERS, 4), dtype=torch.float64, device=dev)
+
+    def step_buckets():
+        for i in range(N_LAYERS):
+            uniform(buckets[i], codes[i], luts[i], qps[i])
+
+    sec = timed(step_buckets, args.steps, args.warmup)
+    elems = BUCKET_ELEMS * N_LAYERS
+    value = 9.0 * elems / sec / 1e9
+
+    # second pass over the same workload with per-launch events: the roofline figures
+    _lib.profile_begin()
+    for _ in range(args.steps):
+        step_buckets()
+    prof = _lib.profile_end()
+    dom = prof["quantize_kernel+hist"]
+    dom_ms = dom["total_ms"] / dom["launches"]
+    achieved = dom["algo_bytes"] / dom["launches"] / (dom_ms * 1e-3) / 1e9
+    kernels = {k: {"avg_us": round(v["total_ms"] / v["launches"] * 1e3, 2),
+                   "algo_GBps": round(v["algo_bytes"] / (v["total_ms"] * 1e-3) / 1e9, 1) if v["total_ms"] > 0 else None,
+                   "launches": v["launches"]} for k, v in prof.items()}
+    roofline = {
+        "bound": "hbm",
+        "kernel": "quantize_kernel<aligned, hist, R=4> (quantize + 256-bin sum/count histogram)",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "algo_bytes_per_launch": 5 * BUCKET_ELEMS,
+        "avg_launch_us": round(dom_ms * 1e3, 2),
+        "kernels": kernels,
+    }
+    del buckets, codes
+    torch.cuda.empty_cache()
+
+    out = {
+        "metric": "quantize+lookup & ring-reduce-step GB/s on 1 GPU; % of HBM peak; vs CPU ops",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE config 2: 22 per-layer pseudo-gradient buckets x 51,380,224 fp32 elements, "
+                        "Student-t(3)*1e-4 (torch cuda generator, seed = layer), uniform_8bit_quantize bucket by bucket",
+            "elements_per_step": elems,
+            "algorithmic_bytes_per_element": 9,
+            "n_bins": 256,
+        },
+        "elements_per_s": round(elems / sec, 1),
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "roofline": roofline,
+    }
+
+    if not args.no_extras:
+        # ---- config 3: ring reduce-scatter hops for W = 8 ranks' chunks ---------------------------
+        chunks = []
+        for r in range(RING_W):
+            g = torch.Generator(device=dev).manual_seed(r)
+            chunks.append(torch.randn(RING_CHUNK, device=dev, generator=g) * 1e-3)
+        pristine = [c.clone() for c in chunks[1:]]
+        cbuf = [torch.empty(RING_CHUNK, dtype=torch.uint8, device=dev) for _ in range(2)]
+        lbuf = [torch.empty(256, dtype=torch.float32, device=dev) for _ in range(2)]
+        qp = torch.empty(4, dtype=torch.float64, device=dev)
+
+        def hops():
+            for r in range(1, RING_W):
+                ring_step(chunks[r], cbuf[(r - 1) % 2], lbuf[(r - 1) % 2], cbuf[r % 2], lbuf[r % 2])
+
+        def restore():
+            for c, p in zip(chunks[1:], pristine):
+                c.copy_(p)
+
+        uniform(chunks[0], cbuf[0], lbuf[0], qp)
+        ring_steps = max(2, args.steps // 2)
+        hop_sec = []
+        for it in range(args.warmup + ring_steps):
+            restore()                   # every pass starts from the ranks' own data
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            hops()
+            torch.cuda.synchronize()
+            if it >= args.warmup:
+                hop_sec.append((time.perf_counter() - t0) / (RING_W - 1))
+        hop = statistics.mean(hop_sec)
+        restore()
+        _lib.profile_begin()
+        hops()
+        rprof = _lib.profile_end()
+        ring_gbs = 14.0 * RING_CHUNK / hop / 1e9
+        out["ring_step"] = {
+            "workload": "BASELINE config 3: W=8 ranks, 2^26-element chunks N(0,1e-3) (seed = rank); per hop: "
+                        "acc += lut[codes]; uniform_8bit_quantize(acc)",
+            "value": round(ring_gbs, 1),
+            "unit": "GB/s",
+            "algorithmic_bytes_per_element": 14,
+            "ms_per_hop": round(hop * 1e3, 4),
+            "elements_per_s": round(RING_CHUNK / hop, 1),
+            "frac_of_hbm_peak": round(ring_gbs / HBM_PEAK_GBS, 4),
+            "kernels": {k: {"avg_us": round(v["total_ms"] / v["launches"] * 1e3, 2),
+                            "algo_GBps": round(v["algo_bytes"] / (v["total_ms"] * 1e-3) / 1e9, 1)} for k, v in rprof.items()},
+        }
+        del chunks, pristine, cbuf
+        torch.cuda.empty_cache()
+
+        # ---- one 2^28-element tensor ---------------------------------------------------------------
+        n28 = 1 << 28
+        g = torch.Generator(device=dev).manual_seed(0)
+        x28 = torch.randn(n28, device=dev, generator=g) * 1e-3
+        c28 = torch.empty(n28, dtype=torch.uint8, device=dev)
+        l28 = torch.empty(256, dtype=torch.float32, device=dev)
+        s28 = timed(lambda: uniform(x28, c28, l28, qp), args.steps, args.warmup)
+        gbs28 = 9.0 * n28 / s28 / 1e9
+        out["tensor_2p28"] = {
+            "workload": "uniform_8bit_quantize on one 2^28-element fp32 tensor N(0,1e-3)",
+            "value": round(gbs28, 1), "unit": "GB/s", "ms": round(s28 * 1e3, 4),
+            "elements_per_s": round(n28 / s28, 1), "frac_of_hbm_peak": round(gbs28 / HBM_PEAK_GBS, 4),
+        }
+        del x28, c28
+        torch.cuda.empty_cache()
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(BUCKET_ELEMS, reps=5)
+        out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1) if out["cpu_baseline"]["value"] else None
+
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -45,12 +45,27 @@ const char* prime_hip_last_error(void);
 int prime_hip_set_option(const char* name, int value);
 int prime_hip_get_option(const char* name, int* value);
 
-/* Workspace: a fixed-size block of ordinary device memory (hipMalloc / torch allocator;
- * not fine-grained or host memory: hardware fp64 atomics are used on it).  It holds
- * per-block partial sums, the grid-level ticket and the 256-bin accumulators.  Initialise it
- * once with prime_workspace_init (a fill kernel, safe under stream capture); every entry
- * point leaves it ready for the next call.  Two calls that share a workspace must be
- * ordered on one stream. */
+/* Per-launch timing with HIP events on the launch stream, for benchmarks: after
+ * prime_hip_profile_begin every kernel the library launches is bracketed by two events;
+ * prime_hip_profile_end waits for them and returns, per kernel, the number of launches, the
+ * summed duration and the summed algorithmic bytes (4 B/element statistics, 5 quantize,
+ * 5 / 9 dequantize set / add).  out is host memory of `capacity` entries; *count receives the
+ * number of kernels seen.  No counterpart in the reference (it times with perf_counter,
+ * src/zeroband/diloco.py:109-113). */
+typedef struct prime_kernel_time {
+    char name[40];
+    int64_t launches;
+    double total_ms;
+    double algo_bytes;
+} prime_kernel_time;
+int prime_hip_profile_begin(void);
+int prime_hip_profile_end(prime_kernel_time* out, int capacity, int* count);
+
+/* Workspace: a fixed-size block of device memory (about 8 MiB) that holds every workgroup's
+ * partial sums and partial 256-bin histogram between a kernel and its second stage.  It
+ * carries no state from one call to the next; prime_workspace_init only validates it and
+ * clears the scale record (a fill kernel, safe under stream capture).  Two calls that share a
+ * workspace must be ordered on one stream. */
 int64_t prime_workspace_bytes(void);
 int prime_workspace_init(void* ws, int64_t ws_bytes, prime_stream_t stream);
 

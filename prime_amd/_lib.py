@@ -25,6 +25,17 @@ class QParams(ctypes.Structure):
     ]
 
 
+class KernelTime(ctypes.Structure):
+    """struct prime_kernel_time."""
+
+    _fields_ = [
+        ("name", ctypes.c_char * 40),
+        ("launches", ctypes.c_int64),
+        ("total_ms", ctypes.c_double),
+        ("algo_bytes", ctypes.c_double),
+    ]
+
+
 QPARAMS_BYTES = ctypes.sizeof(QParams)
 assert QPARAMS_BYTES == 32
 
@@ -39,6 +50,8 @@ SIGNATURES = {
     "prime_hip_last_error": (ctypes.c_char_p, []),
     "prime_hip_set_option": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_int]),
     "prime_hip_get_option": (ctypes.c_int, [ctypes.c_char_p, ctypes.POINTER(ctypes.c_int)]),
+    "prime_hip_profile_begin": (ctypes.c_int, []),
+    "prime_hip_profile_end": (ctypes.c_int, [ctypes.POINTER(KernelTime), ctypes.c_int, ctypes.POINTER(ctypes.c_int)]),
     "prime_workspace_bytes": (_i64, []),
     "prime_workspace_init": (ctypes.c_int, [_vp, _i64, _vp]),
     "prime_stats_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp, _vp]),
@@ -96,3 +109,16 @@ def get_option(name: str) -> int:
     v = ctypes.c_int()
     check(load().prime_hip_get_option(name.encode(), ctypes.byref(v)), f"get_option({name})")
     return v.value
+
+
+def profile_begin() -> None:
+    check(load().prime_hip_profile_begin(), "profile_begin")
+
+
+def profile_end() -> dict:
+    """{kernel name: {"launches", "total_ms", "algo_bytes"}} since profile_begin (synchronises)."""
+    buf = (KernelTime * 32)()
+    n = ctypes.c_int()
+    check(load().prime_hip_profile_end(buf, 32, ctypes.byref(n)), "profile_end")
+    return {buf[i].name.decode(): {"launches": buf[i].launches, "total_ms": buf[i].total_ms,
+                                   "algo_bytes": buf[i].algo_bytes} for i in range(min(n.value, 32))}

@@ -16,6 +16,8 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <vector>
 
 #include "../../include/prime_hip.h"
 
@@ -597,17 +599,65 @@ int launch_check(const char* where) {
     return e == hipSuccess ? 0 : hip_fail(e, where);
 }
 
+// Optional per-launch timing with HIP events on the launch stream (prime_hip_profile_begin /
+// _end): what a benchmark reads to price each kernel against the memory roofline.  Off by
+// default; when off a launch site pays one branch.
+enum KernelId {
+    kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
+    kIdDequantAddStats, kIdBatched, kIdCopy, kIdCount
+};
+const char* const kKernelNames[kIdCount] = {
+    "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
+    "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "batched_kernel", "copy_kernel"};
+
+struct TimedLaunch {
+    int id;
+    double bytes;
+    hipEvent_t a, b;
+};
+struct Profiler {
+    bool on = false;
+    std::mutex m;
+    std::vector<TimedLaunch> launches;
+};
+Profiler g_prof;
+
+// Brackets one kernel launch: construct before it, destroy after it.
+struct LaunchTimer {
+    bool active = false;
+    TimedLaunch t{};
+    hipStream_t st;
+    LaunchTimer(int id, double algo_bytes, hipStream_t stream) : st(stream) {
+        if (!g_prof.on) return;
+        if (hipEventCreate(&t.a) != hipSuccess) return;
+        if (hipEventCreate(&t.b) != hipSuccess) { (void)hipEventDestroy(t.a); return; }
+        t.id = id;
+        t.bytes = algo_bytes;
+        active = hipEventRecord(t.a, st) == hipSuccess;
+    }
+    ~LaunchTimer() {
+        if (!active) return;
+        (void)hipEventRecord(t.b, st);
+        std::lock_guard<std::mutex> lock(g_prof.m);
+        g_prof.launches.push_back(t);
+    }
+};
+
 int run_stats_finalize(Workspace* ws, int nparts, int64_t n, prime_qparams* out, hipStream_t st) {
+    LaunchTimer timer(kIdStatsFinalize, 16.0 * nparts, st);
     hipLaunchKernelGGL(stats_finalize_kernel, dim3(1), dim3(kFinalThreads), 0, st, ws, nparts, n, out);
     return launch_check("stats_finalize_kernel");
 }
 
 int run_stats(const float* x, int64_t n, prime_qparams* out, Workspace* ws, hipStream_t st) {
     const int grid = grid_for(n);
-    if (aligned_to(x, 16))
-        hipLaunchKernelGGL(stats_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, n, ws);
-    else
-        hipLaunchKernelGGL(stats_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+    {
+        LaunchTimer timer(kIdStats, 4.0 * n, st);
+        if (aligned_to(x, 16))
+            hipLaunchKernelGGL(stats_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+        else
+            hipLaunchKernelGGL(stats_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+    }
     if (int rc = launch_check("stats_kernel")) return rc;
     return run_stats_finalize(ws, grid, n, out, st);
 }
@@ -626,6 +676,7 @@ int run_quantize(const float* x, int64_t n, float scale, const prime_qparams* qp
                  bool hist, int reverse, hipStream_t st, int* grid_out) {
     const int grid = grid_for(n);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
+    LaunchTimer timer(hist ? kIdQuantizeHist : kIdQuantize, 5.0 * n, st);
     if (!hist) {
         launch_quantize_r<false, 1>(al, grid, st, x, n, scale, qp, zp, codes, ws, reverse);
     } else {
@@ -645,6 +696,7 @@ int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins
         hipLaunchKernelGGL(lut_zero_kernel, dim3(1), dim3(kThreads), 0, st, lut, n_bins, reinterpret_cast<unsigned long long*>(counts));
         return launch_check("lut_zero_kernel");
     }
+    LaunchTimer timer(kIdLutFinalize, 16.0 * kBins * nparts, st);
     hipLaunchKernelGGL(lut_finalize_kernel, dim3(kBins / kLutBinsPerBlock), dim3(kFinalThreads), 0, st, ws, nparts, lut, n_bins,
                        reinterpret_cast<unsigned long long*>(counts));
     return launch_check("lut_finalize_kernel");
@@ -653,6 +705,7 @@ int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins
 template <bool ADD, bool STATS>
 int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out) {
     const int grid = grid_for(n);
+    LaunchTimer timer(STATS ? kIdDequantAddStats : (ADD ? kIdDequantAdd : kIdDequantSet), (ADD ? 9.0 : 5.0) * n, st);
     if (aligned_to(out, 16) && aligned_to(codes, 4))
         hipLaunchKernelGGL((dequant_kernel<ADD, STATS, true>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
     else
@@ -697,6 +750,46 @@ int prime_hip_get_option(const char* name, int* value) {
     return 0;
 }
 
+int prime_hip_profile_begin(void) {
+    std::lock_guard<std::mutex> lock(g_prof.m);
+    for (auto& t : g_prof.launches) { (void)hipEventDestroy(t.a); (void)hipEventDestroy(t.b); }
+    g_prof.launches.clear();
+    g_prof.on = true;
+    return 0;
+}
+
+int prime_hip_profile_end(prime_kernel_time* out, int capacity, int* count) {
+    if (!out || !count || capacity < 0) return fail(PRIME_EINVAL, "prime_hip_profile_end: bad argument");
+    std::lock_guard<std::mutex> lock(g_prof.m);
+    g_prof.on = false;
+    prime_kernel_time acc[kIdCount];
+    memset(acc, 0, sizeof(acc));
+    int rc = 0;
+    for (auto& t : g_prof.launches) {
+        float ms = 0.f;
+        hipError_t e = hipEventSynchronize(t.b);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, t.a, t.b);
+        if (e != hipSuccess && rc == 0) rc = hip_fail(e, "prime_hip_profile_end");
+        acc[t.id].launches += 1;
+        acc[t.id].total_ms += ms;
+        acc[t.id].algo_bytes += t.bytes;
+        (void)hipEventDestroy(t.a);
+        (void)hipEventDestroy(t.b);
+    }
+    g_prof.launches.clear();
+    int k = 0;
+    for (int id = 0; id < kIdCount; ++id) {
+        if (!acc[id].launches) continue;
+        if (k < capacity) {
+            snprintf(acc[id].name, sizeof(acc[id].name), "%s", kKernelNames[id]);
+            out[k] = acc[id];
+        }
+        ++k;
+    }
+    *count = k;
+    return rc;
+}
+
 int64_t prime_workspace_bytes(void) { return static_cast<int64_t>(sizeof(Workspace)); }
 
 int prime_workspace_init(void* ws, int64_t ws_bytes, prime_stream_t stream) {
@@ -733,6 +826,7 @@ int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64
     if (n > 0) {
         grid = grid_for(n);
         const int nb = static_cast<int>(n_bins < kBins ? n_bins : kBins);
+        LaunchTimer timer(kIdHist, 5.0 * n, st);
         if (aligned_to(x, 16) && aligned_to(codes, 4))
             hipLaunchKernelGGL((hist_kernel<true, 4>), dim3(grid), dim3(kThreads), 0, st, x, codes, n, nb, w);
         else
@@ -772,6 +866,7 @@ int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, 
     if (count < 0 || (count > 0 && (!offsets || !luts))) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: bad argument");
     if (count > 0x7fffffff) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: too many tensors");
     if (count == 0) return 0;
+    LaunchTimer timer(kIdBatched, 0.0, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(batched_kernel, dim3(static_cast<unsigned>(count)), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
                        x, offsets, codes, luts, qparams_out);
     return launch_check("batched_kernel");
@@ -814,6 +909,7 @@ int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t
     if (n_bytes == 0) return 0;
     const int64_t nvec = n_bytes >> 4;
     const int grid = grid_for(nvec * 4);
+    LaunchTimer timer(kIdCopy, 2.0 * n_bytes, static_cast<hipStream_t>(stream));
     hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<f4a*>(dst), static_cast<const f4a*>(src), nvec);
     return launch_check("copy_kernel");
