@@ -41,7 +41,9 @@ typedef struct prime_qparams {
 int prime_hip_abi_version(void);
 const char* prime_hip_last_error(void);
 
-/* Tuning knobs ("blocks_per_cu", "hist_mode", "reverse_second_pass", ...); returns 0 if known. */
+/* Tuning knobs: "blocks_per_cu" (resident workgroups per compute unit), "hist_replicas" (copies
+ * of each LDS histogram bin: 1, 2, 4, 8), "nt_load_min_mib" (tensors at least this large are
+ * read with non-temporal loads).  Returns 0 if the name is known. */
 int prime_hip_set_option(const char* name, int value);
 int prime_hip_get_option(const char* name, int* value);
 

@@ -1,7 +1,7 @@
 // libprime_hip.so - HIP kernels (gfx950 / CDNA4, wave64) and C ABI for the int8 pseudo-gradient
 // compression path: fp64 statistics, uint8 quantization, 256-bin lookup build, lookup
 // dequantization and the ring's accumulate + requantize step.  All kernels are HBM-bound
-// streams: 16-byte loads per lane, 256-thread workgroups that loop over tiles, histogram
+// streams: 16-byte loads per lane, 1024-thread workgroups that loop over tiles, histogram
 // traffic kept in LDS.  Grid-level reductions are two-stage: every workgroup stores its
 // partial result, a small second kernel adds the partials in a fixed order.
 //
@@ -17,29 +17,35 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <type_traits>
 #include <vector>
 
 #include "../../include/prime_hip.h"
 
 namespace {
 
-// Build-time tuning.
+// Build-time tuning (defaults: the best of a sweep on MI355X).
 #ifndef PRIME_UNROLL
 #define PRIME_UNROLL 4                   // 16-byte loads in flight per lane
 #endif
-#ifndef PRIME_NT_LOAD
-#define PRIME_NT_LOAD 0                  // non-temporal hint on streamed loads
+#ifndef PRIME_THREADS
+#define PRIME_THREADS 1024               // workgroup size of the streaming kernels
 #endif
-#ifndef PRIME_NT_STORE
-#define PRIME_NT_STORE 0                 // non-temporal hint on streamed stores
+#ifndef PRIME_BLOCKS_PER_CU
+#define PRIME_BLOCKS_PER_CU 2            // resident workgroups per compute unit (32 wavefronts)
 #endif
 
-constexpr int kThreads = 256;            // 4 wavefronts of 64
+constexpr int kThreads = PRIME_THREADS;   // wavefronts of 64
+constexpr int kBatchThreads = 256;       // workgroup of the one-tensor-per-workgroup kernel
 constexpr int kWaves = kThreads / 64;
 constexpr int kBins = 256;               // compression.cpp:5
 constexpr int kZeroPoint = 128;          // compression.cpp:107
 constexpr int kMaxGrid = 2048;           // per-workgroup partial slots in the workspace
 constexpr int kUnroll = PRIME_UNROLL;
+// wavefronts per SIMD the streaming kernels are compiled for (4 SIMDs per compute unit, at
+// most 8 wavefronts each): bounds their register use so that PRIME_BLOCKS_PER_CU workgroups fit
+constexpr int kWavesPerSimd = (PRIME_THREADS / 64) * PRIME_BLOCKS_PER_CU / 4 > 8 ? 8
+                              : ((PRIME_THREADS / 64) * PRIME_BLOCKS_PER_CU / 4 < 1 ? 1 : (PRIME_THREADS / 64) * PRIME_BLOCKS_PER_CU / 4);
 constexpr int kFinalThreads = 1024;      // workgroup size of the second-stage kernels
 constexpr int kLutBinsPerBlock = 4;      // bins one second-stage workgroup reduces (64 bytes per partial)
 constexpr int64_t kMaxElems = int64_t(1) << 40;   // per-workgroup counts are 32-bit
@@ -67,44 +73,31 @@ struct __attribute__((packed, aligned(4))) F4U { float x, y, z, w; };
 struct __attribute__((packed)) U32U { uint32_t v; };
 
 // Streamed accesses, 4 floats / 4 codes at vector index i.  ALIGNED means the float buffer is
-// 16-byte aligned and the code buffer 4-byte aligned.
-template <bool ALIGNED> struct Mem;
+// 16-byte aligned and the code buffer 4-byte aligned.  NT adds the non-temporal hint to loads:
+// it pays on tensors far larger than the 256 MB last-level cache and costs on smaller ones, so
+// the host picks it by size.  Write-once outputs are always stored non-temporally.
+template <bool ALIGNED, bool NT> struct Mem;
 
-template <> struct Mem<true> {
+template <bool NT> struct Mem<true, NT> {
     static __device__ __forceinline__ f4a ldf4(const float* p, int64_t i) {
         const f4a* q = reinterpret_cast<const f4a*>(p) + i;
-#if PRIME_NT_LOAD
-        return __builtin_nontemporal_load(q);
-#else
-        return *q;
-#endif
+        return NT ? __builtin_nontemporal_load(q) : *q;
     }
     static __device__ __forceinline__ void stf4(float* p, int64_t i, f4a v, bool streaming) {
         f4a* q = reinterpret_cast<f4a*>(p) + i;
-#if PRIME_NT_STORE
-        if (streaming) { __builtin_nontemporal_store(v, q); return; }
-#endif
-        *q = v;
+        if (streaming) __builtin_nontemporal_store(v, q);
+        else *q = v;
     }
     static __device__ __forceinline__ uint32_t ldu32(const uint8_t* p, int64_t i) {
         const uint32_t* q = reinterpret_cast<const uint32_t*>(p) + i;
-#if PRIME_NT_LOAD
-        return __builtin_nontemporal_load(q);
-#else
-        return *q;
-#endif
+        return NT ? __builtin_nontemporal_load(q) : *q;
     }
     static __device__ __forceinline__ void stu32(uint8_t* p, int64_t i, uint32_t v) {
-        uint32_t* q = reinterpret_cast<uint32_t*>(p) + i;
-#if PRIME_NT_STORE
-        __builtin_nontemporal_store(v, q);
-#else
-        *q = v;
-#endif
+        __builtin_nontemporal_store(v, reinterpret_cast<uint32_t*>(p) + i);
     }
 };
 
-template <> struct Mem<false> {
+template <bool NT> struct Mem<false, NT> {
     static __device__ __forceinline__ f4a ldf4(const float* p, int64_t i) {
         const F4U t = reinterpret_cast<const F4U*>(p)[i];
         return f4a{t.x, t.y, t.z, t.w};
@@ -170,17 +163,26 @@ __device__ __forceinline__ void block_stats_store(double s, double q, Workspace*
     }
 }
 
-// Second stage of the statistics: one workgroup adds the partials (tree of fixed shape) and
-// derives the scale.
-__global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace* ws, int nparts, int64_t n,
-                                                                        prime_qparams* out) {
-    __shared__ double sh_s[kFinalThreads / 64];
-    __shared__ double sh_q[kFinalThreads / 64];
-    double a = 0.0, b = 0.0;
-    for (int i = threadIdx.x; i < nparts; i += kFinalThreads) {
-        a += ws->part_sum[i];
-        b += ws->part_sq[i];
+// Second stage of the statistics run by a whole workgroup of the consuming kernel: every
+// workgroup adds the same partials in the same order, so all of them derive the same scale
+// bit for bit and no separate launch is needed.  Returns 1 / scale; workgroup 0 publishes
+// the record.
+template <int THREADS>
+__device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int nparts, int64_t n, prime_qparams* out) {
+    __shared__ double sh_s[THREADS / 64];
+    __shared__ double sh_q[THREADS / 64];
+    __shared__ float sh_inv;
+    constexpr int kIters = (kMaxGrid + THREADS - 1) / THREADS;
+    double ps[kIters], pq[kIters];
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) {       // all loads in flight at once
+        const int i = threadIdx.x + k * THREADS;
+        ps[k] = i < nparts ? ws->part_sum[i] : 0.0;
+        pq[k] = i < nparts ? ws->part_sq[i] : 0.0;
     }
+    double a = 0.0, b = 0.0;
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) { a += ps[k]; b += pq[k]; }
     a = wave_sum(a);
     b = wave_sum(b);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -189,12 +191,43 @@ __global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace
     if (threadIdx.x == 0) {
         double S = sh_s[0], Q = sh_q[0];
 #pragma unroll
-        for (int w = 1; w < kFinalThreads / 64; ++w) { S += sh_s[w]; Q += sh_q[w]; }
+        for (int w = 1; w < THREADS / 64; ++w) { S += sh_s[w]; Q += sh_q[w]; }
         prime_qparams qp;
         finalize_qparams(S, Q, n, &qp);
-        ws->qp = qp;
-        if (out) *out = qp;
+        sh_inv = qp.inv_scale;
+        if (blockIdx.x == 0) {
+            ws->qp = qp;
+            if (out) *out = qp;
+        }
     }
+    __syncthreads();
+    return sh_inv;
+}
+
+// Second stage of the statistics: one workgroup adds the partials (tree of fixed shape) and
+// derives the scale.
+__global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace* ws, int nparts, int64_t n,
+                                                                        prime_qparams* out) {
+    (void)block_scale_from_partials<kFinalThreads>(ws, nparts, n, out);
+}
+
+// Work distribution of the streaming kernels.  The tensor is cut into rows of kThreads
+// 16-byte vectors (16 KiB of floats per row at 1024 threads).  Main part: tiles of kUnroll
+// consecutive rows dealt round-robin to the G workgroups, so the whole grid sweeps the tensor
+// as one sliding window of contiguous 64 KiB pieces and every access of the main part is
+// unguarded.  Tail (fewer than G tiles): single rows dealt round-robin, so no workgroup
+// streams more than one row beyond the average.  body(i0, stride, full) handles the kUnroll
+// vectors i0 + j * stride of the calling lane; `full` is a compile-time flag (true_type in the
+// main part): unless it is set, each vector needs the check i < nvec.
+template <typename Body>
+__device__ __forceinline__ void sweep(int64_t nvec, Body&& body) {
+    const int64_t G = gridDim.x;
+    const int64_t rows = (nvec + kThreads - 1) / kThreads;
+    const int64_t rounds = (nvec / kThreads) / (G * kUnroll);
+    for (int64_t k = 0; k < rounds; ++k)
+        body(((k * G + blockIdx.x) * kUnroll) * kThreads + threadIdx.x, static_cast<int64_t>(kThreads), std::true_type{});
+    const int64_t r0 = rounds * G * kUnroll + blockIdx.x;
+    if (r0 < rows) body(r0 * kThreads + threadIdx.x, G * kThreads, std::false_type{});
 }
 
 __device__ __forceinline__ void stats_add4(const f4a v, double& s, double& q) {
@@ -206,30 +239,24 @@ __device__ __forceinline__ void stats_add4(const f4a v, double& s, double& q) {
 }
 
 // K1: sum and sum of squares in fp64.  4 bytes per element.
-template <bool ALIGNED>
-__global__ __launch_bounds__(kThreads) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
-    using M = Mem<ALIGNED>;
+template <bool ALIGNED, bool NT>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
+    using M = Mem<ALIGNED, NT>;
     const int64_t nvec = n >> 2;
-    const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    for (int64_t base = blockIdx.x * tile; base < nvec; base += static_cast<int64_t>(gridDim.x) * tile) {
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
         f4a v[kUnroll];
-        const int64_t i0 = base + threadIdx.x;
-        if (base + tile <= nvec) {
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) v[j] = M::ldf4(x, i0 + j * kThreads);
-        } else {
-#pragma unroll
-            for (int j = 0; j < kUnroll; ++j) {
-                const int64_t i = i0 + j * kThreads;
-                v[j] = i < nvec ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
-            }
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
             if (j & 1) stats_add4(v[j], s1, q1); else stats_add4(v[j], s0, q0);
         }
-    }
+    });
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const double v = x[(nvec << 2) + threadIdx.x];
         s0 += v;
@@ -264,47 +291,38 @@ __device__ __forceinline__ void hist_add(LdsHist<R>& h, int code, float x) {
 // 16-byte store per lane, 4 KiB contiguous per workgroup.
 template <int R>
 __device__ __forceinline__ void hist_store(LdsHist<R>& h, Workspace* ws) {
-    const int b = threadIdx.x;   // kThreads == kBins
-    BinAcc acc{0.0, 0ull};
+    for (int b = threadIdx.x; b < kBins; b += kThreads) {
+        BinAcc acc{0.0, 0ull};
 #pragma unroll
-    for (int r = 0; r < R; ++r) { acc.sum += h.sum[b * R + r]; acc.cnt += h.cnt[b * R + r]; }
-    ws->hist[blockIdx.x][b] = acc;
+        for (int r = 0; r < R; ++r) { acc.sum += h.sum[b * R + r]; acc.cnt += h.cnt[b * R + r]; }
+        ws->hist[blockIdx.x][b] = acc;
+    }
 }
 
 // K2 (+K3 when HIST): quantize to uint8, 4 codes packed per 32-bit store, and the 256-bin
 // sum / count histogram of the same elements.  5 bytes per element.
-template <bool ALIGNED, bool HIST, int R>
-__global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
-                                                            const prime_qparams* __restrict__ qp, int zero_point,
-                                                            uint8_t* __restrict__ codes, Workspace* ws, int reverse) {
-    using M = Mem<ALIGNED>;
+template <bool ALIGNED, bool NT, bool HIST, int R>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
+                                                            int stats_parts, prime_qparams* qp_out, int zero_point,
+                                                            uint8_t* __restrict__ codes, Workspace* ws) {
+    using M = Mem<ALIGNED, NT>;
     __shared__ LdsHist<HIST ? R : 1> hist;
-    if (HIST) {
-        hist_zero(hist);
-        __syncthreads();
-    }
-    const float inv = qp ? qp->inv_scale : 1.0f / scale_val;
+    if (HIST) hist_zero(hist);
+    // the scale: given by value, or derived here from the statistics partials of the pass before
+    const float inv = stats_parts > 0 ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out) : 1.0f / scale_val;
+    if (HIST) __syncthreads();
     const int64_t nvec = n >> 2;
-    const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
-    const int64_t ntiles = (nvec + tile - 1) / tile;
-    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        const int64_t base = (reverse ? ntiles - 1 - t : t) * tile;
-        const int64_t i0 = base + threadIdx.x;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
         f4a v[kUnroll];
-        const bool full = base + tile <= nvec;
-        if (full) {
 #pragma unroll
-            for (int j = 0; j < kUnroll; ++j) v[j] = M::ldf4(x, i0 + j * kThreads);
-        } else {
-#pragma unroll
-            for (int j = 0; j < kUnroll; ++j) {
-                const int64_t i = i0 + j * kThreads;
-                v[j] = i < nvec ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
-            }
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = i0 + j * kThreads;
+            const int64_t i = i0 + j * stride;
             if (full || i < nvec) {
                 const int a = quantize_code(v[j].x, inv, zero_point);
                 const int b = quantize_code(v[j].y, inv, zero_point);
@@ -320,7 +338,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
                 }
             }
         }
-    }
+    });
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
         const float v = x[i];
@@ -336,28 +354,28 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const float* __restr
 
 // K3 alone: histogram of x under caller-supplied codes (average_buckets).  5 bytes per element.
 template <bool ALIGNED, int R>
-__global__ __launch_bounds__(kThreads) void hist_kernel(const float* __restrict__ x, const uint8_t* __restrict__ codes,
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const float* __restrict__ x, const uint8_t* __restrict__ codes,
                                                         int64_t n, int n_bins, Workspace* ws) {
-    using M = Mem<ALIGNED>;
+    using M = Mem<ALIGNED, false>;
     __shared__ LdsHist<R> hist;
     hist_zero(hist);
     __syncthreads();
     const int64_t nvec = n >> 2;
-    const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
-    for (int64_t base = blockIdx.x * tile; base < nvec; base += static_cast<int64_t>(gridDim.x) * tile) {
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
         f4a v[kUnroll];
         uint32_t c[kUnroll];
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = base + threadIdx.x + j * kThreads;
-            const bool ok = i < nvec;
+            const int64_t i = i0 + j * stride;
+            const bool ok = full || i < nvec;
             v[j] = ok ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
-            c[j] = ok ? M::ldu32(codes, i) : 0xffffffffu;
+            c[j] = ok ? M::ldu32(codes, i) : 0u;
         }
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = base + threadIdx.x + j * kThreads;
-            if (i < nvec) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) {
                 const int a = c[j] & 255, b = (c[j] >> 8) & 255, cc = (c[j] >> 16) & 255, d = c[j] >> 24;
                 if (a < n_bins) hist_add(hist, a, v[j].x);     // compression.cpp:70
                 if (b < n_bins) hist_add(hist, b, v[j].y);
@@ -365,7 +383,7 @@ __global__ __launch_bounds__(kThreads) void hist_kernel(const float* __restrict_
                 if (d < n_bins) hist_add(hist, d, v[j].w);
             }
         }
-    }
+    });
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
         const int a = codes[i];
@@ -389,13 +407,17 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
     const int bl = threadIdx.x % kLutBinsPerBlock;
     const int row = threadIdx.x / kLutBinsPerBlock;
     const int bin = blockIdx.x * kLutBinsPerBlock + bl;
+    constexpr int kIters = kMaxGrid / kRows;
+    BinAcc part[kIters];
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) {          // all loads in flight at once
+        const int p = row + k * kRows;
+        part[k] = p < nparts ? ws->hist[p][bin] : BinAcc{0.0, 0ull};
+    }
     double s = 0.0;
     unsigned long long c = 0;
-    for (int p = row; p < nparts; p += kRows) {
-        const BinAcc a = ws->hist[p][bin];
-        s += a.sum;
-        c += a.cnt;
-    }
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) { s += part[k].sum; c += part[k].cnt; }
     sh_sum[threadIdx.x] = s;
     sh_cnt[threadIdx.x] = c;
     __syncthreads();
@@ -425,31 +447,29 @@ __global__ void lut_zero_kernel(float* __restrict__ lut, int64_t n_bins, unsigne
 // K5 / K4 pass A: out = lut[codes] (collectives.cpp:16-22) or out += lut[codes] (:8-14),
 // the lookup table held in LDS; with STATS the fp64 sum and sum of squares of the updated
 // values are taken in the same pass (the next quantization's scale).
-template <bool ADD, bool STATS, bool ALIGNED>
-__global__ __launch_bounds__(kThreads) void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut,
+template <bool ADD, bool STATS, bool ALIGNED, bool NT>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut,
                                                            const uint8_t* __restrict__ codes, int64_t n, Workspace* ws) {
-    using M = Mem<ALIGNED>;
+    using M = Mem<ALIGNED, NT>;
     __shared__ float s_lut[kBins];
-    s_lut[threadIdx.x] = lut[threadIdx.x];
+    for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
     __syncthreads();
     const int64_t nvec = n >> 2;
-    const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    for (int64_t base = blockIdx.x * tile; base < nvec; base += static_cast<int64_t>(gridDim.x) * tile) {
-        const int64_t i0 = base + threadIdx.x;
-        const bool full = base + tile <= nvec;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
         uint32_t c[kUnroll];
         f4a a[kUnroll];
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = i0 + j * kThreads;
+            const int64_t i = i0 + j * stride;
             const bool ok = full || i < nvec;
             c[j] = ok ? M::ldu32(codes, i) : 0u;
             if (ADD) a[j] = ok ? M::ldf4(out, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = i0 + j * kThreads;
+            const int64_t i = i0 + j * stride;
             f4a v;
             v.x = s_lut[c[j] & 255];
             v.y = s_lut[(c[j] >> 8) & 255];
@@ -463,7 +483,7 @@ __global__ __launch_bounds__(kThreads) void dequant_kernel(float* __restrict__ o
                 }
             }
         }
-    }
+    });
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
         float v = s_lut[codes[i]];
@@ -480,12 +500,12 @@ __global__ __launch_bounds__(kThreads) void dequant_kernel(float* __restrict__ o
 
 // Small tensors: one workgroup per tensor of a flat buffer does the whole of
 // uniform_8bit_quantize (statistics, scale, codes, lookup) without touching the workspace.
-__global__ __launch_bounds__(kThreads) void batched_kernel(const float* __restrict__ x, const int64_t* __restrict__ offsets,
+__global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __restrict__ x, const int64_t* __restrict__ offsets,
                                                            uint8_t* __restrict__ codes, float* __restrict__ luts,
                                                            prime_qparams* __restrict__ qps) {
     __shared__ LdsHist<1> hist;
-    __shared__ double sh_s[kWaves];
-    __shared__ double sh_q[kWaves];
+    __shared__ double sh_s[kBatchThreads / 64];
+    __shared__ double sh_q[kBatchThreads / 64];
     __shared__ prime_qparams sh_qp;
     const int64_t t = blockIdx.x;
     const int64_t lo = offsets[t];
@@ -493,9 +513,9 @@ __global__ __launch_bounds__(kThreads) void batched_kernel(const float* __restri
     const float* __restrict__ xp = x + lo;
     uint8_t* __restrict__ cp = codes + lo;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    hist_zero(hist);
+    for (int i = threadIdx.x; i < kBins; i += kBatchThreads) { hist.sum[i] = 0.0; hist.cnt[i] = 0u; }
     double s = 0.0, q = 0.0;
-    for (int64_t i = threadIdx.x; i < n; i += kThreads) {
+    for (int64_t i = threadIdx.x; i < n; i += kBatchThreads) {
         const double v = xp[i];
         s += v;
         q = fma(v, v, q);
@@ -507,13 +527,13 @@ __global__ __launch_bounds__(kThreads) void batched_kernel(const float* __restri
     if (threadIdx.x == 0) {
         double S = sh_s[0], Q = sh_q[0];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) { S += sh_s[w]; Q += sh_q[w]; }
+        for (int w = 1; w < kBatchThreads / 64; ++w) { S += sh_s[w]; Q += sh_q[w]; }
         finalize_qparams(S, Q, n, &sh_qp);
         if (qps) qps[t] = sh_qp;
     }
     __syncthreads();
     const float inv = sh_qp.inv_scale;
-    for (int64_t i = threadIdx.x; i < n; i += kThreads) {
+    for (int64_t i = threadIdx.x; i < n; i += kBatchThreads) {
         const float v = xp[i];
         const int c = quantize_code(v, inv, kZeroPoint);
         cp[i] = static_cast<uint8_t>(c);
@@ -530,21 +550,22 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
         p[i] = 0u;
 }
 
-__global__ __launch_bounds__(kThreads) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
-    const int64_t tile = static_cast<int64_t>(kThreads) * kUnroll;
-    for (int64_t base = blockIdx.x * tile; base < nvec; base += static_cast<int64_t>(gridDim.x) * tile) {
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
+    using M = Mem<true, false>;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
         f4a v[kUnroll];
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = base + threadIdx.x + j * kThreads;
-            if (i < nvec) v[j] = Mem<true>::ldf4(reinterpret_cast<const float*>(src), i);
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) v[j] = M::ldf4(reinterpret_cast<const float*>(src), i);
         }
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = base + threadIdx.x + j * kThreads;
-            if (i < nvec) Mem<true>::stf4(reinterpret_cast<float*>(dst), i, v[j], true);
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) M::stf4(reinterpret_cast<float*>(dst), i, v[j], true);
         }
-    }
+    });
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -563,9 +584,9 @@ int hip_fail(hipError_t e, const char* where) {
 }
 
 struct Options {
-    int blocks_per_cu = 8;
+    int blocks_per_cu = PRIME_BLOCKS_PER_CU;
+    int nt_load_min_mib = 512;      // tensors of at least this many MiB are loaded with the non-temporal hint
     int hist_replicas = 4;          // 1, 2, 4 or 8 copies of each LDS bin
-    int reverse_second_pass = 0;    // walk the quantize pass from the end of the tensor
 };
 Options g_opt;
 
@@ -581,16 +602,19 @@ int cu_count() {
     return cus[dev];
 }
 
-constexpr int64_t kTileElems = static_cast<int64_t>(kThreads) * kUnroll * 4;
+constexpr int64_t kRowElems = static_cast<int64_t>(kThreads) * 4;
 
-// Workgroups for a kernel whose workgroups each loop over tiles of kTileElems elements.
+// Workgroups for a streaming kernel: one per row of kThreads 16-byte vectors until the
+// device is full (blocks_per_cu per compute unit), then each takes a longer span.
 int grid_for(int64_t n) {
-    int64_t tiles = (n + kTileElems - 1) / kTileElems;
+    int64_t tiles = (n + kRowElems - 1) / kRowElems;
     if (tiles < 1) tiles = 1;
     int64_t cap = static_cast<int64_t>(cu_count()) * g_opt.blocks_per_cu;
     if (cap > kMaxGrid) cap = kMaxGrid;
     return static_cast<int>(tiles < cap ? tiles : cap);
 }
+
+inline bool use_nt(int64_t n) { return (n >> 18) >= g_opt.nt_load_min_mib; }   // n floats = n / 2^18 MiB
 
 inline bool aligned_to(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
@@ -649,42 +673,53 @@ int run_stats_finalize(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
     return launch_check("stats_finalize_kernel");
 }
 
-int run_stats(const float* x, int64_t n, prime_qparams* out, Workspace* ws, hipStream_t st) {
+// First stage only: returns the number of partials through *parts.
+int run_stats_partials(const float* x, int64_t n, Workspace* ws, hipStream_t st, int* parts) {
     const int grid = grid_for(n);
-    {
-        LaunchTimer timer(kIdStats, 4.0 * n, st);
-        if (aligned_to(x, 16))
-            hipLaunchKernelGGL(stats_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, n, ws);
-        else
-            hipLaunchKernelGGL(stats_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, n, ws);
-    }
-    if (int rc = launch_check("stats_kernel")) return rc;
-    return run_stats_finalize(ws, grid, n, out, st);
+    LaunchTimer timer(kIdStats, 4.0 * n, st);
+    if (!aligned_to(x, 16))
+        hipLaunchKernelGGL((stats_kernel<false, false>), dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+    else if (use_nt(n))
+        hipLaunchKernelGGL((stats_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+    else
+        hipLaunchKernelGGL((stats_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+    *parts = grid;
+    return launch_check("stats_kernel");
+}
+
+int run_stats(const float* x, int64_t n, prime_qparams* out, Workspace* ws, hipStream_t st) {
+    int parts = 0;
+    if (int rc = run_stats_partials(x, n, ws, st, &parts)) return rc;
+    return run_stats_finalize(ws, parts, n, out, st);
 }
 
 template <bool HIST, int R>
-void launch_quantize_r(bool al, int grid, hipStream_t st, const float* x, int64_t n, float scale, const prime_qparams* qp,
-                       int zp, uint8_t* codes, Workspace* ws, int reverse) {
-    if (al)
-        hipLaunchKernelGGL((quantize_kernel<true, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, qp, zp, codes, ws, reverse);
+void launch_quantize_r(bool al, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
+                       prime_qparams* qp_out, int zp, uint8_t* codes, Workspace* ws) {
+    if (!al)
+        hipLaunchKernelGGL((quantize_kernel<false, false, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    else if (use_nt(n))
+        hipLaunchKernelGGL((quantize_kernel<true, true, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     else
-        hipLaunchKernelGGL((quantize_kernel<false, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, qp, zp, codes, ws, reverse);
+        hipLaunchKernelGGL((quantize_kernel<true, false, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
 }
 
-// Returns the grid size through *grid_out: the number of histogram partials written.
-int run_quantize(const float* x, int64_t n, float scale, const prime_qparams* qp, int zp, uint8_t* codes, Workspace* ws,
-                 bool hist, int reverse, hipStream_t st, int* grid_out) {
+// stats_parts > 0: take the scale from that many statistics partials in the workspace (and
+// publish it to qp_out); otherwise use `scale`.  Returns the grid size through *grid_out: the
+// number of histogram partials written.
+int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_qparams* qp_out, int zp, uint8_t* codes,
+                 Workspace* ws, bool hist, hipStream_t st, int* grid_out) {
     const int grid = grid_for(n);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
     LaunchTimer timer(hist ? kIdQuantizeHist : kIdQuantize, 5.0 * n, st);
     if (!hist) {
-        launch_quantize_r<false, 1>(al, grid, st, x, n, scale, qp, zp, codes, ws, reverse);
+        launch_quantize_r<false, 1>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     } else {
         switch (g_opt.hist_replicas) {
-            case 1: launch_quantize_r<true, 1>(al, grid, st, x, n, scale, qp, zp, codes, ws, reverse); break;
-            case 2: launch_quantize_r<true, 2>(al, grid, st, x, n, scale, qp, zp, codes, ws, reverse); break;
-            case 8: launch_quantize_r<true, 8>(al, grid, st, x, n, scale, qp, zp, codes, ws, reverse); break;
-            default: launch_quantize_r<true, 4>(al, grid, st, x, n, scale, qp, zp, codes, ws, reverse); break;
+            case 1: launch_quantize_r<true, 1>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
+            case 2: launch_quantize_r<true, 2>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
+            case 8: launch_quantize_r<true, 8>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
+            default: launch_quantize_r<true, 4>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
         }
     }
     if (grid_out) *grid_out = grid;
@@ -706,10 +741,12 @@ template <bool ADD, bool STATS>
 int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out) {
     const int grid = grid_for(n);
     LaunchTimer timer(STATS ? kIdDequantAddStats : (ADD ? kIdDequantAdd : kIdDequantSet), (ADD ? 9.0 : 5.0) * n, st);
-    if (aligned_to(out, 16) && aligned_to(codes, 4))
-        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, true>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
+    if (!(aligned_to(out, 16) && aligned_to(codes, 4)))
+        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, false, false>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
+    else if (use_nt(n))
+        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, true, true>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
     else
-        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, false>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
+        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, true, false>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
     if (grid_out) *grid_out = grid;
     return launch_check("dequant_kernel");
 }
@@ -732,8 +769,9 @@ int prime_hip_set_option(const char* name, int value) {
     } else if (!strcmp(name, "hist_replicas")) {
         if (value != 1 && value != 2 && value != 4 && value != 8) return fail(PRIME_EINVAL, "hist_replicas must be 1, 2, 4 or 8");
         g_opt.hist_replicas = value;
-    } else if (!strcmp(name, "reverse_second_pass")) {
-        g_opt.reverse_second_pass = value ? 1 : 0;
+    } else if (!strcmp(name, "nt_load_min_mib")) {
+        if (value < 0) return fail(PRIME_EINVAL, "nt_load_min_mib must be >= 0");
+        g_opt.nt_load_min_mib = value;
     } else {
         return fail(PRIME_EINVAL, "unknown option");
     }
@@ -744,8 +782,9 @@ int prime_hip_get_option(const char* name, int* value) {
     if (!name || !value) return fail(PRIME_EINVAL, "null argument");
     if (!strcmp(name, "blocks_per_cu")) *value = g_opt.blocks_per_cu;
     else if (!strcmp(name, "hist_replicas")) *value = g_opt.hist_replicas;
-    else if (!strcmp(name, "reverse_second_pass")) *value = g_opt.reverse_second_pass;
+    else if (!strcmp(name, "nt_load_min_mib")) *value = g_opt.nt_load_min_mib;
     else if (!strcmp(name, "unroll")) *value = kUnroll;
+    else if (!strcmp(name, "threads")) *value = kThreads;
     else return fail(PRIME_EINVAL, "unknown option");
     return 0;
 }
@@ -812,7 +851,7 @@ int prime_stats_f32(const float* x, int64_t n, prime_qparams* out, void* ws, pri
 int prime_quantize_u8(const float* x, int64_t n, float scale, int32_t zero_point, uint8_t* codes, prime_stream_t stream) {
     if (bad_n(n) || (n > 0 && (!x || !codes))) return fail(PRIME_EINVAL, "prime_quantize_u8: bad argument");
     if (n == 0) return 0;
-    return run_quantize(x, n, scale, nullptr, zero_point, codes, nullptr, false, 0, static_cast<hipStream_t>(stream), nullptr);
+    return run_quantize(x, n, scale, 0, nullptr, zero_point, codes, nullptr, false, static_cast<hipStream_t>(stream), nullptr);
 }
 
 int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64_t n_bins, float* lut, uint64_t* counts,
@@ -844,7 +883,7 @@ int prime_quantize_lookup_u8(const float* x, int64_t n, float scale, uint8_t* co
     Workspace* w = static_cast<Workspace*>(ws);
     int grid = 0;
     if (n > 0)
-        if (int rc = run_quantize(x, n, scale, nullptr, kZeroPoint, codes, w, true, 0, st, &grid)) return rc;
+        if (int rc = run_quantize(x, n, scale, 0, nullptr, kZeroPoint, codes, w, true, st, &grid)) return rc;
     return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
 }
 
@@ -854,10 +893,13 @@ int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     hipStream_t st = static_cast<hipStream_t>(stream);
     Workspace* w = static_cast<Workspace*>(ws);
-    if (int rc = run_stats(x, n, qparams_out, w, st)) return rc;
-    int grid = 0;
-    if (n > 0)
-        if (int rc = run_quantize(x, n, 0.0f, &w->qp, kZeroPoint, codes, w, true, g_opt.reverse_second_pass, st, &grid)) return rc;
+    if (n == 0) {
+        if (int rc = run_stats(x, 0, qparams_out, w, st)) return rc;
+        return run_lut_finalize(w, 0, lut, kBins, nullptr, st);
+    }
+    int parts = 0, grid = 0;
+    if (int rc = run_stats_partials(x, n, w, st, &parts)) return rc;
+    if (int rc = run_quantize(x, n, 0.0f, parts, qparams_out, kZeroPoint, codes, w, true, st, &grid)) return rc;
     return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
 }
 
@@ -867,7 +909,7 @@ int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, 
     if (count > 0x7fffffff) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: too many tensors");
     if (count == 0) return 0;
     LaunchTimer timer(kIdBatched, 0.0, static_cast<hipStream_t>(stream));
-    hipLaunchKernelGGL(batched_kernel, dim3(static_cast<unsigned>(count)), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(batched_kernel, dim3(static_cast<unsigned>(count)), dim3(kBatchThreads), 0, static_cast<hipStream_t>(stream),
                        x, offsets, codes, luts, qparams_out);
     return launch_check("batched_kernel");
 }
@@ -897,8 +939,7 @@ int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut
     }
     int grid = 0;
     if (int rc = run_dequant<true, true>(acc, lut_in, codes_in, n, w, st, &grid)) return rc;
-    if (int rc = run_stats_finalize(w, grid, n, qparams_out, st)) return rc;
-    if (int rc = run_quantize(acc, n, 0.0f, &w->qp, kZeroPoint, codes_out, w, true, g_opt.reverse_second_pass, st, &grid)) return rc;
+    if (int rc = run_quantize(acc, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid)) return rc;
     return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
 }
 
