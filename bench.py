@@ -39,6 +39,11 @@ BUCKET_ELEMS = 4 * 2048 * 2048 + 3 * 2048 * 5632    # 51,380,224
 N_LAYERS = 22
 RING_W = 8
 RING_CHUNK = 1 << 26
+# HBM bytes one launch of the dominant kernel moves on a 51,380,224-element bucket, from rocprofv3
+# FETCH_SIZE / WRITE_SIZE scaled by the same counters' readings for the 1 GiB copy below
+# (profiles/cfg2_buckets_hbm_traffic.txt): 205.7 MB read + 53.5 MB written (codes + 2 MB of
+# per-workgroup histogram partials) against 256.9 MB algorithmic.
+TRAFFIC_BYTES_PER_LAUNCH = 259.18e6
 
 
 def student_t3(n, device, seed, scale):
@@ -53,6 +58,18 @@ def student_t3(n, device, seed, scale):
         chi.addcmul_(w, w)
     z.div_(chi.div_(3.0).sqrt_()).mul_(scale)
     return z
+
+
+def kernel_table(prof: dict, event_overhead_us: float) -> dict:
+    """Per-kernel average duration (event bracket minus the measured bracket overhead) and the
+    algorithmic GB/s it implies."""
+    out = {}
+    for k, v in prof.items():
+        raw = v["total_ms"] / v["launches"] * 1e3
+        us = max(raw - event_overhead_us, 1e-3)
+        out[k] = {"avg_us": round(us, 2), "avg_us_event_bracket": round(raw, 2),
+                  "algo_GBps": round(v["algo_bytes"] / v["launches"] / (us * 1e-6) / 1e9, 1)}
+    return out
 
 
 def cpu_baseline(sample_elems: int, reps: int) -> dict:
@@ -98,7 +115,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extras", action="store_true", help="skip the ring and 2^28 legs")
+    ap.add_argument("--legs", default="buckets,ring,t28",
+                    help="comma list of buckets (always run: it carries value and roofline), ring, t28")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -132,6 +150,15 @@ def main() -> int:
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
 
+    # A plain copy of known size (1 GiB read + 1 GiB written), untimed: the dispatch a profiler's
+    # FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled against.
+    yard_src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+    yard_dst = torch.empty_like(yard_src)
+    _lib.check(lib.prime_copy_bytes(yard_dst.data_ptr(), yard_src.data_ptr(), yard_src.numel() * 4, st), "copy_bytes")
+    torch.cuda.synchronize()
+    del yard_src, yard_dst
+    torch.cuda.empty_cache()
+
     # ---- config 2: 22 layer buckets, quantize + lookup per bucket -------------------------------
     buckets = [student_t3(BUCKET_ELEMS, dev, layer, 1e-4) for layer in range(N_LAYERS)]
     codes = [torch.empty(BUCKET_ELEMS, dtype=torch.uint8, device=dev) for _ in range(N_LAYERS)]
@@ -146,17 +173,29 @@ def main() -> int:
     elems = BUCKET_ELEMS * N_LAYERS
     value = 9.0 * elems / sec / 1e9
 
-    # second pass over the same workload with per-launch events: the roofline figures
+    # Second pass over the same workload with a start and a stop HIP event on every launch (on the
+    # launch stream): the roofline figures.  An event-bracketed launch cannot overlap its dispatch
+    # with the kernel before it, so each bracket reads a few microseconds long.  That overhead is
+    # measured here, not assumed: the timed region above runs the same launches back to back
+    # (a kernel trace shows no gaps between them), so (sum of bracketed durations per bucket -
+    # wall time per bucket) / launches per bucket is the overhead of one bracket.
     _lib.profile_begin()
     for _ in range(args.steps):
         step_buckets()
     prof = _lib.profile_end()
+    launches_per_bucket = sum(v["launches"] for v in prof.values()) / (args.steps * N_LAYERS)
+    bracketed_us_per_bucket = sum(v["total_ms"] for v in prof.values()) * 1e3 / (args.steps * N_LAYERS)
+    wall_us_per_bucket = sec * 1e6 / N_LAYERS
+    event_overhead_us = max(0.0, (bracketed_us_per_bucket - wall_us_per_bucket) / launches_per_bucket)
     dom = prof["quantize_kernel+hist"]
-    dom_ms = dom["total_ms"] / dom["launches"]
-    achieved = dom["algo_bytes"] / dom["launches"] / (dom_ms * 1e-3) / 1e9
-    kernels = {k: {"avg_us": round(v["total_ms"] / v["launches"] * 1e3, 2),
-                   "algo_GBps": round(v["algo_bytes"] / (v["total_ms"] * 1e-3) / 1e9, 1) if v["total_ms"] > 0 else None,
+    dom_event_us = dom["total_ms"] / dom["launches"] * 1e3
+    dom_us = dom_event_us - event_overhead_us
+    achieved = dom["algo_bytes"] / dom["launches"] / (dom_us * 1e-6) / 1e9
+    kernels = {k: {"avg_us": round(v["total_ms"] / v["launches"] * 1e3 - event_overhead_us, 2),
+                   "avg_us_event_bracket": round(v["total_ms"] / v["launches"] * 1e3, 2),
                    "launches": v["launches"]} for k, v in prof.items()}
+    for k, v in prof.items():
+        kernels[k]["algo_GBps"] = round(v["algo_bytes"] / v["launches"] / (kernels[k]["avg_us"] * 1e-6) / 1e9, 1)
     roofline = {
         "bound": "hbm",
         "kernel": "quantize_kernel<aligned, hist, R=4> (quantize + 256-bin sum/count histogram)",
@@ -164,9 +203,11 @@ def main() -> int:
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH,
         "algo_bytes_per_launch": 5 * BUCKET_ELEMS,
-        "avg_launch_us": round(dom_ms * 1e3, 2),
+        "avg_launch_us": round(dom_us, 2),
+        "avg_launch_us_event_bracket": round(dom_event_us, 2),
+        "event_overhead_us": round(event_overhead_us, 2),
         "kernels": kernels,
     }
     del buckets, codes
@@ -197,7 +238,8 @@ def main() -> int:
         "roofline": roofline,
     }
 
-    if not args.no_extras:
+    legs = set(args.legs.split(","))
+    if "ring" in legs:
         # ---- config 3: ring reduce-scatter hops for W = 8 ranks' chunks ---------------------------
         chunks = []
         for r in range(RING_W):
@@ -242,24 +284,30 @@ def main() -> int:
             "ms_per_hop": round(hop * 1e3, 4),
             "elements_per_s": round(RING_CHUNK / hop, 1),
             "frac_of_hbm_peak": round(ring_gbs / HBM_PEAK_GBS, 4),
-            "kernels": {k: {"avg_us": round(v["total_ms"] / v["launches"] * 1e3, 2),
-                            "algo_GBps": round(v["algo_bytes"] / (v["total_ms"] * 1e-3) / 1e9, 1)} for k, v in rprof.items()},
+            "kernels": kernel_table(rprof, event_overhead_us),
         }
         del chunks, pristine, cbuf
         torch.cuda.empty_cache()
 
+    if "t28" in legs:
         # ---- one 2^28-element tensor ---------------------------------------------------------------
         n28 = 1 << 28
         g = torch.Generator(device=dev).manual_seed(0)
         x28 = torch.randn(n28, device=dev, generator=g) * 1e-3
         c28 = torch.empty(n28, dtype=torch.uint8, device=dev)
         l28 = torch.empty(256, dtype=torch.float32, device=dev)
-        s28 = timed(lambda: uniform(x28, c28, l28, qp), args.steps, args.warmup)
+        qp28 = torch.empty(4, dtype=torch.float64, device=dev)
+        s28 = timed(lambda: uniform(x28, c28, l28, qp28), args.steps, args.warmup)
         gbs28 = 9.0 * n28 / s28 / 1e9
+        _lib.profile_begin()
+        for _ in range(args.steps):
+            uniform(x28, c28, l28, qp28)
+        tprof = _lib.profile_end()
         out["tensor_2p28"] = {
             "workload": "uniform_8bit_quantize on one 2^28-element fp32 tensor N(0,1e-3)",
             "value": round(gbs28, 1), "unit": "GB/s", "ms": round(s28 * 1e3, 4),
             "elements_per_s": round(n28 / s28, 1), "frac_of_hbm_peak": round(gbs28 / HBM_PEAK_GBS, 4),
+            "kernels": kernel_table(tprof, event_overhead_us),
         }
         del x28, c28
         torch.cuda.empty_cache()

@@ -11,6 +11,7 @@
 //   src/zeroband/C/csrc/compression.cpp:106-125 scale formula -> finalize_qparams()
 //   src/zeroband/C/csrc/collectives.cpp:8-22    index add/set -> dequant_kernel
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <climits>
 #include <cstdint>
@@ -628,11 +629,11 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdBatched, kIdCopy, kIdCount
+    kIdDequantAddStats, kIdBatched, kIdCopy, kIdFill, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
-    "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "batched_kernel", "copy_kernel"};
+    "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "batched_kernel", "copy_kernel", "fill_zero_kernel"};
 
 struct TimedLaunch {
     int id;
@@ -646,43 +647,41 @@ struct Profiler {
 };
 Profiler g_prof;
 
-// Brackets one kernel launch: construct before it, destroy after it.
-struct LaunchTimer {
-    bool active = false;
+// Every kernel launch of the library goes through here.  With timing on, the launch carries a
+// start and a stop event that take the dispatch's own begin and end timestamps (the same
+// interval a kernel trace reports); otherwise it is a plain launch.
+template <typename... KArgs, typename... Args>
+void launch(int id, double algo_bytes, void (*kernel)(KArgs...), int grid, int threads, hipStream_t st, Args... args) {
+    if (!g_prof.on) {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), 0, st, static_cast<KArgs>(args)...);
+        return;
+    }
     TimedLaunch t{};
-    hipStream_t st;
-    LaunchTimer(int id, double algo_bytes, hipStream_t stream) : st(stream) {
-        if (!g_prof.on) return;
-        if (hipEventCreate(&t.a) != hipSuccess) return;
-        if (hipEventCreate(&t.b) != hipSuccess) { (void)hipEventDestroy(t.a); return; }
-        t.id = id;
-        t.bytes = algo_bytes;
-        active = hipEventRecord(t.a, st) == hipSuccess;
+    t.id = id;
+    t.bytes = algo_bytes;
+    if (hipEventCreate(&t.a) != hipSuccess || hipEventCreate(&t.b) != hipSuccess) {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), 0, st, static_cast<KArgs>(args)...);
+        return;
     }
-    ~LaunchTimer() {
-        if (!active) return;
-        (void)hipEventRecord(t.b, st);
-        std::lock_guard<std::mutex> lock(g_prof.m);
-        g_prof.launches.push_back(t);
-    }
-};
+    hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(threads), 0, st, t.a, t.b, 0, static_cast<KArgs>(args)...);
+    std::lock_guard<std::mutex> lock(g_prof.m);
+    g_prof.launches.push_back(t);
+}
 
 int run_stats_finalize(Workspace* ws, int nparts, int64_t n, prime_qparams* out, hipStream_t st) {
-    LaunchTimer timer(kIdStatsFinalize, 16.0 * nparts, st);
-    hipLaunchKernelGGL(stats_finalize_kernel, dim3(1), dim3(kFinalThreads), 0, st, ws, nparts, n, out);
+    launch(kIdStatsFinalize, 16.0 * nparts, stats_finalize_kernel, 1, kFinalThreads, st, ws, nparts, n, out);
     return launch_check("stats_finalize_kernel");
 }
 
 // First stage only: returns the number of partials through *parts.
 int run_stats_partials(const float* x, int64_t n, Workspace* ws, hipStream_t st, int* parts) {
     const int grid = grid_for(n);
-    LaunchTimer timer(kIdStats, 4.0 * n, st);
     if (!aligned_to(x, 16))
-        hipLaunchKernelGGL((stats_kernel<false, false>), dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+        launch(kIdStats, 4.0 * n, stats_kernel<false, false>, grid, kThreads, st, x, n, ws);
     else if (use_nt(n))
-        hipLaunchKernelGGL((stats_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+        launch(kIdStats, 4.0 * n, stats_kernel<true, true>, grid, kThreads, st, x, n, ws);
     else
-        hipLaunchKernelGGL((stats_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, x, n, ws);
+        launch(kIdStats, 4.0 * n, stats_kernel<true, false>, grid, kThreads, st, x, n, ws);
     *parts = grid;
     return launch_check("stats_kernel");
 }
@@ -696,12 +695,13 @@ int run_stats(const float* x, int64_t n, prime_qparams* out, Workspace* ws, hipS
 template <bool HIST, int R>
 void launch_quantize_r(bool al, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
                        prime_qparams* qp_out, int zp, uint8_t* codes, Workspace* ws) {
+    const int id = HIST ? kIdQuantizeHist : kIdQuantize;
     if (!al)
-        hipLaunchKernelGGL((quantize_kernel<false, false, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+        launch(id, 5.0 * n, quantize_kernel<false, false, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     else if (use_nt(n))
-        hipLaunchKernelGGL((quantize_kernel<true, true, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+        launch(id, 5.0 * n, quantize_kernel<true, true, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     else
-        hipLaunchKernelGGL((quantize_kernel<true, false, HIST, R>), dim3(grid), dim3(kThreads), 0, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+        launch(id, 5.0 * n, quantize_kernel<true, false, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
 }
 
 // stats_parts > 0: take the scale from that many statistics partials in the workspace (and
@@ -711,7 +711,6 @@ int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_
                  Workspace* ws, bool hist, hipStream_t st, int* grid_out) {
     const int grid = grid_for(n);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
-    LaunchTimer timer(hist ? kIdQuantizeHist : kIdQuantize, 5.0 * n, st);
     if (!hist) {
         launch_quantize_r<false, 1>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     } else {
@@ -728,25 +727,25 @@ int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_
 
 int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins, uint64_t* counts, hipStream_t st) {
     if (nparts == 0) {
-        hipLaunchKernelGGL(lut_zero_kernel, dim3(1), dim3(kThreads), 0, st, lut, n_bins, reinterpret_cast<unsigned long long*>(counts));
+        launch(kIdLutFinalize, 0.0, lut_zero_kernel, 1, 256, st, lut, n_bins, reinterpret_cast<unsigned long long*>(counts));
         return launch_check("lut_zero_kernel");
     }
-    LaunchTimer timer(kIdLutFinalize, 16.0 * kBins * nparts, st);
-    hipLaunchKernelGGL(lut_finalize_kernel, dim3(kBins / kLutBinsPerBlock), dim3(kFinalThreads), 0, st, ws, nparts, lut, n_bins,
-                       reinterpret_cast<unsigned long long*>(counts));
+    launch(kIdLutFinalize, 16.0 * kBins * nparts, lut_finalize_kernel, kBins / kLutBinsPerBlock, kFinalThreads, st, ws, nparts, lut,
+           n_bins, reinterpret_cast<unsigned long long*>(counts));
     return launch_check("lut_finalize_kernel");
 }
 
 template <bool ADD, bool STATS>
 int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out) {
     const int grid = grid_for(n);
-    LaunchTimer timer(STATS ? kIdDequantAddStats : (ADD ? kIdDequantAdd : kIdDequantSet), (ADD ? 9.0 : 5.0) * n, st);
+    const int id = STATS ? kIdDequantAddStats : (ADD ? kIdDequantAdd : kIdDequantSet);
+    const double bytes = (ADD ? 9.0 : 5.0) * n;
     if (!(aligned_to(out, 16) && aligned_to(codes, 4)))
-        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, false, false>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
+        launch(id, bytes, dequant_kernel<ADD, STATS, false, false>, grid, kThreads, st, out, lut, codes, n, ws);
     else if (use_nt(n))
-        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, true, true>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
+        launch(id, bytes, dequant_kernel<ADD, STATS, true, true>, grid, kThreads, st, out, lut, codes, n, ws);
     else
-        hipLaunchKernelGGL((dequant_kernel<ADD, STATS, true, false>), dim3(grid), dim3(kThreads), 0, st, out, lut, codes, n, ws);
+        launch(id, bytes, dequant_kernel<ADD, STATS, true, false>, grid, kThreads, st, out, lut, codes, n, ws);
     if (grid_out) *grid_out = grid;
     return launch_check("dequant_kernel");
 }
@@ -837,8 +836,8 @@ int prime_workspace_init(void* ws, int64_t ws_bytes, prime_stream_t stream) {
     if (!aligned_to(ws, 16)) return fail(PRIME_EWORKSPACE, "workspace must be 16-byte aligned");
     // Only the scale record is ever read before it is written by the same call sequence;
     // clear it so that a stray read is defined.
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
-                       static_cast<uint32_t*>(ws), static_cast<int64_t>(sizeof(prime_qparams) / 4));
+    launch(kIdFill, 0.0, fill_zero_kernel, 1, 64, static_cast<hipStream_t>(stream), static_cast<uint32_t*>(ws),
+           static_cast<int64_t>(sizeof(prime_qparams) / 4));
     return launch_check("fill_zero_kernel");
 }
 
@@ -865,11 +864,10 @@ int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64
     if (n > 0) {
         grid = grid_for(n);
         const int nb = static_cast<int>(n_bins < kBins ? n_bins : kBins);
-        LaunchTimer timer(kIdHist, 5.0 * n, st);
         if (aligned_to(x, 16) && aligned_to(codes, 4))
-            hipLaunchKernelGGL((hist_kernel<true, 4>), dim3(grid), dim3(kThreads), 0, st, x, codes, n, nb, w);
+            launch(kIdHist, 5.0 * n, hist_kernel<true, 4>, grid, kThreads, st, x, codes, n, nb, w);
         else
-            hipLaunchKernelGGL((hist_kernel<false, 4>), dim3(grid), dim3(kThreads), 0, st, x, codes, n, nb, w);
+            launch(kIdHist, 5.0 * n, hist_kernel<false, 4>, grid, kThreads, st, x, codes, n, nb, w);
         if (int rc = launch_check("hist_kernel")) return rc;
     }
     return run_lut_finalize(w, grid, lut, n_bins, counts, st);
@@ -908,9 +906,8 @@ int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, 
     if (count < 0 || (count > 0 && (!offsets || !luts))) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: bad argument");
     if (count > 0x7fffffff) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: too many tensors");
     if (count == 0) return 0;
-    LaunchTimer timer(kIdBatched, 0.0, static_cast<hipStream_t>(stream));
-    hipLaunchKernelGGL(batched_kernel, dim3(static_cast<unsigned>(count)), dim3(kBatchThreads), 0, static_cast<hipStream_t>(stream),
-                       x, offsets, codes, luts, qparams_out);
+    launch(kIdBatched, 0.0, batched_kernel, static_cast<int>(count), kBatchThreads, static_cast<hipStream_t>(stream), x, offsets, codes,
+           luts, qparams_out);
     return launch_check("batched_kernel");
 }
 
@@ -950,9 +947,8 @@ int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t
     if (n_bytes == 0) return 0;
     const int64_t nvec = n_bytes >> 4;
     const int grid = grid_for(nvec * 4);
-    LaunchTimer timer(kIdCopy, 2.0 * n_bytes, static_cast<hipStream_t>(stream));
-    hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(kThreads), 0, static_cast<hipStream_t>(stream),
-                       static_cast<f4a*>(dst), static_cast<const f4a*>(src), nvec);
+    launch(kIdCopy, 2.0 * n_bytes, copy_kernel, grid, kThreads, static_cast<hipStream_t>(stream), static_cast<f4a*>(dst),
+           static_cast<const f4a*>(src), nvec);
     return launch_check("copy_kernel");
 }
 
