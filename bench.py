@@ -126,6 +126,9 @@ def main() -> int:
     from prime_amd import _lib
 
     lib = _lib.load()          # raises if libprime_hip.so is not built: there is no fallback
+    for opt in filter(None, os.environ.get("PRIME_HIP_OPTIONS", "").split(",")):   # tuning sweeps: name=value,...
+        name, val = opt.split("=")
+        _lib.set_option(name, int(val))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     st = torch.cuda.current_stream(dev).cuda_stream
@@ -198,7 +201,7 @@ def main() -> int:
         kernels[k]["algo_GBps"] = round(v["algo_bytes"] / v["launches"] / (kernels[k]["avg_us"] * 1e-6) / 1e9, 1)
     roofline = {
         "bound": "hbm",
-        "kernel": "quantize_kernel<aligned, hist, R=4> (quantize + 256-bin sum/count histogram)",
+        "kernel": "quantize_kernel<aligned, hist, R=8> (quantize + 256-bin sum/count histogram)",
         "achieved": round(achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",

@@ -587,7 +587,8 @@ int hip_fail(hipError_t e, const char* where) {
 struct Options {
     int blocks_per_cu = PRIME_BLOCKS_PER_CU;
     int nt_load_min_mib = 512;      // tensors of at least this many MiB are loaded with the non-temporal hint
-    int hist_replicas = 4;          // 1, 2, 4 or 8 copies of each LDS bin
+    int nt_second_min_mib = 0;      // the same for the quantize pass that re-reads a tensor: its last use, always hinted
+    int hist_replicas = 8;          // 1, 2, 4, 8 or 16 copies of each LDS bin
 };
 Options g_opt;
 
@@ -698,7 +699,7 @@ void launch_quantize_r(bool al, int grid, hipStream_t st, const float* x, int64_
     const int id = HIST ? kIdQuantizeHist : kIdQuantize;
     if (!al)
         launch(id, 5.0 * n, quantize_kernel<false, false, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
-    else if (use_nt(n))
+    else if (stats_parts > 0 ? (n >> 18) >= g_opt.nt_second_min_mib : use_nt(n))
         launch(id, 5.0 * n, quantize_kernel<true, true, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     else
         launch(id, 5.0 * n, quantize_kernel<true, false, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
@@ -717,8 +718,9 @@ int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_
         switch (g_opt.hist_replicas) {
             case 1: launch_quantize_r<true, 1>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
             case 2: launch_quantize_r<true, 2>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
-            case 8: launch_quantize_r<true, 8>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
-            default: launch_quantize_r<true, 4>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
+            default: launch_quantize_r<true, 8>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
+            case 16: launch_quantize_r<true, 16>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
+            case 4: launch_quantize_r<true, 4>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
         }
     }
     if (grid_out) *grid_out = grid;
@@ -766,11 +768,15 @@ int prime_hip_set_option(const char* name, int value) {
         if (value < 1 || value > 16) return fail(PRIME_EINVAL, "blocks_per_cu must be 1..16");
         g_opt.blocks_per_cu = value;
     } else if (!strcmp(name, "hist_replicas")) {
-        if (value != 1 && value != 2 && value != 4 && value != 8) return fail(PRIME_EINVAL, "hist_replicas must be 1, 2, 4 or 8");
+        if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
+            return fail(PRIME_EINVAL, "hist_replicas must be 1, 2, 4, 8 or 16");
         g_opt.hist_replicas = value;
     } else if (!strcmp(name, "nt_load_min_mib")) {
         if (value < 0) return fail(PRIME_EINVAL, "nt_load_min_mib must be >= 0");
         g_opt.nt_load_min_mib = value;
+    } else if (!strcmp(name, "nt_second_min_mib")) {
+        if (value < 0) return fail(PRIME_EINVAL, "nt_second_min_mib must be >= 0");
+        g_opt.nt_second_min_mib = value;
     } else {
         return fail(PRIME_EINVAL, "unknown option");
     }
@@ -782,6 +788,7 @@ int prime_hip_get_option(const char* name, int* value) {
     if (!strcmp(name, "blocks_per_cu")) *value = g_opt.blocks_per_cu;
     else if (!strcmp(name, "hist_replicas")) *value = g_opt.hist_replicas;
     else if (!strcmp(name, "nt_load_min_mib")) *value = g_opt.nt_load_min_mib;
+    else if (!strcmp(name, "nt_second_min_mib")) *value = g_opt.nt_second_min_mib;
     else if (!strcmp(name, "unroll")) *value = kUnroll;
     else if (!strcmp(name, "threads")) *value = kThreads;
     else return fail(PRIME_EINVAL, "unknown option");
@@ -865,9 +872,9 @@ int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64
         grid = grid_for(n);
         const int nb = static_cast<int>(n_bins < kBins ? n_bins : kBins);
         if (aligned_to(x, 16) && aligned_to(codes, 4))
-            launch(kIdHist, 5.0 * n, hist_kernel<true, 4>, grid, kThreads, st, x, codes, n, nb, w);
+            launch(kIdHist, 5.0 * n, hist_kernel<true, 8>, grid, kThreads, st, x, codes, n, nb, w);
         else
-            launch(kIdHist, 5.0 * n, hist_kernel<false, 4>, grid, kThreads, st, x, codes, n, nb, w);
+            launch(kIdHist, 5.0 * n, hist_kernel<false, 8>, grid, kThreads, st, x, codes, n, nb, w);
         if (int rc = launch_check("hist_kernel")) return rc;
     }
     return run_lut_finalize(w, grid, lut, n_bins, counts, st);
