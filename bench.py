@@ -72,9 +72,22 @@ def kernel_table(prof: dict, event_overhead_us: float) -> dict:
     return out
 
 
-def cpu_baseline(sample_elems: int, reps: int) -> dict:
-    """The reference's CPU op on this host: kind "reference" when oracle/_ref is present (the
-    reference's compression.cpp compiled unchanged), else the restatement ("port")."""
+def _median_time(fn, reps: int) -> float:
+    fn()
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return statistics.median(times)
+
+
+def cpu_baseline(sample_elems: int, ring_elems: int, reps: int) -> dict:
+    """The reference's CPU ops on this host, on a bounded sample: one config-2 bucket for
+    quantize + lookup, one config-3 chunk for the ring hop.  kind "reference" when oracle/_ref
+    is present (the reference's compression.cpp compiled unchanged), else the restatement
+    ("port").  The ring's dequantize loops exist only as a restatement (collectives.cpp does
+    not build without the gloo headers); as shipped they run on one thread."""
     import numpy as np
     import torch
     from oracle import oracle as O
@@ -84,18 +97,41 @@ def cpu_baseline(sample_elems: int, reps: int) -> dict:
     if O.ref_available():
         R = O.ref()
         xt = torch.from_numpy(x)
-        fn = lambda: R.uniform_8bit_quantize(xt, True)          # noqa: E731
+        uniform = lambda t: R.uniform_8bit_quantize(t, True)                      # noqa: E731
+        codes_t, _ = uniform(xt)
+        scale = float(O.scale_literal(x))
+        parts = {
+            "norm_ms": _median_time(lambda: xt.norm(), reps) * 1e3,                                    # compression.cpp:113
+            "quantize_ms": _median_time(lambda: R.quantize_per_tensor_uint8(xt, scale, 128), reps) * 1e3,   # :119
+            "average_buckets_ms": _median_time(lambda: R.average_buckets(xt, codes_t, 256), reps) * 1e3,    # :122
+        }
+        fn = lambda: uniform(xt)                                                  # noqa: E731
         kind = "reference"
     else:
+        uniform = None
+        codes = O.quantize_per_tensor_uint8(x, float(O.scale_literal(x)), 128)
+        parts = {
+            "norm_ms": _median_time(lambda: O.norm_literal(x), reps) * 1e3,
+            "quantize_ms": _median_time(lambda: O.quantize_per_tensor_uint8(x, 2e-5, 128), reps) * 1e3,
+            "average_buckets_ms": _median_time(lambda: O.average_buckets(x, codes), reps) * 1e3,
+        }
         fn = lambda: O.uniform_8bit_quantize(x, "literal")      # noqa: E731
         kind = "port"
-    fn()
-    times = []
-    for _ in range(reps):
-        t0 = time.perf_counter()
-        fn()
-        times.append(time.perf_counter() - t0)
-    t = statistics.median(times)
+    t = _median_time(fn, reps)
+
+    # ring hop: chunk += lut[codes] on one thread as shipped, then uniform_8bit_quantize(chunk)
+    rng = np.random.default_rng(1)
+    acc = (rng.standard_normal(ring_elems) * 1e-3).astype(np.float32)
+    rc, rl, _ = O.uniform_8bit_quantize((rng.standard_normal(ring_elems) * 1e-3).astype(np.float32), "literal")
+    t_add = _median_time(lambda: O.index_add(acc, rl, rc, 1), 3)
+    t_add_threads = _median_time(lambda: O.index_add(acc, rl, rc, threads), 3)
+    t_set = _median_time(lambda: O.index_set(acc, rl, rc, 1), 3)
+    if uniform is not None:
+        at = torch.from_numpy(acc)
+        t_q = _median_time(lambda: uniform(at), 3)
+    else:
+        t_q = _median_time(lambda: O.uniform_8bit_quantize(acc, "literal"), 3)
+    hop = t_add + t_q
     return {
         "value": round(9.0 * sample_elems / t / 1e9, 3),
         "unit": "GB/s",
@@ -106,6 +142,18 @@ def cpu_baseline(sample_elems: int, reps: int) -> dict:
                   f"{os.cpu_count()} logical CPUs visible",
         "elements_per_s": round(sample_elems / t, 1),
         "ms_per_bucket": round(t * 1e3, 3),
+        "breakdown_ms": {k: round(v, 3) for k, v in parts.items()},
+        "ring_step": {
+            "value": round(14.0 * ring_elems / hop / 1e9, 3),
+            "unit": "GB/s",
+            "kind": kind + " quantize + port index_add (1 thread, as shipped)",
+            "sample": f"one hop on a {ring_elems}-element chunk, median of 3",
+            "ms_per_hop": round(hop * 1e3, 3),
+            "index_add_1_thread_ms": round(t_add * 1e3, 3),
+            "index_add_unused_thread_variant_ms": round(t_add_threads * 1e3, 3),
+            "index_set_1_thread_ms": round(t_set * 1e3, 3),
+            "uniform_8bit_quantize_ms": round(t_q * 1e3, 3),
+        },
     }
 
 
@@ -316,7 +364,7 @@ def main() -> int:
         torch.cuda.empty_cache()
 
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(BUCKET_ELEMS, reps=5)
+        out["cpu_baseline"] = cpu_baseline(BUCKET_ELEMS, RING_CHUNK, reps=5)
         out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1) if out["cpu_baseline"]["value"] else None
 
     print(json.dumps(out))

@@ -75,3 +75,42 @@ def test_ring_reduce_step_2p26_chunks(abi):
         assert int(cnt.sum()) == n
         inside = (codes > 0) & (codes < 255)
         assert float((lut[codes.long()] - want)[inside].abs().max()) <= float(q["scale"])
+
+
+def test_config4_shard_all_42_buckets(abi):
+    # BASELINE config 4 in full: 1.25e9 elements (5 GB) as 42 buckets, the last 32 longer, N(0, 5e-4)
+    # with 0.01 % of entries at +-50 sigma; quantize + lookup + dequantize per bucket, checked through
+    # properties that hold at any size
+    base, extra, nb = 29_761_904, 32, 42
+    assert base * nb + extra == 1_250_000_000
+    g = torch.Generator(device=abi.dev).manual_seed(4)
+    sigma = 5e-4
+    for b in range(nb):
+        n = base + (extra if b == nb - 1 else 0)
+        x = torch.randn(n, device=abi.dev, generator=g) * sigma
+        k = n // 10000
+        pos = torch.randint(0, n, (k,), device=abi.dev, generator=g)
+        sign = torch.where(torch.rand(k, device=abi.dev, generator=g) < 0.5, -1.0, 1.0)
+        x[pos] = sign * (50 * sigma)
+        if b % 6 == 0:
+            announce(f"cfg4 bucket {b}")
+        codes, lut, qp = abi.uniform(x)
+        out = torch.empty_like(x)
+        abi.dequant(out, lut, codes, add=False)
+        if b % 6 and b != nb - 1:
+            continue                      # every bucket runs; a sample of them is checked in full
+        q = abi.qparams(qp)
+        sumsq = float((x.double() ** 2).sum())
+        want = np.float32(6.0 * (float(np.float32(np.sqrt(sumsq))) / np.sqrt(n - 1)) / 256.0)
+        assert abs(float(q["scale"]) - float(want)) <= 1e-6 * float(want)
+        cnt = torch.bincount(codes.int(), minlength=256)
+        assert int(cnt.sum()) == n
+        c = codes[pos]
+        assert bool(((c == 0) | (c == 255)).all())                    # outliers clip
+        assert torch.equal(out, lut[codes.long()])
+        inside = (codes > 0) & (codes < 255)
+        assert float((out - x)[inside].abs().max()) <= float(q["scale"])
+        sums = torch.zeros(256, dtype=torch.float64, device=abi.dev).index_add_(0, codes.long(), x.double())
+        mean = torch.where(cnt > 0, sums / cnt.clamp(min=1), torch.zeros_like(sums))
+        floor = torch.tensor(float(q["scale"]), device=abi.dev, dtype=torch.float64)
+        assert float(((lut.double() - mean).abs() / torch.maximum(mean.abs(), floor)).max()) <= 1e-6

@@ -358,3 +358,83 @@ def test_results_do_not_depend_on_scheduling(abi):
     c1, l1, q1 = abi.uniform(x)
     c2, l2, q2 = abi.uniform(x)
     assert torch.equal(c1, c2) and torch.equal(l1, l2) and torch.equal(q1, q2)
+
+
+def test_work_on_a_side_stream_is_ordered_and_correct(abi, oracle):
+    # kernels go to the stream the caller names, and a workspace per stream keeps calls apart
+    x = (np.random.default_rng(77).standard_normal(3_000_017) * 1e-3).astype(np.float32)
+    announce("side stream")
+    side = torch.cuda.Stream(device=abi.dev)
+    with torch.cuda.stream(side):
+        abi2 = Abi(abi.dev)                      # binds torch's current stream: the side stream
+        assert abi2.st == side.cuda_stream and abi2.st != abi.st
+        xt = abi2.to_dev(x)
+        codes, lut, qp = abi2.uniform(xt)
+        out = torch.empty_like(xt)
+        abi2.dequant(out, lut, codes, add=False)
+    side.synchronize()
+    q = abi2.qparams(qp)
+    assert q["scale"] == oracle.scale_exact(x)
+    oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
+    assert np.array_equal(codes.cpu().numpy(), oc)
+    assert np.array_equal(out.cpu().numpy(), lut.cpu().numpy()[oc])
+
+
+def test_random_sizes_offsets_and_distributions(abi, oracle):
+    # seeded sweep over what a caller can vary: length, start offset inside an allocation, data
+    rng = np.random.default_rng(2024)
+    big = torch.empty(6_000_000, dtype=torch.float32, device=abi.dev)
+    for case in range(40):
+        n = int(rng.integers(1, 5_000_000)) if case % 4 else int(rng.integers(1, 3000))
+        off = int(rng.integers(0, 9))
+        kind = case % 5
+        if kind == 0:
+            x = rng.standard_normal(n) * 10.0 ** rng.integers(-6, 3)
+        elif kind == 1:
+            x = rng.standard_t(3, n) * 1e-4
+        elif kind == 2:
+            x = rng.uniform(-1, 1, n)
+        elif kind == 3:
+            x = 1 + rng.standard_normal(n) * 1e-2
+        else:
+            x = rng.standard_normal(n) * 1e-3
+            x[rng.random(n) < 0.7] = 0.0
+        x = x.astype(np.float32)
+        announce(f"sweep case {case}: n={n} off={off} kind={kind}")
+        view = big[off:off + n]
+        view.copy_(abi.to_dev(x))
+        codes, lut, qp = abi.uniform(view)
+        q = abi.qparams(qp)
+        want = oracle.scale_exact(x)
+        assert np.array_equal(np.array([q["scale"]]), np.array([want]), equal_nan=True), case
+        oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
+        gc = codes.cpu().numpy()
+        assert np.array_equal(gc, oc), case
+        mean, _ = oracle.average_buckets_f64(x, oc)
+        floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+        assert lut_rel_err(lut.cpu().numpy(), mean, floor) <= LUT_TOL, case
+        # accumulate back onto the same misaligned view: one ring hop's first half
+        abi.dequant(view, lut, codes, add=True)
+        ref = x.copy()
+        oracle.index_add(ref, lut.cpu().numpy(), oc)
+        assert np.array_equal(view.cpu().numpy(), ref), case
+
+
+def test_layer_buckets_as_views_of_one_flat_buffer(abi, oracle):
+    # the caller's layout (src/zeroband/diloco.py:147-201): one flat fp32 buffer, one view per layer
+    # bucket; bucket sizes need not be multiples of four, so most views start misaligned
+    rng = np.random.default_rng(31)
+    sizes = [1_000_003, 512 * 1024, 777_777, 2_000_001, 65_537]
+    flat = (rng.standard_t(3, sum(sizes)) * 1e-4).astype(np.float32)
+    ft = abi.to_dev(flat)
+    lo = 0
+    for i, n in enumerate(sizes):
+        announce(f"flat-buffer bucket {i} n={n} start={lo}")
+        codes, lut, qp = abi.uniform(ft[lo:lo + n])
+        q = abi.qparams(qp)
+        x = flat[lo:lo + n]
+        assert q["scale"] == oracle.scale_exact(x)
+        oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
+        assert np.array_equal(codes.cpu().numpy(), oc)
+        lo += n
+    assert np.array_equal(ft.cpu().numpy(), flat)          # inputs are never modified
