@@ -124,6 +124,14 @@ int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut
                            uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out,
                            void* ws, prime_stream_t stream);
 
+/* One hop of the ring's all-gather as ring_allreduce runs it, collectives.cpp:200-215:
+ * chunk[i] = lut_in[codes_in[i]] (fast_index_set_omp), then (codes_out, lut_out) =
+ * uniform_8bit_quantize(chunk) for forwarding.  The statistics are taken while the chunk is
+ * written, so it is written once and read once. */
+int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_t n,
+                           uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out,
+                           void* ws, prime_stream_t stream);
+
 /* A plain device copy of n bytes (16-byte vectors): the yardstick the profiler's byte
  * counters are scaled against.  No counterpart in the reference. */
 int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t stream);

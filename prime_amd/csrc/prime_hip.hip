@@ -630,11 +630,12 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdBatched, kIdCopy, kIdFill, kIdCount
+    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
-    "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "batched_kernel", "copy_kernel", "fill_zero_kernel"};
+    "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
+    "batched_kernel", "copy_kernel", "fill_zero_kernel"};
 
 struct TimedLaunch {
     int id;
@@ -740,7 +741,7 @@ int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins
 template <bool ADD, bool STATS>
 int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out) {
     const int grid = grid_for(n);
-    const int id = STATS ? kIdDequantAddStats : (ADD ? kIdDequantAdd : kIdDequantSet);
+    const int id = STATS ? (ADD ? kIdDequantAddStats : kIdDequantSetStats) : (ADD ? kIdDequantAdd : kIdDequantSet);
     const double bytes = (ADD ? 9.0 : 5.0) * n;
     if (!(aligned_to(out, 16) && aligned_to(codes, 4)))
         launch(id, bytes, dequant_kernel<ADD, STATS, false, false>, grid, kThreads, st, out, lut, codes, n, ws);
@@ -930,21 +931,43 @@ int prime_dequant_add(float* out, const float* lut, const uint8_t* codes, int64_
     return run_dequant<true, false>(out, lut, codes, n, nullptr, static_cast<hipStream_t>(stream), nullptr);
 }
 
-int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out,
-                           float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
-    if (bad_n(n) || (n > 0 && (!acc || !codes_in || !codes_out)) || !lut_in || !lut_out)
-        return fail(PRIME_EINVAL, "prime_ring_reduce_step: bad argument");
+}  // extern "C"
+
+namespace {
+
+// One received message of the ring: chunk (+)= lut_in[codes_in] with the statistics of the
+// result taken in the same pass, then the requantization of the chunk.
+template <bool ADD>
+int ring_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out, float* lut_out,
+              prime_qparams* qparams_out, void* ws, prime_stream_t stream, const char* who) {
+    if (bad_n(n) || (n > 0 && (!chunk || !codes_in || !codes_out)) || !lut_in || !lut_out) return fail(PRIME_EINVAL, who);
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     hipStream_t st = static_cast<hipStream_t>(stream);
     Workspace* w = static_cast<Workspace*>(ws);
     if (n == 0) {
-        if (int rc = run_stats(acc, 0, qparams_out, w, st)) return rc;
+        if (int rc = run_stats(chunk, 0, qparams_out, w, st)) return rc;
         return run_lut_finalize(w, 0, lut_out, kBins, nullptr, st);
     }
     int grid = 0;
-    if (int rc = run_dequant<true, true>(acc, lut_in, codes_in, n, w, st, &grid)) return rc;
-    if (int rc = run_quantize(acc, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid)) return rc;
+    if (int rc = run_dequant<ADD, true>(chunk, lut_in, codes_in, n, w, st, &grid)) return rc;
+    if (int rc = run_quantize(chunk, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid)) return rc;
     return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
+}
+
+}  // namespace
+
+extern "C" {
+
+int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out,
+                           float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
+    return ring_step<true>(acc, codes_in, lut_in, n, codes_out, lut_out, qparams_out, ws, stream,
+                           "prime_ring_reduce_step: bad argument");
+}
+
+int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out,
+                           float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
+    return ring_step<false>(chunk, codes_in, lut_in, n, codes_out, lut_out, qparams_out, ws, stream,
+                            "prime_ring_gather_step: bad argument");
 }
 
 int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t stream) {

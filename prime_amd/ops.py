@@ -10,6 +10,7 @@ Schemas mirror the Python signatures of the reference's wrappers
     prime::dequantize(Tensor codes, Tensor lut) -> Tensor
     prime::dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()
     prime::ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
+    prime::ring_gather_step(Tensor(a!) chunk, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
     prime::uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)
     prime::uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)
 
@@ -37,6 +38,7 @@ _LIB.define("quantize_per_tensor_uint8(Tensor tensor, float scale, int zero_poin
 _LIB.define("dequantize(Tensor codes, Tensor lut) -> Tensor")
 _LIB.define("dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()")
 _LIB.define("ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
+_LIB.define("ring_gather_step(Tensor(a!) chunk, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
 _LIB.define("uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)")
 _LIB.define("uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)")
 
@@ -161,13 +163,21 @@ def _dequantize_(out: torch.Tensor, codes: torch.Tensor, lut: torch.Tensor, accu
 
 
 def _ring_reduce_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor):
-    _need_f32(acc, "ring_reduce_step")
-    _need_u8(codes_in, "ring_reduce_step")
-    lut_in = _need_lut(lut_in, "ring_reduce_step")
+    return _ring_step(acc, codes_in, lut_in, "ring_reduce_step")
+
+
+def _ring_gather_step(chunk: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor):
+    return _ring_step(chunk, codes_in, lut_in, "ring_gather_step")
+
+
+def _ring_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, which: str):
+    _need_f32(acc, which)
+    _need_u8(codes_in, which)
+    lut_in = _need_lut(lut_in, which)
     if not acc.is_contiguous():
-        raise RuntimeError("ring_reduce_step: acc must be contiguous (it is updated in place)")
+        raise RuntimeError(f"{which}: the chunk must be contiguous (it is updated in place)")
     if acc.numel() != codes_in.numel():
-        raise RuntimeError("ring_reduce_step: acc and codes_in differ in numel")
+        raise RuntimeError(f"{which}: chunk and codes_in differ in numel")
     lib = _lib.load()
     c = codes_in.contiguous()
     dev = acc.device
@@ -175,10 +185,9 @@ def _ring_reduce_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.T
         codes = torch.empty(acc.shape, dtype=torch.uint8, device=dev)
         lut = torch.empty(N_BINS, dtype=torch.float32, device=dev)
         ws = workspace(dev)
-        _lib.check(
-            lib.prime_ring_reduce_step(acc.data_ptr(), c.data_ptr(), lut_in.data_ptr(), acc.numel(), codes.data_ptr(),
-                                       lut.data_ptr(), None, ws.data_ptr(), _stream(dev)),
-            "prime_ring_reduce_step")
+        fn = lib.prime_ring_reduce_step if which == "ring_reduce_step" else lib.prime_ring_gather_step
+        _lib.check(fn(acc.data_ptr(), c.data_ptr(), lut_in.data_ptr(), acc.numel(), codes.data_ptr(), lut.data_ptr(), None,
+                      ws.data_ptr(), _stream(dev)), f"prime_{which}")
     return codes, lut
 
 
@@ -211,6 +220,7 @@ _LIB.impl("quantize_per_tensor_uint8", _quantize_per_tensor_uint8, "CUDA")
 _LIB.impl("dequantize", _dequantize, "CUDA")
 _LIB.impl("dequantize_", _dequantize_, "CUDA")
 _LIB.impl("ring_reduce_step", _ring_reduce_step, "CUDA")
+_LIB.impl("ring_gather_step", _ring_gather_step, "CUDA")
 _LIB.impl("uniform_8bit_quantize_stats", _uniform_8bit_quantize_stats, "CUDA")
 _LIB.impl("uniform_8bit_quantize_batched", _uniform_8bit_quantize_batched, "CUDA")
 
@@ -241,6 +251,11 @@ def _(acc, codes_in, lut_in):
     return acc.new_empty(acc.shape, dtype=torch.uint8), acc.new_empty(N_BINS, dtype=torch.float32)
 
 
+@torch.library.register_fake("prime::ring_gather_step")
+def _(chunk, codes_in, lut_in):
+    return chunk.new_empty(chunk.shape, dtype=torch.uint8), chunk.new_empty(N_BINS, dtype=torch.float32)
+
+
 def unpack_qparams(qp: torch.Tensor) -> dict:
     """Host view of one ``prime_qparams`` record (synchronises)."""
     raw = qp.detach().cpu().contiguous().view(torch.uint8).numpy().tobytes()
@@ -254,5 +269,6 @@ quantize_per_tensor_uint8 = torch.ops.prime.quantize_per_tensor_uint8
 dequantize = torch.ops.prime.dequantize
 dequantize_ = torch.ops.prime.dequantize_
 ring_reduce_step = torch.ops.prime.ring_reduce_step
+ring_gather_step = torch.ops.prime.ring_gather_step
 uniform_8bit_quantize_stats = torch.ops.prime.uniform_8bit_quantize_stats
 uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched

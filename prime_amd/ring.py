@@ -76,8 +76,11 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False)
                 ch = chunk(r, c)
                 msg = inbox[r].pop(step - BUFFER_COUNT, None)
                 sending = step <= (W - 1) * BUFFER_COUNT                    # :136 / :212
-                if msg is not None and phase == 1 and sending:
-                    codes, lut = ops.ring_reduce_step(ch, msg[0], msg[1])   # :128-138 fused
+                if msg is not None and sending:
+                    if phase == 1:
+                        codes, lut = ops.ring_reduce_step(ch, msg[0], msg[1])   # :128-138 fused
+                    else:
+                        codes, lut = ops.ring_gather_step(ch, msg[0], msg[1])   # :204-215 fused
                     posted.append(((r + 1) % W, step, codes, lut))
                     continue
                 if msg is not None:

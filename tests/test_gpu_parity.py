@@ -438,3 +438,78 @@ def test_layer_buckets_as_views_of_one_flat_buffer(abi, oracle):
         assert np.array_equal(codes.cpu().numpy(), oc)
         lo += n
     assert np.array_equal(ft.cpu().numpy(), flat)          # inputs are never modified
+
+
+@pytest.mark.parametrize("n", [1, 4097, 1 << 20, 3_000_001])
+def test_ring_gather_step_is_set_then_requantize(abi, oracle, n):
+    # all-gather hop (collectives.cpp:204-215): chunk = lut[codes], then uniform_8bit_quantize(chunk)
+    rng = np.random.default_rng(n)
+    src = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    announce(f"gather step n={n}")
+    codes_in, lut_in, _ = abi.uniform(abi.to_dev(src))
+    chunk = abi.to_dev(rng.standard_normal(n).astype(np.float32))          # overwritten entirely
+    codes, lut, qp = abi.ring_step(chunk, codes_in, lut_in, gather=True)
+    torch.cuda.synchronize()
+    ci, li = codes_in.cpu().numpy(), lut_in.cpu().numpy()
+    want = np.empty(n, np.float32)
+    oracle.index_set(want, li, ci)
+    assert np.array_equal(chunk.cpu().numpy(), want)
+    q = abi.qparams(qp)
+    assert np.array_equal(np.array([q["scale"]]), np.array([oracle.scale_exact(want)]), equal_nan=True)
+    oc, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q["scale"]))
+    assert np.array_equal(codes.cpu().numpy(), oc)
+    mean, _ = oracle.average_buckets_f64(want, oc)
+    floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+    assert lut_rel_err(lut.cpu().numpy(), mean, floor) <= LUT_TOL
+
+
+def test_entry_points_replay_from_a_hip_graph(abi, oracle):
+    # nothing in the library allocates, synchronises or records a memset: a sequence of calls can be
+    # captured once and replayed; every replay must reproduce the eager result on fresh inputs
+    sizes = [70_001, 1 << 16, 300_000, 4099]
+    rng = np.random.default_rng(404)
+    xs = [torch.empty(n, dtype=torch.float32, device=abi.dev) for n in sizes]
+    accs = [torch.empty(n, dtype=torch.float32, device=abi.dev) for n in sizes]
+    side = torch.cuda.Stream(device=abi.dev)
+    with torch.cuda.stream(side):
+        g_abi = Abi(abi.dev)                      # workspace bound to the capture stream
+        outs = []
+
+        def sequence():
+            res = []
+            for x, acc in zip(xs, accs):
+                c, l, qp = g_abi.uniform(x)
+                c2, l2, qp2 = g_abi.ring_step(acc, c, l)
+                res.append((c, l, qp, c2, l2, qp2))
+            return res
+
+        for x, acc in zip(xs, accs):
+            x.normal_()
+            acc.normal_()
+        sequence()                                # warm-up outside capture
+        side.synchronize()
+        announce("graph capture")
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            outs = sequence()
+    for replay in range(3):
+        hx = [(rng.standard_normal(n) * 10.0 ** (-replay)).astype(np.float32) for n in sizes]
+        ha = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+        for x, acc, a, b in zip(xs, accs, hx, ha):
+            x.copy_(abi.to_dev(a))
+            acc.copy_(abi.to_dev(b))
+        torch.cuda.synchronize()
+        announce(f"graph replay {replay}")
+        graph.replay()
+        torch.cuda.synchronize()
+        for (c, l, qp, c2, l2, qp2), a, b, acc in zip(outs, hx, ha, accs):
+            q = abi.qparams(qp)
+            assert q["scale"] == oracle.scale_exact(a)
+            oc, _, _ = oracle.uniform_8bit_quantize(a, "given", scale=float(q["scale"]))
+            assert np.array_equal(c.cpu().numpy(), oc)
+            want = b.copy()
+            oracle.index_add(want, l.cpu().numpy(), oc)
+            assert np.array_equal(acc.cpu().numpy(), want)
+            q2 = abi.qparams(qp2)
+            oc2, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q2["scale"]))
+            assert q2["scale"] == oracle.scale_exact(want) and np.array_equal(c2.cpu().numpy(), oc2)
