@@ -37,7 +37,7 @@ namespace {
 #endif
 
 constexpr int kThreads = PRIME_THREADS;   // wavefronts of 64
-constexpr int kBatchThreads = 256;       // workgroup of the one-tensor-per-workgroup kernel
+constexpr int kBatchThreads = 512;       // workgroup of the one-tensor-per-workgroup kernel
 constexpr int kWaves = kThreads / 64;
 constexpr int kBins = 256;               // compression.cpp:5
 constexpr int kZeroPoint = 128;          // compression.cpp:107
@@ -501,28 +501,56 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float*
 
 // Small tensors: one workgroup per tensor of a flat buffer does the whole of
 // uniform_8bit_quantize (statistics, scale, codes, lookup) without touching the workspace.
+// With VEC (flat buffer 16-byte aligned, code buffer 4-byte aligned) the part of the tensor
+// between its first and last multiple-of-4 global index is read as 16-byte vectors and its
+// codes stored 4 at a time; the ragged ends, which share vectors with the neighbouring
+// tensors, go element by element.  The second read of a tensor comes from L2.
+template <bool VEC>
 __global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __restrict__ x, const int64_t* __restrict__ offsets,
-                                                           uint8_t* __restrict__ codes, float* __restrict__ luts,
-                                                           prime_qparams* __restrict__ qps) {
-    __shared__ LdsHist<1> hist;
+                                                                uint8_t* __restrict__ codes, float* __restrict__ luts,
+                                                                prime_qparams* __restrict__ qps) {
+    constexpr int R = 4;
+    __shared__ LdsHist<R> hist;
     __shared__ double sh_s[kBatchThreads / 64];
     __shared__ double sh_q[kBatchThreads / 64];
     __shared__ prime_qparams sh_qp;
     const int64_t t = blockIdx.x;
     const int64_t lo = offsets[t];
-    const int64_t n = offsets[t + 1] - lo;
-    const float* __restrict__ xp = x + lo;
-    uint8_t* __restrict__ cp = codes + lo;
+    const int64_t hi = offsets[t + 1];
+    const int64_t n = hi - lo;
+    // [lo, a) and [b, hi) element by element, [a, b) as vectors
+    int64_t a = VEC ? (lo + 3) & ~int64_t(3) : hi;
+    int64_t b = VEC ? hi & ~int64_t(3) : hi;
+    if (a > b) { a = hi; b = hi; }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int i = threadIdx.x; i < kBins; i += kBatchThreads) { hist.sum[i] = 0.0; hist.cnt[i] = 0u; }
-    double s = 0.0, q = 0.0;
-    for (int64_t i = threadIdx.x; i < n; i += kBatchThreads) {
-        const double v = xp[i];
-        s += v;
-        q = fma(v, v, q);
+    for (int i = threadIdx.x; i < kBins * R; i += kBatchThreads) { hist.sum[i] = 0.0; hist.cnt[i] = 0u; }
+    double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
+    const f4a* __restrict__ x4 = reinterpret_cast<const f4a*>(x);
+    constexpr int U = 4;
+    for (int64_t v0 = (a >> 2) + threadIdx.x; v0 < (b >> 2); v0 += kBatchThreads * U) {
+        f4a v[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = v0 + j * kBatchThreads;
+            v[j] = i < (b >> 2) ? x4[i] : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if (j & 1) stats_add4(v[j], s1, q1); else stats_add4(v[j], s0, q0);
+        }
     }
-    s = wave_sum(s);
-    q = wave_sum(q);
+    for (int64_t i = lo + threadIdx.x; i < a; i += kBatchThreads) {        // ragged head (everything without VEC)
+        const double v = x[i];
+        s0 += v;
+        q0 = fma(v, v, q0);
+    }
+    for (int64_t i = b + threadIdx.x; i < hi; i += kBatchThreads) {        // ragged tail
+        const double v = x[i];
+        s1 += v;
+        q1 = fma(v, v, q1);
+    }
+    double s = wave_sum(s0 + s1);
+    double q = wave_sum(q0 + q1);
     if (lane == 0) { sh_s[wave] = s; sh_q[wave] = q; }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -534,15 +562,48 @@ __global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __r
     }
     __syncthreads();
     const float inv = sh_qp.inv_scale;
-    for (int64_t i = threadIdx.x; i < n; i += kBatchThreads) {
-        const float v = xp[i];
-        const int c = quantize_code(v, inv, kZeroPoint);
-        cp[i] = static_cast<uint8_t>(c);
-        hist_add(hist, c, v);
+    uint32_t* __restrict__ c4 = reinterpret_cast<uint32_t*>(codes);
+    for (int64_t v0 = (a >> 2) + threadIdx.x; v0 < (b >> 2); v0 += kBatchThreads * U) {
+        f4a v[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = v0 + j * kBatchThreads;
+            v[j] = i < (b >> 2) ? x4[i] : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = v0 + j * kBatchThreads;
+            if (i < (b >> 2)) {
+                const int ca = quantize_code(v[j].x, inv, kZeroPoint);
+                const int cb = quantize_code(v[j].y, inv, kZeroPoint);
+                const int cc = quantize_code(v[j].z, inv, kZeroPoint);
+                const int cd = quantize_code(v[j].w, inv, kZeroPoint);
+                c4[i] = static_cast<uint32_t>(ca) | (static_cast<uint32_t>(cb) << 8) | (static_cast<uint32_t>(cc) << 16) |
+                        (static_cast<uint32_t>(cd) << 24);
+                hist_add(hist, ca, v[j].x);
+                hist_add(hist, cb, v[j].y);
+                hist_add(hist, cc, v[j].z);
+                hist_add(hist, cd, v[j].w);
+            }
+        }
+    }
+    for (int part = 0; part < 2; ++part) {
+        const int64_t from = part ? b : lo, to = part ? hi : a;
+        for (int64_t i = from + threadIdx.x; i < to; i += kBatchThreads) {
+            const float v = x[i];
+            const int c = quantize_code(v, inv, kZeroPoint);
+            codes[i] = static_cast<uint8_t>(c);
+            hist_add(hist, c, v);
+        }
     }
     __syncthreads();
-    const unsigned c = hist.cnt[threadIdx.x];
-    luts[t * kBins + threadIdx.x] = c ? static_cast<float>(hist.sum[threadIdx.x] / static_cast<double>(c)) : 0.0f;
+    for (int bin = threadIdx.x; bin < kBins; bin += kBatchThreads) {
+        double sum = 0.0;
+        unsigned long long cnt = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) { sum += hist.sum[bin * R + r]; cnt += hist.cnt[bin * R + r]; }
+        luts[t * kBins + bin] = cnt ? static_cast<float>(sum / static_cast<double>(cnt)) : 0.0f;
+    }
 }
 
 __global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
@@ -914,8 +975,12 @@ int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, 
     if (count < 0 || (count > 0 && (!offsets || !luts))) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: bad argument");
     if (count > 0x7fffffff) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: too many tensors");
     if (count == 0) return 0;
-    launch(kIdBatched, 0.0, batched_kernel, static_cast<int>(count), kBatchThreads, static_cast<hipStream_t>(stream), x, offsets, codes,
-           luts, qparams_out);
+    if (aligned_to(x, 16) && aligned_to(codes, 4))
+        launch(kIdBatched, 0.0, batched_kernel<true>, static_cast<int>(count), kBatchThreads, static_cast<hipStream_t>(stream), x,
+               offsets, codes, luts, qparams_out);
+    else
+        launch(kIdBatched, 0.0, batched_kernel<false>, static_cast<int>(count), kBatchThreads, static_cast<hipStream_t>(stream), x,
+               offsets, codes, luts, qparams_out);
     return launch_check("batched_kernel");
 }
 

@@ -513,3 +513,37 @@ def test_entry_points_replay_from_a_hip_graph(abi, oracle):
             q2 = abi.qparams(qp2)
             oc2, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q2["scale"]))
             assert q2["scale"] == oracle.scale_exact(want) and np.array_equal(c2.cpu().numpy(), oc2)
+
+
+@pytest.mark.parametrize("shift", [0, 1, 3])
+def test_batched_entry_point_with_ragged_tensors_and_misaligned_base(abi, oracle, shift):
+    # tensors of every small length packed back to back, so each starts at a different alignment;
+    # shift > 0 also misaligns the flat buffer itself (the element-wise variant of the kernel)
+    rng = np.random.default_rng(90 + shift)
+    sizes = np.concatenate([np.arange(1, 40), rng.integers(1, 5000, 60), [65536, 4096, 1]])
+    off = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    flat = (rng.standard_normal(off[-1]) * 1e-3).astype(np.float32)
+    announce(f"batched shift={shift} count={len(sizes)}")
+    base = torch.zeros(off[-1] + 8, dtype=torch.float32, device=abi.dev)
+    ft = base[shift:shift + off[-1]]
+    ft.copy_(abi.to_dev(flat))
+    cbase = torch.zeros(off[-1] + 8, dtype=torch.uint8, device=abi.dev)
+    count = len(sizes)
+    luts = torch.empty((count, 256), dtype=torch.float32, device=abi.dev)
+    qps = torch.empty((count, 4), dtype=torch.float64, device=abi.dev)
+    from prime_amd import _lib as L
+    L.check(abi.lib.prime_uniform_8bit_quantize_batched(ft.data_ptr(), abi.to_dev(off).data_ptr(), count,
+                                                        cbase.data_ptr() + shift, luts.data_ptr(), qps.data_ptr(), abi.st), "batched")
+    torch.cuda.synchronize()
+    gc = cbase[shift:shift + off[-1]].cpu().numpy()
+    gl = luts.cpu().numpy()
+    for t in range(count):
+        xs = flat[off[t]:off[t + 1]]
+        q = abi.qparams(qps[t].cpu())
+        assert np.array_equal(np.array([q["scale"]]), np.array([oracle.scale_exact(xs)]), equal_nan=True), (t, xs.size)
+        oc, _, _ = oracle.uniform_8bit_quantize(xs, "given", scale=float(q["scale"]))
+        assert np.array_equal(gc[off[t]:off[t + 1]], oc), (t, xs.size)
+        mean, _ = oracle.average_buckets_f64(xs, oc)
+        floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+        assert lut_rel_err(gl[t], mean, floor) <= LUT_TOL, (t, xs.size)
+    assert not cbase[:shift].cpu().numpy().any() and not cbase[shift + off[-1]:].cpu().numpy().any()
