@@ -99,6 +99,18 @@ int prime_quantize_lookup_u8(const float* x, int64_t n, float scale, uint8_t* co
 int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float* lut,
                                 prime_qparams* qparams_out, void* ws, prime_stream_t stream);
 
+/* Large buckets, pipelined: bucket i is quantized as prime_uniform_8bit_quantize would, on
+ * streams[i % n_streams] with workspaces[i % n_streams], so that the statistics pass of one
+ * bucket overlaps the quantize pass and the launch ramps of its neighbours (three streams
+ * give +18 % on 205 MB buckets).  This is the loop over per-layer buckets of
+ * Diloco.sync_pseudo_gradient (src/zeroband/diloco.py:108-110) without the network in between.
+ * xs, ns, codes, workspaces and streams are host arrays; luts is count x 256 on the device and
+ * qparams_out (optional) count records.  The caller orders the streams against its own work. */
+int prime_uniform_8bit_quantize_buckets(const float* const* xs, const int64_t* ns, int64_t count,
+                                        uint8_t* const* codes, float* luts, prime_qparams* qparams_out,
+                                        void* const* workspaces, const prime_stream_t* streams,
+                                        int n_streams);
+
 /* Many tensors in one launch: tensor t is x[offsets[t] .. offsets[t+1]) of a flat buffer, the
  * layout of the per-layer views of Diloco's flat pseudo-gradient buffer
  * (src/zeroband/diloco.py:147-201), each handled as uniform_8bit_quantize handles one tensor.

@@ -970,6 +970,22 @@ int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float
     return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
 }
 
+int prime_uniform_8bit_quantize_buckets(const float* const* xs, const int64_t* ns, int64_t count, uint8_t* const* codes,
+                                        float* luts, prime_qparams* qparams_out, void* const* workspaces,
+                                        const prime_stream_t* streams, int n_streams) {
+    if (count < 0 || n_streams < 1 || (count > 0 && (!xs || !ns || !codes || !luts)) || !workspaces || !streams)
+        return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_buckets: bad argument");
+    for (int k = 0; k < n_streams; ++k)
+        if (!workspaces[k]) return fail(PRIME_EWORKSPACE, "prime_uniform_8bit_quantize_buckets: a workspace is null");
+    for (int64_t i = 0; i < count; ++i) {
+        const int k = static_cast<int>(i % n_streams);
+        if (int rc = prime_uniform_8bit_quantize(xs[i], ns[i], codes[i], luts + i * kBins, qparams_out ? qparams_out + i : nullptr,
+                                                 workspaces[k], streams[k]))
+            return rc;
+    }
+    return 0;
+}
+
 int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, int64_t count, uint8_t* codes, float* luts,
                                         prime_qparams* qparams_out, prime_stream_t stream) {
     if (count < 0 || (count > 0 && (!offsets || !luts))) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: bad argument");

@@ -272,3 +272,87 @@ ring_reduce_step = torch.ops.prime.ring_reduce_step
 ring_gather_step = torch.ops.prime.ring_gather_step
 uniform_8bit_quantize_stats = torch.ops.prime.uniform_8bit_quantize_stats
 uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched
+
+
+# --------------------------------------------------------------------------------------------
+# Pipelined quantization of many large buckets (the per-layer loop of
+# Diloco.sync_pseudo_gradient, src/zeroband/diloco.py:108-110, without the network in between).
+
+PIPELINE_STREAMS = 3     # measured best on MI355X for 205 MB buckets (1: 5.7, 2: 6.3, 3: 6.8, 4: 6.0 TB/s)
+_side_streams: Dict[int, list] = {}
+
+
+def _pipeline_streams(dev: torch.device, n: int) -> list:
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    pool = _side_streams.setdefault(idx, [])
+    while len(pool) < n:
+        pool.append(torch.cuda.Stream(device=dev))     # default priority
+    return pool[:n]
+
+
+class BucketPlan:
+    """Pointer tables for one set of buckets and their outputs, built once and replayed: the
+    C entry point takes host arrays, and rebuilding them per call would cost more than the
+    launches for small sets."""
+
+    def __init__(self, tensors, codes, luts: torch.Tensor, qparams: torch.Tensor, n_streams: int = PIPELINE_STREAMS):
+        import ctypes
+
+        if len(tensors) != len(codes) or luts.shape != (len(tensors), N_BINS) or qparams.shape != (len(tensors), 4):
+            raise RuntimeError("BucketPlan: outputs do not match the buckets")
+        dev = luts.device
+        for t, c in zip(tensors, codes):
+            _need_f32(t, "quantize_buckets")
+            _need_u8(c, "quantize_buckets")
+            if not (t.is_contiguous() and c.is_contiguous()) or t.numel() != c.numel() or t.device != dev or c.device != dev:
+                raise RuntimeError("quantize_buckets: buckets and codes must be contiguous, of equal size, on one device")
+        if luts.dtype != torch.float32 or qparams.dtype != torch.float64 or not luts.is_contiguous() or not qparams.is_contiguous():
+            raise RuntimeError("quantize_buckets: luts must be contiguous float32, qparams contiguous float64")
+        self.keep = (list(tensors), list(codes), luts, qparams)      # the tables hold raw pointers
+        self.dev = dev
+        self.count = len(tensors)
+        self.n_streams = max(1, min(int(n_streams), max(self.count, 1)))
+        self.streams = _pipeline_streams(dev, self.n_streams)
+        n = self.count
+        self.xs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in tensors])
+        self.ns = (ctypes.c_int64 * n)(*[t.numel() for t in tensors])
+        self.cs = (ctypes.c_void_p * n)(*[c.data_ptr() for c in codes])
+        with torch.cuda.device(dev):
+            self.ws = []
+            for s in self.streams:
+                with torch.cuda.stream(s):
+                    self.ws.append(workspace(dev))
+        self.wss = (ctypes.c_void_p * self.n_streams)(*[w.data_ptr() for w in self.ws])
+        self.sts = (ctypes.c_void_p * self.n_streams)(*[s.cuda_stream for s in self.streams])
+
+    def run(self) -> None:
+        """Enqueue every bucket; returns with the current stream ordered after all of them."""
+        lib = _lib.load()
+        cur = torch.cuda.current_stream(self.dev)
+        start = cur.record_event()
+        for s in self.streams:
+            s.wait_event(start)
+        with torch.cuda.device(self.dev):
+            _lib.check(
+                lib.prime_uniform_8bit_quantize_buckets(self.xs, self.ns, self.count, self.cs, self.keep[2].data_ptr(),
+                                                        self.keep[3].data_ptr(), self.wss, self.sts, self.n_streams),
+                "prime_uniform_8bit_quantize_buckets")
+        for s in self.streams:
+            cur.wait_event(s.record_event())
+
+
+def quantize_buckets(tensors, n_streams: int = PIPELINE_STREAMS):
+    """uniform_8bit_quantize of every bucket in ``tensors``, spread over ``n_streams`` HIP streams so
+    that one bucket's statistics pass overlaps its neighbours' quantize pass.  Results are those of
+    calling uniform_8bit_quantize bucket by bucket.  Returns (list of codes, luts [count, 256],
+    qparams [count, 4]); the current stream is ordered after all the work."""
+    if len(tensors) == 0:
+        raise RuntimeError("quantize_buckets: no buckets")
+    dev = tensors[0].device
+    xs = [t.contiguous() for t in tensors]
+    with torch.cuda.device(dev):
+        codes = [torch.empty(t.shape, dtype=torch.uint8, device=dev) for t in xs]
+        luts = torch.empty((len(xs), N_BINS), dtype=torch.float32, device=dev)
+        qps = torch.empty((len(xs), 4), dtype=torch.float64, device=dev)
+    BucketPlan(xs, codes, luts, qps, n_streams).run()
+    return codes, luts, qps

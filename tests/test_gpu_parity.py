@@ -547,3 +547,33 @@ def test_batched_entry_point_with_ragged_tensors_and_misaligned_base(abi, oracle
         floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
         assert lut_rel_err(gl[t], mean, floor) <= LUT_TOL, (t, xs.size)
     assert not cbase[:shift].cpu().numpy().any() and not cbase[shift + off[-1]:].cpu().numpy().any()
+
+
+@pytest.mark.parametrize("n_streams", [1, 2, 3, 5])
+def test_pipelined_buckets_equal_one_by_one(abi, oracle, n_streams):
+    # buckets spread over several streams give what the one-by-one loop gives, bit for bit
+    from prime_amd import ops
+
+    rng = np.random.default_rng(55)
+    sizes = [1_500_003, 2_000_000, 700_001, 1 << 20, 3, 1_234_567, 999_999]
+    hx = [(rng.standard_t(3, n) * 1e-4).astype(np.float32) for n in sizes]
+    xs = [abi.to_dev(a) for a in hx]
+    announce(f"pipelined buckets over {n_streams} streams")
+    codes, luts, qps = ops.quantize_buckets(xs, n_streams=n_streams)
+    torch.cuda.synchronize()
+    for i, a in enumerate(hx):
+        c1, l1, q1 = abi.uniform(xs[i])
+        assert torch.equal(codes[i], c1) and torch.equal(luts[i], l1) and torch.equal(qps[i], q1)
+        q = abi.qparams(qps[i])
+        assert q["scale"] == oracle.scale_exact(a)
+        oc, _, _ = oracle.uniform_8bit_quantize(a, "given", scale=float(q["scale"]))
+        assert np.array_equal(codes[i].cpu().numpy(), oc)
+    # a plan is replayable: new data in the same buffers, same call
+    plan = ops.BucketPlan(xs, codes, luts, qps, n_streams=n_streams)
+    for x in xs:
+        x.mul_(3.0)
+    plan.run()
+    torch.cuda.synchronize()
+    for i in range(len(xs)):
+        c1, l1, q1 = abi.uniform(xs[i])
+        assert torch.equal(codes[i], c1) and torch.equal(luts[i], l1)
