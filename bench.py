@@ -167,8 +167,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--streams", type=int, default=3,
                     help="HIP streams the buckets are spread over in the timed region (1 = strictly one after another)")
-    ap.add_argument("--legs", default="buckets,ring,t28",
-                    help="comma list of buckets (always run: it carries value and roofline), ring, t28")
+    ap.add_argument("--legs", default="buckets,ring,t28,outer",
+                    help="comma list of buckets (always run: it carries value and roofline), ring, t28, outer")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -376,6 +376,47 @@ def main() -> int:
             "kernels": kernel_table(tprof, event_overhead_us),
         }
         del x28, c28
+        torch.cuda.empty_cache()
+
+    if "outer" in legs:
+        # ---- the callers either side of the path: pseudo-gradient and outer optimizer step -----------
+        n_o = 1 << 28
+        g = torch.Generator(device=dev).manual_seed(7)
+        outer_p = torch.randn(n_o, device=dev, generator=g)
+        inner_p = outer_p + torch.randn(n_o, device=dev, generator=g) * 1e-3
+        grad = torch.empty(n_o, device=dev)
+        mom = torch.zeros(n_o, device=dev)
+        c_o = torch.empty(n_o, dtype=torch.uint8, device=dev)
+        l_o = torch.empty(256, dtype=torch.float32, device=dev)
+        q_o = torch.empty(4, dtype=torch.float64, device=dev)
+
+        def pg():
+            _lib.check(lib.prime_pseudo_gradient_f32(outer_p.data_ptr(), inner_p.data_ptr(), n_o, 8.0, grad.data_ptr(), st), "pg")
+
+        def sgd():
+            _lib.check(lib.prime_outer_sgd_nesterov_f32(outer_p.data_ptr(), mom.data_ptr(), grad.data_ptr(), inner_p.data_ptr(),
+                                                        n_o, 0.7, 0.9, 0, st), "sgd")
+
+        def sgd_codes():
+            _lib.check(lib.prime_outer_sgd_nesterov_u8(outer_p.data_ptr(), mom.data_ptr(), c_o.data_ptr(), l_o.data_ptr(),
+                                                       inner_p.data_ptr(), n_o, 0.7, 0.9, 0, st), "sgd_codes")
+
+        t_pg = timed(pg, args.steps, args.warmup)
+        uniform(grad, c_o, l_o, q_o)
+        t_sgd = timed(sgd, args.steps, args.warmup)
+        t_sgdc = timed(sgd_codes, args.steps, args.warmup)
+        out["outer_step"] = {
+            "workload": "2^28 fp32 parameters: pseudo-gradient (outer - inner) / W; SGD-Nesterov outer step fused with the "
+                        "copy to the inner model, from an fp32 gradient and from uint8 codes + lookup",
+            "pseudo_gradient": {"GBps": round(12.0 * n_o / t_pg / 1e9, 1), "bytes_per_element": 12, "ms": round(t_pg * 1e3, 4),
+                                "frac_of_hbm_peak": round(12.0 * n_o / t_pg / 1e9 / HBM_PEAK_GBS, 4)},
+            "outer_sgd_nesterov": {"GBps": round(24.0 * n_o / t_sgd / 1e9, 1), "bytes_per_element": 24, "ms": round(t_sgd * 1e3, 4),
+                                   "frac_of_hbm_peak": round(24.0 * n_o / t_sgd / 1e9 / HBM_PEAK_GBS, 4)},
+            "outer_sgd_nesterov_from_codes": {"GBps": round(21.0 * n_o / t_sgdc / 1e9, 1), "bytes_per_element": 21,
+                                              "ms": round(t_sgdc * 1e3, 4),
+                                              "frac_of_hbm_peak": round(21.0 * n_o / t_sgdc / 1e9 / HBM_PEAK_GBS, 4)},
+        }
+        del outer_p, inner_p, grad, mom, c_o
         torch.cuda.empty_cache()
 
     if not args.no_cpu_baseline:

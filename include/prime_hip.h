@@ -144,6 +144,30 @@ int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* l
                            uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out,
                            void* ws, prime_stream_t stream);
 
+/* ---- the callers either side of the compression path (src/zeroband/diloco.py) ---- */
+
+/* out[i] = (outer[i] - inner[i]) / world_size: the pseudo-gradient of one bucket as
+ * Diloco.sync_pseudo_gradient forms it, diloco.py:93-101 (grad = cpu_param - gpu_param, then
+ * offloaded_grad_flat_tensor.div_(world_size)), with both parameter copies on the device. */
+int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n, float world_size,
+                              float* out, prime_stream_t stream);
+
+/* The outer optimizer step on one bucket: torch.optim.SGD(lr, momentum, nesterov=True),
+ * diloco.py:72-74 and :212-213, rounded as libtorch's CPU kernels round it
+ * (buf = buf*mu + g, or g on the first step; d = fma(buf, mu, g); p = fma(d, -lr, p)),
+ * followed by the copy of the new parameters to the inner model (sync_inner_model,
+ * diloco.py:137-144) when inner_out is not NULL.  param and momentum_buf are updated in place. */
+int prime_outer_sgd_nesterov_f32(float* param, float* momentum_buf, const float* grad, float* inner_out,
+                                 int64_t n, float lr, float momentum, int first_step,
+                                 prime_stream_t stream);
+
+/* The same step with the reduced pseudo-gradient still in wire form (uint8 codes and their
+ * 256-entry lookup, as the all-gather delivers them, collectives.cpp:204-209): the
+ * dequantize pass is folded in. */
+int prime_outer_sgd_nesterov_u8(float* param, float* momentum_buf, const uint8_t* codes, const float* lut,
+                                float* inner_out, int64_t n, float lr, float momentum, int first_step,
+                                prime_stream_t stream);
+
 /* A plain device copy of n bytes (16-byte vectors): the yardstick the profiler's byte
  * counters are scaled against.  No counterpart in the reference. */
 int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t stream);

@@ -65,6 +65,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_index_add_threads.argtypes = [_f32p, _f32p, _u8p, ctypes.c_int64, ctypes.c_int]
         L.oracle_index_set_threads.argtypes = [_f32p, _f32p, _u8p, ctypes.c_int64, ctypes.c_int]
         L.oracle_div_scalar.argtypes = [_f32p, ctypes.c_int64, ctypes.c_float]
+        L.oracle_pseudo_gradient.argtypes = [_f32p, _f32p, ctypes.c_int64, ctypes.c_float, _f32p]
+        L.oracle_outer_sgd_nesterov.argtypes = [_f32p, _f32p, _f32p, ctypes.c_int64, ctypes.c_float, ctypes.c_float, ctypes.c_int]
         _lib = L
     return _lib
 
@@ -172,6 +174,23 @@ def index_set(out: np.ndarray, lut: np.ndarray, codes: np.ndarray, threads: int 
 def div_scalar(x: np.ndarray, d: float) -> None:
     assert x.dtype == np.float32 and x.flags.c_contiguous
     lib().oracle_div_scalar(_p(x, _f32p), x.size, ctypes.c_float(d))
+
+
+def pseudo_gradient(outer: np.ndarray, inner: np.ndarray, world_size: float) -> np.ndarray:
+    """src/zeroband/diloco.py:93-101: (outer - inner) / world_size in fp32."""
+    outer, inner = _f32(outer), _f32(inner)
+    out = np.empty(outer.size, np.float32)
+    lib().oracle_pseudo_gradient(_p(outer, _f32p), _p(inner, _f32p), outer.size, ctypes.c_float(world_size), _p(out, _f32p))
+    return out
+
+
+def outer_sgd_nesterov(param: np.ndarray, buf: np.ndarray, grad: np.ndarray, lr: float, momentum: float, first_step: bool) -> None:
+    """One step of torch.optim.SGD(lr, momentum, nesterov=True) (diloco.py:72-74), in place on
+    param and buf."""
+    assert param.dtype == np.float32 and buf.dtype == np.float32 and param.flags.c_contiguous and buf.flags.c_contiguous
+    grad = _f32(grad)
+    lib().oracle_outer_sgd_nesterov(_p(param, _f32p), _p(buf, _f32p), _p(grad, _f32p), param.size, ctypes.c_float(lr),
+                                    ctypes.c_float(momentum), int(first_step))
 
 
 def torch_chunk_bounds(n: int, parts: int) -> List[Tuple[int, int]]:

@@ -22,6 +22,9 @@
 //                               the order used by the reference's pinned torch 2.5.1 cannot be
 //                               checked offline: "parity unpinned" for that version only
 //   oracle_index_add / _set     numpy lut[codes] bitwise
+//   oracle_pseudo_gradient      torch (a - b).div_(W) bitwise
+//   oracle_outer_sgd_nesterov   torch.optim.SGD(momentum, nesterov=True) on CPU, bitwise over several
+//                               steps and sizes (vector body and scalar tail of libtorch's kernels)
 //
 // Build: see oracle/build.py (g++ -O3, the reference's only flag, src/zeroband/C/compression.py:8).
 
@@ -265,6 +268,34 @@ void oracle_index_set_threads(float* out, const float* lut, const uint8_t* idx, 
 // collectives.cpp:157  chunk.div_(world_size): libtorch divides fp32 by the scalar in fp32.
 void oracle_div_scalar(float* x, int64_t n, float d) {
     for (int64_t i = 0; i < n; ++i) x[i] = x[i] / d;
+}
+
+// Diloco.sync_pseudo_gradient, src/zeroband/diloco.py:93-101: grad = outer - inner (fp32), then
+// the flat gradient buffer divided by the world size (fp32 division).
+void oracle_pseudo_gradient(const float* outer, const float* inner, int64_t n, float world_size, float* out) {
+    for (int64_t i = 0; i < n; ++i) {
+        volatile float d = outer[i] - inner[i];
+        out[i] = d / world_size;
+    }
+}
+
+// torch.optim.SGD(lr, momentum, nesterov=True).step() on fp32 CPU tensors (the outer optimizer,
+// src/zeroband/diloco.py:72-74,212-213), as libtorch rounds it, found by matching torch bit for
+// bit: buf.mul_(mu).add_(g) is a rounded product plus a rounded sum (buf = g on the first
+// step); g.add(buf, alpha=mu) and p.add_(d, alpha=-lr) are fused multiply-adds.
+void oracle_outer_sgd_nesterov(float* param, float* buf, const float* grad, int64_t n, float lr, float mu, int first_step) {
+    const float neg_lr = -lr;
+    for (int64_t i = 0; i < n; ++i) {
+        const float g = grad[i];
+        if (first_step) {
+            buf[i] = g;
+        } else {
+            volatile float prod = buf[i] * mu;   // rounded on its own
+            buf[i] = prod + g;
+        }
+        const float d = std::fma(buf[i], mu, g);
+        param[i] = std::fma(d, neg_lr, param[i]);
+    }
 }
 
 }  // extern "C"

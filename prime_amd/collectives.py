@@ -15,7 +15,22 @@ def gloo_all_reduce(
     op: dist.ReduceOp = dist.ReduceOp.SUM,
     group: Optional[dist.ProcessGroup] = None,
 ) -> None:
-    """Uncompressed path: pre-divide for AVG, then a SUM all-reduce (collectives.py:12-28)."""
+    """Uncompressed path: pre-divide for AVG, then a SUM all-reduce (collectives.py:12-28).
+    A ``SimulatedRing`` group is reduced in place, rank 0's tensor first."""
+    from .C.collectives import SimulatedRing
+
+    if isinstance(group, SimulatedRing):
+        if op not in [dist.ReduceOp.SUM, dist.ReduceOp.AVG]:
+            raise ValueError(f"Unsupported reduce operation {op}. Only SUM and AVG are supported.")
+        if op == dist.ReduceOp.AVG:
+            for t in group.tensors:
+                t.div_(group.size())
+        total = group.tensors[0].clone()
+        for t in group.tensors[1:]:
+            total.add_(t)
+        for t in group.tensors:
+            t.copy_(total)
+        return
     if group is None:
         group = dist.distributed_c10d._get_default_group()
     if op not in [dist.ReduceOp.SUM, dist.ReduceOp.AVG]:

@@ -612,6 +612,113 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
         p[i] = 0u;
 }
 
+// The pseudo-gradient of one bucket as Diloco.sync_pseudo_gradient forms it
+// (src/zeroband/diloco.py:93-101): grad = outer_param - inner_param, then the whole flat buffer
+// divided by the world size; an fp32 subtraction and an fp32 division per element.
+// 12 bytes per element.
+template <bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer,
+                                                                                   const float* __restrict__ inner, int64_t n,
+                                                                                   float world_size, float* __restrict__ out) {
+    using M = Mem<ALIGNED, false>;
+    const int64_t nvec = n >> 2;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a a[kUnroll], b[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            const bool ok = full || i < nvec;
+            a[j] = ok ? M::ldf4(outer, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            b[j] = ok ? M::ldf4(inner, i) : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) M::stf4(out, i, (a[j] - b[j]) / world_size, false);
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        out[i] = (outer[i] - inner[i]) / world_size;
+    }
+}
+
+// One element of the outer optimizer, torch.optim.SGD(lr, momentum, nesterov=True) as the
+// reference builds it (src/zeroband/diloco.py:72-74) and libtorch's CPU kernels round it:
+//   buf = buf * mu + g     (a product and a sum, each rounded; buf = g on the first step)
+//   d   = fma(buf, mu, g)  (add with alpha: one rounding)
+//   p   = fma(d, -lr, p)
+__device__ __forceinline__ void outer_sgd_one(float& p, float& buf, float g, float neg_lr, float mu, bool first) {
+    buf = first ? g : buf * mu + g;
+    const float d = fmaf(buf, mu, g);
+    p = fmaf(d, neg_lr, p);
+}
+
+// Outer step of DiLoCo on one bucket (diloco.py:212-215): SGD with Nesterov momentum on the
+// outer parameters with the reduced pseudo-gradient, and the copy of the new parameters to
+// the inner model (sync_inner_model, :137-144) in the same pass.  The gradient is fp32
+// (24 bytes per element) or, with CODES, uint8 codes and their lookup table (21 bytes per
+// element, and the dequantize pass is saved).
+template <bool CODES, bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom,
+                                                                              const float* __restrict__ grad,
+                                                                              const uint8_t* __restrict__ codes,
+                                                                              const float* __restrict__ lut,
+                                                                              float* __restrict__ inner, int64_t n, float neg_lr,
+                                                                              float mu, int first) {
+    using M = Mem<ALIGNED, false>;
+    __shared__ float s_lut[kBins];
+    if (CODES) {
+        for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
+        __syncthreads();
+    }
+    const int64_t nvec = n >> 2;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a p[kUnroll], m[kUnroll], g[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            const bool ok = full || i < nvec;
+            p[j] = ok ? M::ldf4(param, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            m[j] = (ok && !first) ? M::ldf4(mom, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            if (CODES) {
+                const uint32_t c = ok ? M::ldu32(codes, i) : 0u;
+                g[j] = f4a{s_lut[c & 255], s_lut[(c >> 8) & 255], s_lut[(c >> 16) & 255], s_lut[c >> 24]};
+            } else {
+                g[j] = ok ? M::ldf4(grad, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float pc = p[j][c], mc = m[j][c];
+                    outer_sgd_one(pc, mc, g[j][c], neg_lr, mu, first);
+                    p[j][c] = pc;
+                    m[j][c] = mc;
+                }
+                M::stf4(param, i, p[j], false);
+                M::stf4(mom, i, m[j], false);
+                if (inner) M::stf4(inner, i, p[j], true);
+            }
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        float p = param[i];
+        float m = first ? 0.f : mom[i];
+        const float g = CODES ? s_lut[codes[i]] : grad[i];
+        outer_sgd_one(p, m, g, neg_lr, mu, first);
+        param[i] = p;
+        mom[i] = m;
+        if (inner) inner[i] = p;
+    }
+}
+
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
     using M = Mem<true, false>;
     sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
@@ -691,12 +798,12 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdCount
+    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
     "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
-    "batched_kernel", "copy_kernel", "fill_zero_kernel"};
+    "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>"};
 
 struct TimedLaunch {
     int id;
@@ -1049,6 +1156,55 @@ int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* l
                            float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
     return ring_step<false>(chunk, codes_in, lut_in, n, codes_out, lut_out, qparams_out, ws, stream,
                             "prime_ring_gather_step: bad argument");
+}
+
+int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n, float world_size, float* out,
+                              prime_stream_t stream) {
+    if (bad_n(n) || (n > 0 && (!outer || !inner || !out))) return fail(PRIME_EINVAL, "prime_pseudo_gradient_f32: bad argument");
+    if (n == 0) return 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int grid = grid_for(n);
+    if (aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(out, 16))
+        launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<true>, grid, kThreads, st, outer, inner, n, world_size, out);
+    else
+        launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<false>, grid, kThreads, st, outer, inner, n, world_size, out);
+    return launch_check("pseudo_gradient_kernel");
+}
+
+int prime_outer_sgd_nesterov_f32(float* param, float* momentum_buf, const float* grad, float* inner_out, int64_t n, float lr,
+                                 float momentum, int first_step, prime_stream_t stream) {
+    if (bad_n(n) || (n > 0 && (!param || !momentum_buf || !grad)))
+        return fail(PRIME_EINVAL, "prime_outer_sgd_nesterov_f32: bad argument");
+    if (n == 0) return 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int grid = grid_for(n);
+    const bool al = aligned_to(param, 16) && aligned_to(momentum_buf, 16) && aligned_to(grad, 16) && aligned_to(inner_out, 16);
+    const double bytes = (inner_out ? 24.0 : 20.0) * n;
+    if (al)
+        launch(kIdOuterStep, bytes, outer_step_kernel<false, true>, grid, kThreads, st, param, momentum_buf, grad, nullptr, nullptr,
+               inner_out, n, -lr, momentum, first_step);
+    else
+        launch(kIdOuterStep, bytes, outer_step_kernel<false, false>, grid, kThreads, st, param, momentum_buf, grad, nullptr, nullptr,
+               inner_out, n, -lr, momentum, first_step);
+    return launch_check("outer_step_kernel");
+}
+
+int prime_outer_sgd_nesterov_u8(float* param, float* momentum_buf, const uint8_t* codes, const float* lut, float* inner_out,
+                                int64_t n, float lr, float momentum, int first_step, prime_stream_t stream) {
+    if (bad_n(n) || (n > 0 && (!param || !momentum_buf || !codes)) || !lut)
+        return fail(PRIME_EINVAL, "prime_outer_sgd_nesterov_u8: bad argument");
+    if (n == 0) return 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int grid = grid_for(n);
+    const bool al = aligned_to(param, 16) && aligned_to(momentum_buf, 16) && aligned_to(codes, 4) && aligned_to(inner_out, 16);
+    const double bytes = (inner_out ? 21.0 : 17.0) * n;
+    if (al)
+        launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, true>, grid, kThreads, st, param, momentum_buf, nullptr, codes, lut,
+               inner_out, n, -lr, momentum, first_step);
+    else
+        launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, false>, grid, kThreads, st, param, momentum_buf, nullptr, codes, lut,
+               inner_out, n, -lr, momentum, first_step);
+    return launch_check("outer_step_kernel");
 }
 
 int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t stream) {

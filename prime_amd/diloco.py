@@ -1,0 +1,130 @@
+"""The DiLoCo outer step around the compression path, with everything resident on the GPU.
+
+Counterpart of the parts of ``zeroband.diloco.Diloco`` (src/zeroband/diloco.py) that sit either
+side of the compressed all-reduce:
+
+  get_offloaded_param   :147-201  one flat fp32 buffer for the outer parameters, one for the
+                                  pseudo-gradient, one view per parameter, one view per layer
+                                  bucket (parameters whose names share their first number)
+  sync_pseudo_gradient  :78-134   grad = outer - inner, flat buffer / world size, all_reduce per bucket
+  outer optimizer       :72-74    torch.optim.SGD(lr=outer_lr, momentum=0.9, nesterov=True)
+  sync_inner_model      :137-144  copy the new outer parameters into the model
+
+The reference keeps the outer copy, the gradient and the optimizer state in host memory and
+pays a device-to-host copy of every parameter per outer step; with 288 GB of HBM they stay on
+the device: the pseudo-gradient is one fused kernel per parameter, and the optimizer step
+and the copy back to the model are one more.  Elastic membership, retries and the barrier of
+the reference (:84,:92-126) belong to its control plane and are not here.
+"""
+from __future__ import annotations
+
+import re
+from functools import lru_cache
+from typing import List, Optional, Sequence
+
+import torch
+import torch.distributed as dist
+from torch import nn
+
+from . import ops
+from .collectives import all_reduce
+from .config import Compression
+
+OUTER_MOMENTUM = 0.9     # diloco.py:73
+
+
+@lru_cache(maxsize=None)
+def _find_first_number(s: str) -> int:
+    """The layer index a parameter name carries, -1 without one (diloco.py:14-21)."""
+    match = re.search(r"\d+", s)
+    return int(match.group()) if match else -1
+
+
+class Diloco:
+    def __init__(self, outer_lr: float, model: nn.Module, compression: Compression = Compression.UINT8):
+        self.outer_lr = float(outer_lr)
+        self.compression = compression
+        self._first_step = True
+        self._init_outer_state(model)
+
+    @torch.no_grad()
+    def _init_outer_state(self, model: nn.Module) -> None:
+        items = [(name, p) for name, p in model.named_parameters() if p.requires_grad]
+        if not items:
+            raise ValueError("model has no trainable parameter")
+        dev = items[0][1].device
+        for name, p in items:
+            if p.dtype != torch.float32 or p.device != dev or not p.data.is_contiguous():
+                raise RuntimeError(f"parameter {name}: contiguous fp32 parameters on one device are required")
+        numel = sum(p.numel() for _, p in items)
+        self.outer_data_flat = torch.empty(numel, device=dev, dtype=torch.float32)
+        self.grad_flat = torch.zeros(numel, device=dev, dtype=torch.float32)
+        self.momentum_flat = torch.zeros(numel, device=dev, dtype=torch.float32)
+        self._views = []                     # (outer, grad, momentum) flat views per parameter
+        cutoffs = []
+        offset, prev = 0, None
+        for name, p in items:
+            if _find_first_number(name) != prev:            # diloco.py:165-167
+                cutoffs.append(offset)
+                prev = _find_first_number(name)
+            n = p.numel()
+            sl = slice(offset, offset + n)
+            self.outer_data_flat[sl].copy_(p.data.reshape(-1))
+            self._views.append((self.outer_data_flat[sl], self.grad_flat[sl], self.momentum_flat[sl]))
+            offset += n
+        cutoffs.append(offset)
+        self.grad_buckets = [self.grad_flat[i:j] for i, j in zip(cutoffs, cutoffs[1:])]      # diloco.py:192-195
+
+    def _params(self, model: nn.Module) -> List[nn.Parameter]:
+        ps = [p for p in model.parameters() if p.requires_grad]
+        if len(ps) != len(self._views):
+            raise RuntimeError("model does not match the one this state was built from")
+        return ps
+
+    @torch.no_grad()
+    def compute_pseudo_gradient(self, model: nn.Module, world_size: int, fake: bool = False) -> None:
+        """grad = (outer - inner) / world_size for every parameter (diloco.py:93-101)."""
+        if fake:
+            self.grad_flat.zero_()                                   # :95-96
+            return
+        for (outer, grad, _), p in zip(self._views, self._params(model)):
+            ops.pseudo_gradient_(grad, outer, p.data.view(-1), float(world_size))
+
+    @torch.no_grad()
+    def all_reduce_buckets(self, group: Optional[object]) -> None:
+        """One all-reduce per layer bucket (diloco.py:108-110)."""
+        for bucket in self.grad_buckets:
+            all_reduce(self.compression, bucket, dist.ReduceOp.SUM, group)
+
+    @torch.no_grad()
+    def outer_step(self, model: nn.Module) -> None:
+        """outer_optimizer.step() and sync_inner_model (diloco.py:212-215), one kernel per parameter."""
+        for (outer, grad, mom), p in zip(self._views, self._params(model)):
+            ops.outer_sgd_nesterov_(outer, mom, grad, p.data.view(-1), self.outer_lr, OUTER_MOMENTUM, self._first_step)
+        self._first_step = False
+
+    @torch.no_grad()
+    def step(self, model: nn.Module, group: Optional[object] = None, world_size: Optional[int] = None, fake: bool = False) -> None:
+        """The whole outer step of one worker (diloco.py:203-215)."""
+        if world_size is None:
+            world_size = group.size() if group is not None else dist.get_world_size()
+        self.compute_pseudo_gradient(model, world_size, fake=fake)
+        self.all_reduce_buckets(group)
+        self.outer_step(model)
+
+
+@torch.no_grad()
+def step_simulated_workers(workers: Sequence[Diloco], models: Sequence[nn.Module], fake: bool = False) -> None:
+    """The outer step of W workers that live in one process on one GPU: every worker forms its
+    pseudo-gradient, each layer bucket goes through the ring all-reduce of W simulated ranks, and
+    every worker applies the outer optimizer."""
+    from .C.collectives import SimulatedRing
+
+    W = len(workers)
+    for w, m in zip(workers, models):
+        w.compute_pseudo_gradient(m, W, fake=fake)
+    for b in range(len(workers[0].grad_buckets)):
+        bucket = [w.grad_buckets[b] for w in workers]
+        all_reduce(workers[0].compression, bucket[0], dist.ReduceOp.SUM, SimulatedRing(bucket))
+    for w, m in zip(workers, models):
+        w.outer_step(m)

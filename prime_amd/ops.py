@@ -275,6 +275,71 @@ uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched
 
 
 # --------------------------------------------------------------------------------------------
+# The callers either side of the path (src/zeroband/diloco.py): pseudo-gradient and outer step.
+
+_LIB.define("pseudo_gradient_(Tensor(a!) out, Tensor outer, Tensor inner, float world_size) -> ()")
+_LIB.define("outer_sgd_nesterov_(Tensor(a!) param, Tensor(b!) momentum_buf, Tensor grad, Tensor(c!)? inner, "
+            "float lr, float momentum, bool first_step) -> ()")
+_LIB.define("outer_sgd_nesterov_codes_(Tensor(a!) param, Tensor(b!) momentum_buf, Tensor codes, Tensor lut, "
+            "Tensor(c!)? inner, float lr, float momentum, bool first_step) -> ()")
+
+
+def _need_flat_f32(t: torch.Tensor, name: str, n: int) -> None:
+    _need_f32(t, name)
+    if not t.is_contiguous() or t.numel() != n:
+        raise RuntimeError(f"{name}: operands must be contiguous fp32 tensors of one size")
+
+
+def _pseudo_gradient_(out: torch.Tensor, outer: torch.Tensor, inner: torch.Tensor, world_size: float) -> None:
+    n = out.numel()
+    for t in (out, outer, inner):
+        _need_flat_f32(t, "pseudo_gradient_", n)
+    lib = _lib.load()
+    dev = out.device
+    with torch.cuda.device(dev):
+        _lib.check(lib.prime_pseudo_gradient_f32(outer.data_ptr(), inner.data_ptr(), n, float(world_size), out.data_ptr(),
+                                                 _stream(dev)), "prime_pseudo_gradient_f32")
+
+
+def _outer_sgd_nesterov_(param, momentum_buf, grad, inner, lr: float, momentum: float, first_step: bool) -> None:
+    n = param.numel()
+    for t in (param, momentum_buf, grad) + ((inner,) if inner is not None else ()):
+        _need_flat_f32(t, "outer_sgd_nesterov_", n)
+    lib = _lib.load()
+    dev = param.device
+    with torch.cuda.device(dev):
+        _lib.check(lib.prime_outer_sgd_nesterov_f32(param.data_ptr(), momentum_buf.data_ptr(), grad.data_ptr(),
+                                                    inner.data_ptr() if inner is not None else None, n, float(lr),
+                                                    float(momentum), int(first_step), _stream(dev)),
+                   "prime_outer_sgd_nesterov_f32")
+
+
+def _outer_sgd_nesterov_codes_(param, momentum_buf, codes, lut, inner, lr: float, momentum: float, first_step: bool) -> None:
+    n = param.numel()
+    for t in (param, momentum_buf) + ((inner,) if inner is not None else ()):
+        _need_flat_f32(t, "outer_sgd_nesterov_codes_", n)
+    _need_u8(codes, "outer_sgd_nesterov_codes_")
+    lut = _need_lut(lut, "outer_sgd_nesterov_codes_")
+    if codes.numel() != n or not codes.is_contiguous():
+        raise RuntimeError("outer_sgd_nesterov_codes_: codes must be contiguous and match param in numel")
+    lib = _lib.load()
+    dev = param.device
+    with torch.cuda.device(dev):
+        _lib.check(lib.prime_outer_sgd_nesterov_u8(param.data_ptr(), momentum_buf.data_ptr(), codes.data_ptr(), lut.data_ptr(),
+                                                   inner.data_ptr() if inner is not None else None, n, float(lr),
+                                                   float(momentum), int(first_step), _stream(dev)),
+                   "prime_outer_sgd_nesterov_u8")
+
+
+_LIB.impl("pseudo_gradient_", _pseudo_gradient_, "CUDA")
+_LIB.impl("outer_sgd_nesterov_", _outer_sgd_nesterov_, "CUDA")
+_LIB.impl("outer_sgd_nesterov_codes_", _outer_sgd_nesterov_codes_, "CUDA")
+pseudo_gradient_ = torch.ops.prime.pseudo_gradient_
+outer_sgd_nesterov_ = torch.ops.prime.outer_sgd_nesterov_
+outer_sgd_nesterov_codes_ = torch.ops.prime.outer_sgd_nesterov_codes_
+
+
+# --------------------------------------------------------------------------------------------
 # Pipelined quantization of many large buckets (the per-layer loop of
 # Diloco.sync_pseudo_gradient, src/zeroband/diloco.py:108-110, without the network in between).
 

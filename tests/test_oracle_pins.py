@@ -319,3 +319,38 @@ def test_oracle_against_compiled_reference(oracle):
         assert lut_rel_err(ol, rl.numpy().astype(np.float64), sc) < 5e-5
         q = R.quantize_per_tensor_uint8(torch.from_numpy(x.copy()), 3e-5, 100).numpy()
         assert np.array_equal(q, oracle.quantize_per_tensor_uint8(x, 3e-5, 100))
+
+
+# ---------------------------------------------------------------- callers of the path (src/zeroband/diloco.py)
+
+def test_pseudo_gradient_is_torch_sub_then_div(oracle):
+    import torch
+
+    rng = np.random.default_rng(13)
+    for n in (1, 7, 1000, 65543):
+        a = rng.standard_normal(n).astype(np.float32)
+        b = (a + rng.standard_normal(n).astype(np.float32) * 1e-3).astype(np.float32)
+        for W in (1.0, 2.0, 3.0, 8.0, 14.0):
+            want = (torch.from_numpy(a) - torch.from_numpy(b)).div_(W).numpy()       # diloco.py:96-101
+            assert np.array_equal(oracle.pseudo_gradient(a, b, W), want)
+
+
+def test_outer_sgd_nesterov_is_torch_sgd_bit_for_bit(oracle):
+    # the reference's outer optimizer: torch.optim.SGD(lr=outer_lr, momentum=0.9, nesterov=True) (diloco.py:72-74)
+    import torch
+
+    rng = np.random.default_rng(14)
+    for n in (1, 3, 8, 15, 17, 33, 1003, 65541):
+        for lr, mu in ((0.7, 0.9), (0.1, 0.5), (1.0, 0.9)):
+            p0 = rng.standard_normal(n).astype(np.float32)
+            p = torch.nn.Parameter(torch.from_numpy(p0.copy()))
+            opt = torch.optim.SGD([p], lr=lr, momentum=mu, nesterov=True)
+            mine = p0.copy()
+            buf = np.zeros(n, np.float32)
+            for step in range(3):
+                g = (rng.standard_normal(n) * 1e-2).astype(np.float32)
+                p.grad = torch.from_numpy(g.copy())
+                opt.step()
+                oracle.outer_sgd_nesterov(mine, buf, g, lr, mu, first_step=(step == 0))
+                assert np.array_equal(mine, p.detach().numpy()), (n, lr, mu, step)
+                assert np.array_equal(buf, opt.state[p]["momentum_buffer"].numpy()), (n, lr, mu, step)
