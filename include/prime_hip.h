@@ -144,6 +144,10 @@ int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* l
                            uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out,
                            void* ws, prime_stream_t stream);
 
+/* x[i] = x[i] / divisor in place: chunk.div_(world_size) of the ring's ReduceOp::AVG,
+ * collectives.cpp:155-159. */
+int prime_div_f32(float* x, int64_t n, float divisor, prime_stream_t stream);
+
 /* ---- the callers either side of the compression path (src/zeroband/diloco.py) ---- */
 
 /* out[i] = (outer[i] - inner[i]) / world_size: the pseudo-gradient of one bucket as

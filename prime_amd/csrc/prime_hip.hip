@@ -13,6 +13,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
+#include <atomic>
 #include <climits>
 #include <cstdint>
 #include <cstdio>
@@ -612,6 +613,31 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
         p[i] = 0u;
 }
 
+// chunk /= world_size for ReduceOp::AVG (collectives.cpp:155-159): an fp32 division in place.
+template <bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void div_kernel(float* __restrict__ x, int64_t n, float d) {
+    using M = Mem<ALIGNED, false>;
+    const int64_t nvec = n >> 2;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a v[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) M::stf4(x, i, v[j] / d, false);
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        x[i] = x[i] / d;
+    }
+}
+
 // The pseudo-gradient of one bucket as Diloco.sync_pseudo_gradient forms it
 // (src/zeroband/diloco.py:93-101): grad = outer_param - inner_param, then the whole flat buffer
 // divided by the world size; an fp32 subtraction and an fp32 division per element.
@@ -798,12 +824,12 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdCount
+    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
     "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
-    "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>"};
+    "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>", "div_kernel"};
 
 struct TimedLaunch {
     int id;
@@ -811,7 +837,7 @@ struct TimedLaunch {
     hipEvent_t a, b;
 };
 struct Profiler {
-    bool on = false;
+    std::atomic<bool> on{false};
     std::mutex m;
     std::vector<TimedLaunch> launches;
 };
@@ -1156,6 +1182,17 @@ int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* l
                            float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
     return ring_step<false>(chunk, codes_in, lut_in, n, codes_out, lut_out, qparams_out, ws, stream,
                             "prime_ring_gather_step: bad argument");
+}
+
+int prime_div_f32(float* x, int64_t n, float divisor, prime_stream_t stream) {
+    if (bad_n(n) || (n > 0 && !x)) return fail(PRIME_EINVAL, "prime_div_f32: bad argument");
+    if (n == 0) return 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (aligned_to(x, 16))
+        launch(kIdDiv, 8.0 * n, div_kernel<true>, grid_for(n), kThreads, st, x, n, divisor);
+    else
+        launch(kIdDiv, 8.0 * n, div_kernel<false>, grid_for(n), kThreads, st, x, n, divisor);
+    return launch_check("div_kernel");
 }
 
 int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n, float world_size, float* out,

@@ -277,6 +277,7 @@ uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched
 # --------------------------------------------------------------------------------------------
 # The callers either side of the path (src/zeroband/diloco.py): pseudo-gradient and outer step.
 
+_LIB.define("div_(Tensor(a!) x, float divisor) -> ()")
 _LIB.define("pseudo_gradient_(Tensor(a!) out, Tensor outer, Tensor inner, float world_size) -> ()")
 _LIB.define("outer_sgd_nesterov_(Tensor(a!) param, Tensor(b!) momentum_buf, Tensor grad, Tensor(c!)? inner, "
             "float lr, float momentum, bool first_step) -> ()")
@@ -288,6 +289,14 @@ def _need_flat_f32(t: torch.Tensor, name: str, n: int) -> None:
     _need_f32(t, name)
     if not t.is_contiguous() or t.numel() != n:
         raise RuntimeError(f"{name}: operands must be contiguous fp32 tensors of one size")
+
+
+def _div_(x: torch.Tensor, divisor: float) -> None:
+    """chunk.div_(world_size) of the ring's AVG (collectives.cpp:155-159)."""
+    _need_flat_f32(x, "div_", x.numel())
+    dev = x.device
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().prime_div_f32(x.data_ptr(), x.numel(), float(divisor), _stream(dev)), "prime_div_f32")
 
 
 def _pseudo_gradient_(out: torch.Tensor, outer: torch.Tensor, inner: torch.Tensor, world_size: float) -> None:
@@ -331,9 +340,11 @@ def _outer_sgd_nesterov_codes_(param, momentum_buf, codes, lut, inner, lr: float
                    "prime_outer_sgd_nesterov_u8")
 
 
+_LIB.impl("div_", _div_, "CUDA")
 _LIB.impl("pseudo_gradient_", _pseudo_gradient_, "CUDA")
 _LIB.impl("outer_sgd_nesterov_", _outer_sgd_nesterov_, "CUDA")
 _LIB.impl("outer_sgd_nesterov_codes_", _outer_sgd_nesterov_codes_, "CUDA")
+div_ = torch.ops.prime.div_
 pseudo_gradient_ = torch.ops.prime.pseudo_gradient_
 outer_sgd_nesterov_ = torch.ops.prime.outer_sgd_nesterov_
 outer_sgd_nesterov_codes_ = torch.ops.prime.outer_sgd_nesterov_codes_

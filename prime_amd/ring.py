@@ -95,7 +95,7 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False)
                 for i in range(BUFFER_COUNT):
                     ch = chunk(r, i + r * BUFFER_COUNT)
                     if avg:
-                        ch.div_(W)                                          # :155-159
+                        ops.div_(ch, float(W))                              # :155-159
                     codes, lut = ops.uniform_8bit_quantize(ch, True)        # :162
                     ops.dequantize_(ch, codes, lut, False)                  # :167-172
 

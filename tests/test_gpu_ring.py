@@ -119,3 +119,18 @@ def test_ops_layer_checks_on_device_tensors(dev):
     assert bool((q == 255).all())
     d = ops.dequantize(c1, l1)
     assert torch.equal(d, l1[c1.long()])
+
+
+def test_div_kernel_is_fp32_division(dev, oracle):
+    # chunk.div_(world_size) of ReduceOp::AVG (collectives.cpp:155-159)
+    from prime_amd import ops
+
+    rng = np.random.default_rng(19)
+    for n in (1, 6, 4097, 1_000_001):
+        x = rng.standard_normal(n).astype(np.float32)
+        for d in (2.0, 3.0, 14.0):
+            t = torch.from_numpy(x.copy()).to(dev)
+            ops.div_(t, d)
+            want = x.copy()
+            oracle.div_scalar(want, d)
+            assert np.array_equal(t.cpu().numpy(), want)
