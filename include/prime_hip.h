@@ -136,6 +136,18 @@ int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut
                            uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out,
                            void* ws, prime_stream_t stream);
 
+/* The last accumulation into a rank's own chunk (reduce-scatter steps past
+ * (world_size - 1) * BUFFER_COUNT, which forward nothing: collectives.cpp:124-133) together
+ * with what ring_allreduce does to that chunk next (:155-162):
+ * acc[i] = (acc[i] + lut_in[codes_in[i]]) / divisor  (chunk.div_(world_size) of ReduceOp::AVG;
+ * pass 1.0f for SUM, which skips the division), then (codes_out, lut_out) =
+ * uniform_8bit_quantize(acc).  The write-back acc = lut_out[codes_out] of :167-172 is
+ * prime_dequant_set, or prime_ring_gather_step when the chunk is forwarded in the all-gather.
+ * 14 bytes per element where the separate calls move 26. */
+int prime_ring_reduce_div_step(float* acc, const uint8_t* codes_in, const float* lut_in, int64_t n, float divisor,
+                               uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out, void* ws,
+                               prime_stream_t stream);
+
 /* One hop of the ring's all-gather as ring_allreduce runs it, collectives.cpp:200-215:
  * chunk[i] = lut_in[codes_in[i]] (fast_index_set_omp), then (codes_out, lut_out) =
  * uniform_8bit_quantize(chunk) for forwarding.  The statistics are taken while the chunk is

@@ -448,10 +448,13 @@ __global__ void lut_zero_kernel(float* __restrict__ lut, int64_t n_bins, unsigne
 
 // K5 / K4 pass A: out = lut[codes] (collectives.cpp:16-22) or out += lut[codes] (:8-14),
 // the lookup table held in LDS; with STATS the fp64 sum and sum of squares of the updated
-// values are taken in the same pass (the next quantization's scale).
-template <bool ADD, bool STATS, bool ALIGNED, bool NT>
+// values are taken in the same pass (the next quantization's scale).  With DIV the updated value
+// is divided by `divisor` before it is stored and counted: chunk.div_(world_size) of
+// ReduceOp::AVG (collectives.cpp:155-159) folded into the last accumulation of a chunk.
+template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV = false>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut,
-                                                           const uint8_t* __restrict__ codes, int64_t n, Workspace* ws) {
+                                                           const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
+                                                           float divisor) {
     using M = Mem<ALIGNED, NT>;
     __shared__ float s_lut[kBins];
     for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
@@ -478,6 +481,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float*
             v.z = s_lut[(c[j] >> 16) & 255];
             v.w = s_lut[c[j] >> 24];
             if (ADD) v += a[j];
+            if (DIV) v = v / divisor;
             if (full || i < nvec) {
                 M::stf4(out, i, v, !STATS);   // with STATS the quantize pass reads it again: no streaming hint
                 if (STATS) {
@@ -490,6 +494,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float*
         const int64_t i = (nvec << 2) + threadIdx.x;
         float v = s_lut[codes[i]];
         if (ADD) v += out[i];
+        if (DIV) v = v / divisor;
         out[i] = v;
         if (STATS) {
             const double d = v;
@@ -932,17 +937,18 @@ int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins
     return launch_check("lut_finalize_kernel");
 }
 
-template <bool ADD, bool STATS>
-int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out) {
+template <bool ADD, bool STATS, bool DIV = false>
+int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out,
+                float divisor = 1.0f) {
     const int grid = grid_for(n);
     const int id = STATS ? (ADD ? kIdDequantAddStats : kIdDequantSetStats) : (ADD ? kIdDequantAdd : kIdDequantSet);
     const double bytes = (ADD ? 9.0 : 5.0) * n;
     if (!(aligned_to(out, 16) && aligned_to(codes, 4)))
-        launch(id, bytes, dequant_kernel<ADD, STATS, false, false>, grid, kThreads, st, out, lut, codes, n, ws);
+        launch(id, bytes, dequant_kernel<ADD, STATS, false, false, DIV>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
     else if (use_nt(n))
-        launch(id, bytes, dequant_kernel<ADD, STATS, true, true>, grid, kThreads, st, out, lut, codes, n, ws);
+        launch(id, bytes, dequant_kernel<ADD, STATS, true, true, DIV>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
     else
-        launch(id, bytes, dequant_kernel<ADD, STATS, true, false>, grid, kThreads, st, out, lut, codes, n, ws);
+        launch(id, bytes, dequant_kernel<ADD, STATS, true, false, DIV>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
     if (grid_out) *grid_out = grid;
     return launch_check("dequant_kernel");
 }
@@ -1153,7 +1159,7 @@ namespace {
 // result taken in the same pass, then the requantization of the chunk.
 template <bool ADD>
 int ring_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out, float* lut_out,
-              prime_qparams* qparams_out, void* ws, prime_stream_t stream, const char* who) {
+              prime_qparams* qparams_out, void* ws, prime_stream_t stream, const char* who, float divisor = 1.0f) {
     if (bad_n(n) || (n > 0 && (!chunk || !codes_in || !codes_out)) || !lut_in || !lut_out) return fail(PRIME_EINVAL, who);
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1163,7 +1169,11 @@ int ring_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_
         return run_lut_finalize(w, 0, lut_out, kBins, nullptr, st);
     }
     int grid = 0;
-    if (int rc = run_dequant<ADD, true>(chunk, lut_in, codes_in, n, w, st, &grid)) return rc;
+    if (ADD && divisor != 1.0f) {
+        if (int rc = run_dequant<ADD, true, ADD>(chunk, lut_in, codes_in, n, w, st, &grid, divisor)) return rc;
+    } else {
+        if (int rc = run_dequant<ADD, true>(chunk, lut_in, codes_in, n, w, st, &grid)) return rc;
+    }
     if (int rc = run_quantize(chunk, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid)) return rc;
     return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
 }
@@ -1176,6 +1186,13 @@ int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut
                            float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
     return ring_step<true>(acc, codes_in, lut_in, n, codes_out, lut_out, qparams_out, ws, stream,
                            "prime_ring_reduce_step: bad argument");
+}
+
+int prime_ring_reduce_div_step(float* acc, const uint8_t* codes_in, const float* lut_in, int64_t n, float divisor,
+                               uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
+    if (!(divisor == divisor) || divisor == 0.0f) return fail(PRIME_EINVAL, "prime_ring_reduce_div_step: divisor must be a non-zero number");
+    return ring_step<true>(acc, codes_in, lut_in, n, codes_out, lut_out, qparams_out, ws, stream,
+                           "prime_ring_reduce_div_step: bad argument", divisor);
 }
 
 int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out,

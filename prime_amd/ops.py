@@ -11,6 +11,7 @@ Schemas mirror the Python signatures of the reference's wrappers
     prime::dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()
     prime::ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
     prime::ring_gather_step(Tensor(a!) chunk, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
+    prime::ring_reduce_div_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in, float divisor) -> (Tensor, Tensor)
     prime::uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)
     prime::uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)
 
@@ -39,6 +40,7 @@ _LIB.define("dequantize(Tensor codes, Tensor lut) -> Tensor")
 _LIB.define("dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()")
 _LIB.define("ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
 _LIB.define("ring_gather_step(Tensor(a!) chunk, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
+_LIB.define("ring_reduce_div_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in, float divisor) -> (Tensor, Tensor)")
 _LIB.define("uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)")
 _LIB.define("uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)")
 
@@ -170,7 +172,13 @@ def _ring_gather_step(chunk: torch.Tensor, codes_in: torch.Tensor, lut_in: torch
     return _ring_step(chunk, codes_in, lut_in, "ring_gather_step")
 
 
-def _ring_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, which: str):
+def _ring_reduce_div_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, divisor: float):
+    """acc = (acc + lut_in[codes_in]) / divisor, then its quantization: the last accumulation into
+    a rank's own chunk with ReduceOp::AVG's division (collectives.cpp:124-133, :155-162)."""
+    return _ring_step(acc, codes_in, lut_in, "ring_reduce_div_step", float(divisor))
+
+
+def _ring_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, which: str, divisor: float = None):
     _need_f32(acc, which)
     _need_u8(codes_in, which)
     lut_in = _need_lut(lut_in, which)
@@ -185,9 +193,14 @@ def _ring_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, 
         codes = torch.empty(acc.shape, dtype=torch.uint8, device=dev)
         lut = torch.empty(N_BINS, dtype=torch.float32, device=dev)
         ws = workspace(dev)
-        fn = lib.prime_ring_reduce_step if which == "ring_reduce_step" else lib.prime_ring_gather_step
-        _lib.check(fn(acc.data_ptr(), c.data_ptr(), lut_in.data_ptr(), acc.numel(), codes.data_ptr(), lut.data_ptr(), None,
-                      ws.data_ptr(), _stream(dev)), f"prime_{which}")
+        if divisor is not None:
+            rc = lib.prime_ring_reduce_div_step(acc.data_ptr(), c.data_ptr(), lut_in.data_ptr(), acc.numel(), divisor,
+                                                codes.data_ptr(), lut.data_ptr(), None, ws.data_ptr(), _stream(dev))
+        else:
+            fn = lib.prime_ring_reduce_step if which == "ring_reduce_step" else lib.prime_ring_gather_step
+            rc = fn(acc.data_ptr(), c.data_ptr(), lut_in.data_ptr(), acc.numel(), codes.data_ptr(), lut.data_ptr(), None,
+                    ws.data_ptr(), _stream(dev))
+        _lib.check(rc, f"prime_{which}")
     return codes, lut
 
 
@@ -221,6 +234,7 @@ _LIB.impl("dequantize", _dequantize, "CUDA")
 _LIB.impl("dequantize_", _dequantize_, "CUDA")
 _LIB.impl("ring_reduce_step", _ring_reduce_step, "CUDA")
 _LIB.impl("ring_gather_step", _ring_gather_step, "CUDA")
+_LIB.impl("ring_reduce_div_step", _ring_reduce_div_step, "CUDA")
 _LIB.impl("uniform_8bit_quantize_stats", _uniform_8bit_quantize_stats, "CUDA")
 _LIB.impl("uniform_8bit_quantize_batched", _uniform_8bit_quantize_batched, "CUDA")
 
@@ -256,6 +270,11 @@ def _(chunk, codes_in, lut_in):
     return chunk.new_empty(chunk.shape, dtype=torch.uint8), chunk.new_empty(N_BINS, dtype=torch.float32)
 
 
+@torch.library.register_fake("prime::ring_reduce_div_step")
+def _(acc, codes_in, lut_in, divisor):
+    return acc.new_empty(acc.shape, dtype=torch.uint8), acc.new_empty(N_BINS, dtype=torch.float32)
+
+
 def unpack_qparams(qp: torch.Tensor) -> dict:
     """Host view of one ``prime_qparams`` record (synchronises)."""
     raw = qp.detach().cpu().contiguous().view(torch.uint8).numpy().tobytes()
@@ -270,6 +289,7 @@ dequantize = torch.ops.prime.dequantize
 dequantize_ = torch.ops.prime.dequantize_
 ring_reduce_step = torch.ops.prime.ring_reduce_step
 ring_gather_step = torch.ops.prime.ring_gather_step
+ring_reduce_div_step = torch.ops.prime.ring_reduce_div_step
 uniform_8bit_quantize_stats = torch.ops.prime.uniform_8bit_quantize_stats
 uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched
 

@@ -64,6 +64,7 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False)
     def chunk(r: int, c: int) -> torch.Tensor:
         return flats[r][c * csz:(c + 1) * csz]
 
+    own: dict = {}     # (rank, chunk) -> (codes, lut) of the rank's reduced chunk, not yet written back
     for phase in (1, 2):
         inbox: List[dict] = [dict() for _ in range(W)]
         for step in range(1, nb + 1):
@@ -82,22 +83,29 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False)
                     else:
                         codes, lut = ops.ring_gather_step(ch, msg[0], msg[1])   # :204-215 fused
                     posted.append(((r + 1) % W, step, codes, lut))
-                    continue
-                if msg is not None:
-                    ops.dequantize_(ch, msg[0], msg[1], phase == 1)         # :128-133 / :204-209
-                if sending:
-                    codes, lut = ops.uniform_8bit_quantize(ch, False)       # :138 / :215
+                elif msg is not None and phase == 1:
+                    # the last accumulation into one of the rank's own chunks, its division for AVG
+                    # and its quantization in two passes (:128-133, :155-162)
+                    own[(r, c)] = ops.ring_reduce_div_step(ch, msg[0], msg[1], float(W) if avg else 1.0)
+                elif msg is not None:
+                    ops.dequantize_(ch, msg[0], msg[1], False)              # :204-209, nothing forwarded
+                elif sending and (r, c) in own:
+                    # the write-back of the rank's own codes (:167-172) and the quantization that
+                    # forwards the chunk (:215), as one gather step
+                    codes, lut = ops.ring_gather_step(ch, *own.pop((r, c)))
+                    posted.append(((r + 1) % W, step, codes, lut))
+                elif sending:
+                    codes, lut = ops.uniform_8bit_quantize(ch, False)       # :138
                     posted.append(((r + 1) % W, step, codes, lut))
             for dst, st, codes, lut in posted:
                 inbox[dst][st] = (codes, lut)
-        if phase == 1:
-            for r in range(W):
-                for i in range(BUFFER_COUNT):
-                    ch = chunk(r, i + r * BUFFER_COUNT)
-                    if avg:
-                        ops.div_(ch, float(W))                              # :155-159
-                    codes, lut = ops.uniform_8bit_quantize(ch, True)        # :162
-                    ops.dequantize_(ch, codes, lut, False)                  # :167-172
+        if phase == 1 and W == 1:
+            # one rank receives nothing: both chunks take the round trip on their own (:155-173)
+            for i in range(BUFFER_COUNT):
+                ch = chunk(0, i)
+                codes, lut = ops.uniform_8bit_quantize(ch, True)            # :162 (dividing by 1 changes nothing)
+                ops.dequantize_(ch, codes, lut, False)                      # :167-172
+    assert not own
 
 
 def ring_allreduce_single(tensor: torch.Tensor, avg: bool = False) -> None:

@@ -67,14 +67,20 @@ class Abi:
         fn = self.lib.prime_dequant_add if add else self.lib.prime_dequant_set
         _lib.check(fn(out.data_ptr(), lut.data_ptr(), codes.data_ptr(), out.numel(), self.st), "dequant")
 
-    def ring_step(self, acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, gather: bool = False):
+    def ring_step(self, acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, gather: bool = False,
+                  divisor: float = None):
         n = acc.numel()
         codes = torch.empty(n, dtype=torch.uint8, device=self.dev)
         lut = torch.empty(256, dtype=torch.float32, device=self.dev)
         qp = torch.empty(4, dtype=torch.float64, device=self.dev)
-        fn = self.lib.prime_ring_gather_step if gather else self.lib.prime_ring_reduce_step
-        _lib.check(fn(acc.data_ptr(), codes_in.data_ptr(), lut_in.data_ptr(), n, codes.data_ptr(), lut.data_ptr(), qp.data_ptr(),
-                      self.ws.data_ptr(), self.st), "ring_step")
+        if divisor is not None:
+            rc = self.lib.prime_ring_reduce_div_step(acc.data_ptr(), codes_in.data_ptr(), lut_in.data_ptr(), n, divisor,
+                                                     codes.data_ptr(), lut.data_ptr(), qp.data_ptr(), self.ws.data_ptr(), self.st)
+        else:
+            fn = self.lib.prime_ring_gather_step if gather else self.lib.prime_ring_reduce_step
+            rc = fn(acc.data_ptr(), codes_in.data_ptr(), lut_in.data_ptr(), n, codes.data_ptr(), lut.data_ptr(), qp.data_ptr(),
+                    self.ws.data_ptr(), self.st)
+        _lib.check(rc, "ring_step")
         return codes, lut, qp
 
     def batched(self, flat: torch.Tensor, offsets: torch.Tensor):

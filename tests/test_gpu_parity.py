@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 import torch
 
+from prime_amd import _lib
 from tests.conftest import lut_rel_err
 from tests.golden.make_fixtures import CASES, case_input
 from tests.gpu_util import Abi, announce
@@ -461,6 +462,50 @@ def test_ring_gather_step_is_set_then_requantize(abi, oracle, n):
     mean, _ = oracle.average_buckets_f64(want, oc)
     floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
     assert lut_rel_err(lut.cpu().numpy(), mean, floor) <= LUT_TOL
+
+
+@pytest.mark.parametrize("n,divisor", [(1, 2.0), (4097, 3.0), (1 << 20, 8.0), (3_000_001, 14.0), (65536, 1.0)])
+def test_ring_reduce_div_step_is_add_divide_requantize(abi, oracle, n, divisor):
+    # last accumulation into a rank's own chunk and ReduceOp::AVG's division
+    # (collectives.cpp:128-133, :155-162): acc = (acc + lut[codes]) / W, then uniform_8bit_quantize(acc)
+    rng = np.random.default_rng(n + int(divisor))
+    src = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    acc0 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    announce(f"reduce+div step n={n} divisor={divisor}")
+    codes_in, lut_in, _ = abi.uniform(abi.to_dev(src))
+    acc = abi.to_dev(acc0)
+    codes, lut, qp = abi.ring_step(acc, codes_in, lut_in, divisor=divisor)
+    # the same through the separate entry points
+    acc2 = abi.to_dev(acc0)
+    abi.dequant(acc2, lut_in, codes_in, add=True)
+    _lib.check(abi.lib.prime_div_f32(acc2.data_ptr(), n, divisor, abi.st), "div")
+    codes2, lut2, qp2 = abi.uniform(acc2)
+    torch.cuda.synchronize()
+    want = acc0.copy()
+    oracle.index_add(want, lut_in.cpu().numpy(), codes_in.cpu().numpy())
+    oracle.div_scalar(want, divisor)
+    assert np.array_equal(acc.cpu().numpy(), want)
+    assert np.array_equal(acc2.cpu().numpy(), want)
+    q = abi.qparams(qp)
+    assert np.array_equal(np.array([q["scale"]]), np.array([oracle.scale_exact(want)]), equal_nan=True)
+    oc, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q["scale"]))
+    assert np.array_equal(codes.cpu().numpy(), oc)
+    assert torch.equal(codes, codes2)
+    mean, _ = oracle.average_buckets_f64(want, oc)
+    floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+    assert lut_rel_err(lut.cpu().numpy(), mean, floor) <= LUT_TOL
+    assert lut_rel_err(lut2.cpu().numpy(), mean, floor) <= LUT_TOL
+
+
+def test_ring_reduce_div_step_rejects_a_zero_or_nan_divisor(abi):
+    acc = abi.to_dev(np.ones(16, np.float32))
+    codes = torch.zeros(16, dtype=torch.uint8, device=abi.dev)
+    lut = torch.zeros(256, device=abi.dev)
+    for bad in (0.0, float("nan")):
+        with pytest.raises(Exception, match="divisor"):
+            abi.ring_step(acc, codes, lut, divisor=bad)
+    torch.cuda.synchronize()
+    assert bool((acc == 1).all())
 
 
 def test_entry_points_replay_from_a_hip_graph(abi, oracle):

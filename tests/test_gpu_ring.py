@@ -94,6 +94,32 @@ def test_ring_avg_and_single_rank(dev, oracle):
     assert len(np.unique(codes_a)) == len(np.unique(got[: n // 2]))
 
 
+@pytest.mark.parametrize("W,avg", [(2, True), (3, True), (4, False), (8, True)])
+def test_whole_schedule_tracks_the_cpu_ring_element_by_element(dev, oracle, W, avg):
+    # Same schedule, same arithmetic: the two runs differ only through lookup entries that
+    # agree to 1e-6, which moves a value across a bin edge now and then.  Nearly every element
+    # must agree to float rounding, and none may be further than a bin or two away.
+    from prime_amd import ring
+
+    n = 2 * W * 20_000
+    xs = _inputs(W, n, 100 + W)
+    cpu = [x.copy() for x in xs]
+    oracle.ring_allreduce_sim(cpu, avg=avg)
+    announce(f"ring element-wise W={W} avg={avg}")
+    gpu = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    ring.ring_allreduce_simulated(gpu, avg=avg)
+    torch.cuda.synchronize()
+    bin_width = 6 * 10 * math.sqrt(W) / 256 / (W if avg else 1)
+    for r in range(W):
+        d = np.abs(gpu[r].cpu().numpy() - cpu[r])
+        assert d.max() < 2.5 * bin_width
+        assert (d > 1e-2 * bin_width).mean() < 2e-3
+    # every rank ends with the same tensor except for the chunks it did not requantize last
+    ref_t = gpu[0].cpu().numpy()
+    for r in range(1, W):
+        assert np.abs(gpu[r].cpu().numpy() - ref_t).max() < 2.5 * bin_width
+
+
 def test_ops_layer_checks_on_device_tensors(dev):
     from prime_amd.C import compression as C
     from prime_amd import ops
