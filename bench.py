@@ -416,7 +416,47 @@ def main() -> int:
                                               "ms": round(t_sgdc * 1e3, 4),
                                               "frac_of_hbm_peak": round(21.0 * n_o / t_sgdc / 1e9 / HBM_PEAK_GBS, 4)},
         }
-        del outer_p, inner_p, grad, mom, c_o
+        # a chunk's first visit in the ring with the pseudo-gradient formed on the way (config 3's chunk
+        # shape), against pseudo-gradient, then ring step as separate calls
+        n_c = RING_CHUNK
+        ci = torch.empty(n_c, dtype=torch.uint8, device=dev)
+        li = torch.empty(256, dtype=torch.float32, device=dev)
+        uniform(grad[:n_c], ci, li, q_o)
+        co = torch.empty(n_c, dtype=torch.uint8, device=dev)
+        lo = torch.empty(256, dtype=torch.float32, device=dev)
+        # eight chunk-sized windows, so that no pass finds its operands in the last-level cache
+        wins = [slice(k * n_c, (k + 1) * n_c) for k in range(n_o // n_c)]
+
+        def touch(with_msg):
+            for w in wins:
+                _lib.check(lib.prime_ring_first_touch(outer_p[w].data_ptr(), inner_p[w].data_ptr(), n_c, 8.0,
+                                                      ci.data_ptr() if with_msg else None, li.data_ptr() if with_msg else None,
+                                                      1.0, grad[w].data_ptr(), co.data_ptr(), lo.data_ptr(), None, ws.data_ptr(), st),
+                           "first touch")
+
+        def separate(with_msg):
+            for w in wins:
+                _lib.check(lib.prime_pseudo_gradient_f32(outer_p[w].data_ptr(), inner_p[w].data_ptr(), n_c, 8.0,
+                                                         grad[w].data_ptr(), st), "pg")
+                if with_msg:
+                    ring_step(grad[w], ci, li, co, lo)
+                else:
+                    uniform(grad[w], co, lo, q_o)
+
+        ft = {}
+        for name, with_msg, fused_b, sep_b in (("send_first", False, 17, 21), ("with_message", True, 18, 26)):
+            t_f = timed(lambda: touch(with_msg), args.steps, args.warmup) / len(wins)
+            t_s = timed(lambda: separate(with_msg), args.steps, args.warmup) / len(wins)
+            ft[name] = {"fused_ms": round(t_f * 1e3, 4), "fused_bytes_per_element": fused_b,
+                        "fused_GBps": round(fused_b * n_c / t_f / 1e9, 1),
+                        "fused_frac_of_hbm_peak": round(fused_b * n_c / t_f / 1e9 / HBM_PEAK_GBS, 4),
+                        "separate_ms": round(t_s * 1e3, 4), "separate_bytes_per_element": sep_b,
+                        "speedup": round(t_s / t_f, 3)}
+        out["outer_step"]["ring_first_touch"] = dict(
+            workload="2^26-element chunks: grad = (outer - inner) / W [+ lut[codes]] and uniform_8bit_quantize(grad) in two "
+                     "passes, against prime_pseudo_gradient_f32 followed by prime_uniform_8bit_quantize / prime_ring_reduce_step",
+            **ft)
+        del outer_p, inner_p, grad, mom, c_o, ci, co
         torch.cuda.empty_cache()
 
     if not args.no_cpu_baseline:

@@ -168,6 +168,22 @@ int prime_div_f32(float* x, int64_t n, float divisor, prime_stream_t stream);
 int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n, float world_size,
                               float* out, prime_stream_t stream);
 
+/* A chunk's first touch in the ring with the pseudo-gradient formed on the way.  Every chunk of
+ * a rank is visited exactly once in the reduce-scatter (collectives.cpp:115-116), so the pass
+ * that would read the pseudo-gradient back can compute it instead:
+ *   grad_out[i] = (outer[i] - inner[i]) / world_size                        (diloco.py:93-101)
+ *   with codes_in:  grad_out[i] = (grad_out[i] + lut_in[codes_in[i]]) / divisor
+ *                   (fast_index_add_omp, collectives.cpp:128-133; chunk.div_ for AVG on a
+ *                   rank's own chunks, :155-159; 1.0f skips the division)
+ *   (codes_out, lut_out) = uniform_8bit_quantize(grad_out)                  (:138 / :162)
+ * codes_in == NULL is the quantization of a chunk that is sent before anything is received
+ * (steps 1 and 2).  17 bytes per element against 12 + 9 for prime_pseudo_gradient_f32 followed
+ * by prime_uniform_8bit_quantize, and 18 against 12 + 14 with a received message. */
+int prime_ring_first_touch(const float* outer, const float* inner, int64_t n, float world_size,
+                           const uint8_t* codes_in, const float* lut_in, float divisor, float* grad_out,
+                           uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out, void* ws,
+                           prime_stream_t stream);
+
 /* The outer optimizer step on one bucket: torch.optim.SGD(lr, momentum, nesterov=True),
  * diloco.py:72-74 and :212-213, rounded as libtorch's CPU kernels round it
  * (buf = buf*mu + g, or g on the first step; d = fma(buf, mu, g); p = fma(d, -lr, p)),

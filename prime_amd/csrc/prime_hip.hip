@@ -675,6 +675,74 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void pseudo_gradient_kerne
     }
 }
 
+// A chunk's first touch in the ring when the pseudo-gradient has not been written yet: every
+// chunk of a rank is visited exactly once in the reduce-scatter (collectives.cpp:115-116), so
+// grad = (outer - inner) / world_size (diloco.py:93-101) can be formed in the pass that would
+// otherwise read it back.  With CODES the received message is accumulated,
+// acc = grad + lut[codes] (collectives.cpp:128-133), and with a divisor other than 1 the sum is
+// divided (ReduceOp::AVG, :155-159).  The fp64 sum and sum of squares of what is stored are the
+// statistics of the quantization that follows.  12 bytes per element, 13 with codes.
+template <bool CODES, bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(const float* __restrict__ outer,
+                                                                               const float* __restrict__ inner, int64_t n,
+                                                                               float world_size, const uint8_t* __restrict__ codes,
+                                                                               const float* __restrict__ lut, float divisor,
+                                                                               float* __restrict__ out, Workspace* ws) {
+    using M = Mem<ALIGNED, false>;
+    __shared__ float s_lut[kBins];
+    if (CODES) {
+        for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
+        __syncthreads();
+    }
+    const bool div = divisor != 1.0f;
+    const int64_t nvec = n >> 2;
+    double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a a[kUnroll], b[kUnroll];
+        uint32_t c[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            const bool ok = full || i < nvec;
+            a[j] = ok ? M::ldf4(outer, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            b[j] = ok ? M::ldf4(inner, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            if (CODES) c[j] = ok ? M::ldu32(codes, i) : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            f4a v = (a[j] - b[j]) / world_size;
+            if (CODES) {
+                f4a l;
+                l.x = s_lut[c[j] & 255];
+                l.y = s_lut[(c[j] >> 8) & 255];
+                l.z = s_lut[(c[j] >> 16) & 255];
+                l.w = s_lut[c[j] >> 24];
+                v += l;
+                if (div) v = v / divisor;
+            }
+            if (full || i < nvec) {
+                M::stf4(out, i, v, false);       // the quantize pass reads it again: no streaming hint
+                if (j & 1) stats_add4(v, s1, q1); else stats_add4(v, s0, q0);
+            }
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        float v = (outer[i] - inner[i]) / world_size;
+        if (CODES) {
+            v += s_lut[codes[i]];
+            if (div) v = v / divisor;
+        }
+        out[i] = v;
+        const double d = v;
+        s0 += d;
+        q0 = fma(d, d, q0);
+    }
+    block_stats_store(s0 + s1, q0 + q1, ws);
+}
+
 // One element of the outer optimizer, torch.optim.SGD(lr, momentum, nesterov=True) as the
 // reference builds it (src/zeroband/diloco.py:72-74) and libtorch's CPU kernels round it:
 //   buf = buf * mu + g     (a product and a sum, each rounded; buf = g on the first step)
@@ -829,12 +897,13 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdCount
+    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouch, kIdFirstTouchCodes, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
     "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
-    "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>", "div_kernel"};
+    "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>", "div_kernel",
+    "first_touch_kernel", "first_touch_kernel<codes>"};
 
 struct TimedLaunch {
     int id;
@@ -1223,6 +1292,43 @@ int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n,
     else
         launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<false>, grid, kThreads, st, outer, inner, n, world_size, out);
     return launch_check("pseudo_gradient_kernel");
+}
+
+int prime_ring_first_touch(const float* outer, const float* inner, int64_t n, float world_size, const uint8_t* codes_in,
+                           const float* lut_in, float divisor, float* grad_out, uint8_t* codes_out, float* lut_out,
+                           prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
+    if (bad_n(n) || (n > 0 && (!outer || !inner || !grad_out || !codes_out)) || !lut_out || (codes_in && !lut_in))
+        return fail(PRIME_EINVAL, "prime_ring_first_touch: bad argument");
+    if (!(divisor == divisor) || divisor == 0.0f) return fail(PRIME_EINVAL, "prime_ring_first_touch: divisor must be a non-zero number");
+    if (!codes_in && divisor != 1.0f)
+        return fail(PRIME_EINVAL, "prime_ring_first_touch: a divisor goes with a received message only (fold it into world_size)");
+    if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Workspace* w = static_cast<Workspace*>(ws);
+    if (n == 0) {
+        if (int rc = run_stats(outer, 0, qparams_out, w, st)) return rc;
+        return run_lut_finalize(w, 0, lut_out, kBins, nullptr, st);
+    }
+    int grid = grid_for(n);
+    const bool al = aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(grad_out, 16) && (!codes_in || aligned_to(codes_in, 4));
+    if (codes_in) {
+        if (al)
+            launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, true>, grid, kThreads, st, outer, inner, n, world_size,
+                   codes_in, lut_in, divisor, grad_out, w);
+        else
+            launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, false>, grid, kThreads, st, outer, inner, n, world_size,
+                   codes_in, lut_in, divisor, grad_out, w);
+    } else {
+        if (al)
+            launch(kIdFirstTouch, 12.0 * n, first_touch_kernel<false, true>, grid, kThreads, st, outer, inner, n, world_size,
+                   nullptr, nullptr, 1.0f, grad_out, w);
+        else
+            launch(kIdFirstTouch, 12.0 * n, first_touch_kernel<false, false>, grid, kThreads, st, outer, inner, n, world_size,
+                   nullptr, nullptr, 1.0f, grad_out, w);
+    }
+    if (int rc = launch_check("first_touch_kernel")) return rc;
+    if (int rc = run_quantize(grad_out, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid)) return rc;
+    return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
 }
 
 int prime_outer_sgd_nesterov_f32(float* param, float* momentum_buf, const float* grad, float* inner_out, int64_t n, float lr,

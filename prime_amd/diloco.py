@@ -15,6 +15,12 @@ pays a device-to-host copy of every parameter per outer step; with 288 GB of HBM
 the device: the pseudo-gradient is one fused kernel per parameter, and the optimizer step
 and the copy back to the model are one more.  Elastic membership, retries and the barrier of
 the reference (:84,:92-126) belong to its control plane and are not here.
+
+With ``flat_inner=True`` the model's own parameters are moved into a fourth flat buffer laid
+out like the other three (each ``param.data`` becomes a view of it).  The pseudo-gradient and
+the outer step are then one launch each over the whole model, and the ring can form the
+pseudo-gradient of a chunk in the pass that first visits it instead of reading it back
+(``prime_amd.ring.ring_allreduce_simulated(..., sources=...)``).
 """
 from __future__ import annotations
 
@@ -41,11 +47,25 @@ def _find_first_number(s: str) -> int:
 
 
 class Diloco:
-    def __init__(self, outer_lr: float, model: nn.Module, compression: Compression = Compression.UINT8):
+    def __init__(self, outer_lr: float, model: nn.Module, compression: Compression = Compression.UINT8,
+                 flat_inner: bool = False):
         self.outer_lr = float(outer_lr)
         self.compression = compression
         self._first_step = True
+        self.inner_flat: Optional[torch.Tensor] = None
         self._init_outer_state(model)
+        if flat_inner:
+            self._flatten_inner(model)
+
+    @torch.no_grad()
+    def _flatten_inner(self, model: nn.Module) -> None:
+        """Move the model's parameters into one flat buffer with the layout of the outer copy."""
+        self.inner_flat = self.outer_data_flat.clone()
+        offset = 0
+        for p in self._params(model):
+            n = p.numel()
+            p.data = self.inner_flat[offset:offset + n].view(p.shape)
+            offset += n
 
     @torch.no_grad()
     def _init_outer_state(self, model: nn.Module) -> None:
@@ -73,6 +93,7 @@ class Diloco:
             self._views.append((self.outer_data_flat[sl], self.grad_flat[sl], self.momentum_flat[sl]))
             offset += n
         cutoffs.append(offset)
+        self.bucket_bounds = list(zip(cutoffs, cutoffs[1:]))
         self.grad_buckets = [self.grad_flat[i:j] for i, j in zip(cutoffs, cutoffs[1:])]      # diloco.py:192-195
 
     def _params(self, model: nn.Module) -> List[nn.Parameter]:
@@ -81,11 +102,25 @@ class Diloco:
             raise RuntimeError("model does not match the one this state was built from")
         return ps
 
+    def _inner_is_flat(self, model: nn.Module) -> bool:
+        """True while every parameter still is the view of ``inner_flat`` it was given."""
+        if self.inner_flat is None:
+            return False
+        offset = 0
+        for p in self._params(model):
+            if p.data.data_ptr() != self.inner_flat.data_ptr() + 4 * offset or not p.data.is_contiguous():
+                return False
+            offset += p.numel()
+        return True
+
     @torch.no_grad()
     def compute_pseudo_gradient(self, model: nn.Module, world_size: int, fake: bool = False) -> None:
         """grad = (outer - inner) / world_size for every parameter (diloco.py:93-101)."""
         if fake:
             self.grad_flat.zero_()                                   # :95-96
+            return
+        if self._inner_is_flat(model):
+            ops.pseudo_gradient_(self.grad_flat, self.outer_data_flat, self.inner_flat, float(world_size))
             return
         for (outer, grad, _), p in zip(self._views, self._params(model)):
             ops.pseudo_gradient_(grad, outer, p.data.view(-1), float(world_size))
@@ -98,7 +133,13 @@ class Diloco:
 
     @torch.no_grad()
     def outer_step(self, model: nn.Module) -> None:
-        """outer_optimizer.step() and sync_inner_model (diloco.py:212-215), one kernel per parameter."""
+        """outer_optimizer.step() and sync_inner_model (diloco.py:212-215), one kernel per parameter
+        (one for the whole model when the inner parameters are flat)."""
+        if self._inner_is_flat(model):
+            ops.outer_sgd_nesterov_(self.outer_data_flat, self.momentum_flat, self.grad_flat, self.inner_flat, self.outer_lr,
+                                    OUTER_MOMENTUM, self._first_step)
+            self._first_step = False
+            return
         for (outer, grad, mom), p in zip(self._views, self._params(model)):
             ops.outer_sgd_nesterov_(outer, mom, grad, p.data.view(-1), self.outer_lr, OUTER_MOMENTUM, self._first_step)
         self._first_step = False
@@ -121,6 +162,20 @@ def step_simulated_workers(workers: Sequence[Diloco], models: Sequence[nn.Module
     from .C.collectives import SimulatedRing
 
     W = len(workers)
+    lazy = (not fake and workers[0].compression == Compression.UINT8
+            and all(w._inner_is_flat(m) for w, m in zip(workers, models))
+            and all((j - i) % (2 * W) == 0 for i, j in workers[0].bucket_bounds))
+    if lazy:
+        # the pseudo-gradient of a chunk is formed in the ring pass that first visits it
+        from . import ring
+
+        for b, (i, j) in enumerate(workers[0].bucket_bounds):
+            ring.ring_allreduce_simulated([w.grad_buckets[b] for w in workers], avg=False,
+                                          sources=[(w.outer_data_flat[i:j], w.inner_flat[i:j]) for w in workers],
+                                          world_size=float(W))
+        for w, m in zip(workers, models):
+            w.outer_step(m)
+        return
     for w, m in zip(workers, models):
         w.compute_pseudo_gradient(m, W, fake=fake)
     for b in range(len(workers[0].grad_buckets)):

@@ -23,7 +23,7 @@ current stream; all arithmetic happens in libprime_hip.so.
 """
 from __future__ import annotations
 
-from typing import Dict, Tuple
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -299,6 +299,8 @@ uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched
 
 _LIB.define("div_(Tensor(a!) x, float divisor) -> ()")
 _LIB.define("pseudo_gradient_(Tensor(a!) out, Tensor outer, Tensor inner, float world_size) -> ()")
+_LIB.define("ring_first_touch_(Tensor(a!) grad, Tensor outer, Tensor inner, float world_size, Tensor? codes_in, Tensor? lut_in, "
+            "float divisor) -> (Tensor, Tensor)")
 _LIB.define("outer_sgd_nesterov_(Tensor(a!) param, Tensor(b!) momentum_buf, Tensor grad, Tensor(c!)? inner, "
             "float lr, float momentum, bool first_step) -> ()")
 _LIB.define("outer_sgd_nesterov_codes_(Tensor(a!) param, Tensor(b!) momentum_buf, Tensor codes, Tensor lut, "
@@ -328,6 +330,37 @@ def _pseudo_gradient_(out: torch.Tensor, outer: torch.Tensor, inner: torch.Tenso
     with torch.cuda.device(dev):
         _lib.check(lib.prime_pseudo_gradient_f32(outer.data_ptr(), inner.data_ptr(), n, float(world_size), out.data_ptr(),
                                                  _stream(dev)), "prime_pseudo_gradient_f32")
+
+
+def _ring_first_touch_(grad: torch.Tensor, outer: torch.Tensor, inner: torch.Tensor, world_size: float,
+                       codes_in: Optional[torch.Tensor], lut_in: Optional[torch.Tensor], divisor: float):
+    """A chunk's only visit in the reduce-scatter with the pseudo-gradient formed on the way:
+    grad = (outer - inner) / world_size (diloco.py:93-101); with a received message
+    grad = (grad + lut_in[codes_in]) / divisor (collectives.cpp:128-133, :155-159); then
+    (codes, lut) = uniform_8bit_quantize(grad).  Returns (codes, lut)."""
+    n = grad.numel()
+    for t in (grad, outer, inner):
+        _need_flat_f32(t, "ring_first_touch_", n)
+    if (codes_in is None) != (lut_in is None):
+        raise RuntimeError("ring_first_touch_: codes_in and lut_in go together")
+    cp = lp = None
+    if codes_in is not None:
+        _need_u8(codes_in, "ring_first_touch_")
+        lut_in = _need_lut(lut_in, "ring_first_touch_")
+        if codes_in.numel() != n:
+            raise RuntimeError("ring_first_touch_: chunk and codes_in differ in numel")
+        codes_in = codes_in.contiguous()
+        cp, lp = codes_in.data_ptr(), lut_in.data_ptr()
+    lib = _lib.load()
+    dev = grad.device
+    with torch.cuda.device(dev):
+        codes = torch.empty(grad.shape, dtype=torch.uint8, device=dev)
+        lut = torch.empty(N_BINS, dtype=torch.float32, device=dev)
+        ws = workspace(dev)
+        _lib.check(lib.prime_ring_first_touch(outer.data_ptr(), inner.data_ptr(), n, float(world_size), cp, lp, float(divisor),
+                                              grad.data_ptr(), codes.data_ptr(), lut.data_ptr(), None, ws.data_ptr(), _stream(dev)),
+                   "prime_ring_first_touch")
+    return codes, lut
 
 
 def _outer_sgd_nesterov_(param, momentum_buf, grad, inner, lr: float, momentum: float, first_step: bool) -> None:
@@ -361,11 +394,13 @@ def _outer_sgd_nesterov_codes_(param, momentum_buf, codes, lut, inner, lr: float
 
 
 _LIB.impl("div_", _div_, "CUDA")
+_LIB.impl("ring_first_touch_", _ring_first_touch_, "CUDA")
 _LIB.impl("pseudo_gradient_", _pseudo_gradient_, "CUDA")
 _LIB.impl("outer_sgd_nesterov_", _outer_sgd_nesterov_, "CUDA")
 _LIB.impl("outer_sgd_nesterov_codes_", _outer_sgd_nesterov_codes_, "CUDA")
 div_ = torch.ops.prime.div_
 pseudo_gradient_ = torch.ops.prime.pseudo_gradient_
+ring_first_touch_ = torch.ops.prime.ring_first_touch_
 outer_sgd_nesterov_ = torch.ops.prime.outer_sgd_nesterov_
 outer_sgd_nesterov_codes_ = torch.ops.prime.outer_sgd_nesterov_codes_
 

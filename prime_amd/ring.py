@@ -14,7 +14,7 @@ Here every "rank" is a tensor on the same device and a send is a hand-over of th
 """
 from __future__ import annotations
 
-from typing import List, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -50,19 +50,41 @@ def _check_ring_inputs(tensors: Sequence[torch.Tensor]) -> int:
     return n
 
 
-def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False) -> None:
+def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
+                             sources: Optional[Sequence[Tuple[torch.Tensor, torch.Tensor]]] = None,
+                             world_size: Optional[float] = None) -> None:
     """The whole of ``ring_allreduce`` for ``len(tensors)`` ranks, in place, in lock step.
 
     A message posted at step s is consumed at step s + 2 (BUFFER_COUNT receive slots,
-    collectives.cpp:118-122), which lock-stepping the ranks reproduces exactly."""
+    collectives.cpp:118-122), which lock-stepping the ranks reproduces exactly.
+
+    With ``sources`` = one (outer, inner) pair of flat tensors per rank, ``tensors[r]`` need not
+    hold anything yet: rank r's pseudo-gradient (outer - inner) / world_size (diloco.py:93-101) is
+    formed chunk by chunk in the reduce-scatter, where every chunk of a rank is visited exactly
+    once, and the result is what the all-reduce of the materialized pseudo-gradients gives."""
     W = len(tensors)
     n = _check_ring_inputs(tensors)
+    if sources is not None:
+        if len(sources) != W:
+            raise ValueError("one (outer, inner) pair per simulated rank is needed")
+        for o, i in sources:
+            if o.numel() != n or i.numel() != n:
+                raise ValueError("outer and inner must have the size of the rank's tensor")
+        if world_size is None:
+            world_size = float(W)
     nb = BUFFER_COUNT * W
     csz = n // nb
     flats = [t.view(-1) for t in tensors]
 
     def chunk(r: int, c: int) -> torch.Tensor:
         return flats[r][c * csz:(c + 1) * csz]
+
+    def touch(r: int, c: int, msg, divisor: float):
+        # first and only visit of chunk c by rank r in the reduce-scatter, pseudo-gradient included
+        o, i = sources[r]
+        sl = slice(c * csz, (c + 1) * csz)
+        return ops.ring_first_touch_(chunk(r, c), o.view(-1)[sl], i.view(-1)[sl], float(world_size),
+                                     None if msg is None else msg[0], None if msg is None else msg[1], divisor)
 
     own: dict = {}     # (rank, chunk) -> (codes, lut) of the rank's reduced chunk, not yet written back
     for phase in (1, 2):
@@ -77,7 +99,13 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False)
                 ch = chunk(r, c)
                 msg = inbox[r].pop(step - BUFFER_COUNT, None)
                 sending = step <= (W - 1) * BUFFER_COUNT                    # :136 / :212
-                if msg is not None and sending:
+                if phase == 1 and sources is not None and (msg is not None or sending):
+                    pair = touch(r, c, msg, float(W) if (avg and not sending) else 1.0)
+                    if sending:
+                        posted.append(((r + 1) % W, step, pair[0], pair[1]))
+                    else:
+                        own[(r, c)] = pair
+                elif msg is not None and sending:
                     if phase == 1:
                         codes, lut = ops.ring_reduce_step(ch, msg[0], msg[1])   # :128-138 fused
                     else:
@@ -103,7 +131,10 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False)
             # one rank receives nothing: both chunks take the round trip on their own (:155-173)
             for i in range(BUFFER_COUNT):
                 ch = chunk(0, i)
-                codes, lut = ops.uniform_8bit_quantize(ch, True)            # :162 (dividing by 1 changes nothing)
+                if sources is not None:
+                    codes, lut = touch(0, i, None, 1.0)
+                else:
+                    codes, lut = ops.uniform_8bit_quantize(ch, True)        # :162 (dividing by 1 changes nothing)
                 ops.dequantize_(ch, codes, lut, False)                      # :167-172
     assert not own
 

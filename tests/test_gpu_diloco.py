@@ -170,6 +170,113 @@ def test_outer_step_of_simulated_workers_against_cpu_emulation(dev, oracle):
     assert float((a - b).abs().max()) < 1e-4
 
 
+@pytest.mark.parametrize("n,with_msg,divisor", [(1, False, 1.0), (4099, False, 1.0), (1 << 20, False, 1.0),
+                                                (5, True, 1.0), (4099, True, 3.0), (1 << 20, True, 1.0), (3_000_001, True, 8.0)])
+def test_ring_first_touch_is_pseudo_gradient_then_ring_step(dev, oracle, n, with_msg, divisor):
+    # grad = (outer - inner) / W (diloco.py:93-101), [grad = (grad + lut[codes]) / divisor
+    # (collectives.cpp:128-133, :155-159)], then uniform_8bit_quantize(grad): through the C ABI,
+    # against the oracle and against the separate entry points
+    from prime_amd import _lib
+    from tests.conftest import lut_rel_err
+    from tests.gpu_util import Abi
+
+    abi = Abi(dev)
+    rng = np.random.default_rng(n + 17)
+    W = 4.0
+    outer = rng.standard_normal(n).astype(np.float32)
+    inner = (outer + rng.standard_normal(n).astype(np.float32) * 1e-3).astype(np.float32)
+    announce(f"first touch n={n} msg={with_msg} divisor={divisor}")
+    want = oracle.pseudo_gradient(outer, inner, W)
+    codes_in = lut_in = None
+    if with_msg:
+        codes_in, lut_in, _ = abi.uniform(abi.to_dev((rng.standard_normal(n) * 2.5e-4).astype(np.float32)))
+        oracle.index_add(want, lut_in.cpu().numpy(), codes_in.cpu().numpy())
+        oracle.div_scalar(want, divisor)
+    to, ti = abi.to_dev(outer), abi.to_dev(inner)
+    grad = torch.full((n,), 7.0, device=dev)                         # overwritten entirely
+    codes = torch.empty(n, dtype=torch.uint8, device=dev)
+    lut = torch.empty(256, device=dev)
+    qp = torch.empty(4, dtype=torch.float64, device=dev)
+    _lib.check(abi.lib.prime_ring_first_touch(to.data_ptr(), ti.data_ptr(), n, W,
+                                              codes_in.data_ptr() if with_msg else None, lut_in.data_ptr() if with_msg else None,
+                                              divisor, grad.data_ptr(), codes.data_ptr(), lut.data_ptr(), qp.data_ptr(),
+                                              abi.ws.data_ptr(), abi.st), "first touch")
+    # the separate entry points
+    g2 = torch.empty(n, device=dev)
+    _lib.check(abi.lib.prime_pseudo_gradient_f32(to.data_ptr(), ti.data_ptr(), n, W, g2.data_ptr(), abi.st), "pg")
+    if with_msg:
+        abi.dequant(g2, lut_in, codes_in, add=True)
+        _lib.check(abi.lib.prime_div_f32(g2.data_ptr(), n, divisor, abi.st), "div")
+    codes2, lut2, qp2 = abi.uniform(g2)
+    torch.cuda.synchronize()
+    assert np.array_equal(grad.cpu().numpy(), want)
+    assert np.array_equal(g2.cpu().numpy(), want)
+    q = abi.qparams(qp)
+    assert np.array_equal(np.array([q["scale"]]), np.array([oracle.scale_exact(want)]), equal_nan=True)
+    oc, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q["scale"]))
+    assert np.array_equal(codes.cpu().numpy(), oc)
+    assert torch.equal(codes, codes2)
+    mean, _ = oracle.average_buckets_f64(want, oc)
+    floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+    assert lut_rel_err(lut.cpu().numpy(), mean, floor) <= 1e-6
+    assert np.array_equal(to.cpu().numpy(), outer) and np.array_equal(ti.cpu().numpy(), inner)
+
+
+def test_ring_first_touch_rejects_bad_arguments(dev):
+    from prime_amd import ops
+
+    n = 64
+    o, i, g = (torch.zeros(n, device=dev) for _ in range(3))
+    codes = torch.zeros(n, dtype=torch.uint8, device=dev)
+    lut = torch.zeros(256, device=dev)
+    with pytest.raises(RuntimeError, match="together"):
+        ops.ring_first_touch_(g, o, i, 2.0, codes, None, 1.0)
+    with pytest.raises(RuntimeError, match="divisor"):
+        ops.ring_first_touch_(g, o, i, 2.0, None, None, 2.0)
+    with pytest.raises(RuntimeError, match="divisor"):
+        ops.ring_first_touch_(g, o, i, 2.0, codes, lut, 0.0)
+    with pytest.raises(RuntimeError, match="numel"):
+        ops.ring_first_touch_(g, o, i, 2.0, codes[:8], lut, 1.0)
+
+
+@pytest.mark.parametrize("W", [1, 2, 4])
+def test_flat_inner_workers_with_lazy_pseudo_gradient_equal_the_plain_ones(dev, W):
+    # same arithmetic, fewer passes: with the model's parameters in one flat buffer the ring forms
+    # each chunk's pseudo-gradient on its first visit; parameters after two outer steps must equal
+    # those of workers that materialize the pseudo-gradient first, bit for bit
+    from prime_amd.diloco import Diloco, step_simulated_workers
+
+    torch.manual_seed(1)
+    base = TinyLlama()
+    plain = [TinyLlama().to(dev) for _ in range(W)]
+    flat = [TinyLlama().to(dev) for _ in range(W)]
+    for m in plain + flat:
+        m.load_state_dict(base.state_dict())
+    wp = [Diloco(0.7, m) for m in plain]
+    wf = [Diloco(0.7, m, flat_inner=True) for m in flat]
+    assert all(w._inner_is_flat(m) for w, m in zip(wf, flat))
+    for outer in range(2):
+        gen = torch.Generator().manual_seed(200 + outer)
+        for mp, mf in zip(plain, flat):
+            for p, f in zip(mp.parameters(), mf.parameters()):
+                delta = (torch.randn(p.shape, generator=gen) * 1e-3).to(dev)
+                p.data.add_(delta)
+                f.data.add_(delta)
+        announce(f"flat-inner diloco W={W} outer step {outer}")
+        step_simulated_workers(wp, plain)
+        step_simulated_workers(wf, flat)
+        torch.cuda.synchronize()
+        for mp, mf, w in zip(plain, flat, wf):
+            assert w._inner_is_flat(mf)
+            for p, f in zip(mp.parameters(), mf.parameters()):
+                assert torch.equal(p.detach(), f.detach())
+        for a, b in zip(wp, wf):
+            assert torch.equal(a.outer_data_flat, b.outer_data_flat) and torch.equal(a.momentum_flat, b.momentum_flat)
+    # a model can still be used as a module: forward through the flat views
+    y = flat[0].output(torch.randn(2, 64, device=dev))
+    assert y.shape == (2, 256)
+
+
 def test_uncompressed_simulated_all_reduce_and_fake_step(dev):
     from prime_amd.C.collectives import SimulatedRing
     from prime_amd.collectives import Compression, all_reduce
