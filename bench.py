@@ -167,8 +167,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--streams", type=int, default=3,
                     help="HIP streams the buckets are spread over in the timed region (1 = strictly one after another)")
-    ap.add_argument("--legs", default="buckets,ring,t28,outer",
-                    help="comma list of buckets (always run: it carries value and roofline), ring, t28, outer")
+    ap.add_argument("--legs", default="buckets,ring,t28,outer,diloco",
+                    help="comma list of buckets (always run: it carries value and roofline), ring, t28, outer, diloco")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -457,6 +457,55 @@ def main() -> int:
                      "passes, against prime_pseudo_gradient_f32 followed by prime_uniform_8bit_quantize / prime_ring_reduce_step",
             **ft)
         del outer_p, inner_p, grad, mom, c_o, ci, co
+        torch.cuda.empty_cache()
+
+    if "diloco" in legs:
+        # ---- a whole outer step of W simulated workers: pseudo-gradient, ring all-reduce, outer step --
+        from prime_amd import ring
+
+        W_d, n_d = 4, 8 * RING_CHUNK                   # 2 W chunks of config 3's chunk size per worker
+        g = torch.Generator(device=dev).manual_seed(11)
+        outers, inners, grads, moms = [], [], [], []
+        for r in range(W_d):
+            o = torch.randn(n_d, device=dev, generator=g)
+            outers.append(o)
+            inners.append(o + torch.randn(n_d, device=dev, generator=g) * 1e-3)
+            grads.append(torch.empty(n_d, device=dev))
+            moms.append(torch.zeros(n_d, device=dev))
+        csz = n_d // (2 * W_d)
+
+        def step_plain():
+            for r in range(W_d):
+                ops.pseudo_gradient_(grads[r], outers[r], inners[r], float(W_d))
+            ring.ring_allreduce_simulated(grads)
+            for r in range(W_d):
+                ops.outer_sgd_nesterov_(outers[r], moms[r], grads[r], inners[r], 0.7, 0.9, False)
+
+        def step_fused():
+            final = ring.ring_allreduce_simulated(grads, sources=list(zip(outers, inners)), world_size=float(W_d), keep_codes=True)
+            for r in range(W_d):
+                for c, (cd, lt) in enumerate(final[r]):
+                    sl = slice(c * csz, (c + 1) * csz)
+                    ops.outer_sgd_nesterov_codes_(outers[r][sl], moms[r][sl], cd, lt, inners[r][sl], 0.7, 0.9, False)
+
+        d_steps = max(2, args.steps // 3)
+        t_plain = timed(step_plain, d_steps, 1)
+        t_fused = timed(step_fused, d_steps, 1)
+        nb_d = 2 * W_d
+        plain_b = (12 * nb_d + 2 * 9 + (nb_d - 2) * 14 + (nb_d - 2) * 10 + 2 * 5 + 24 * nb_d) / nb_d
+        fused_b = (2 * 17 + (nb_d - 2) * 18 + (nb_d - 2) * 3 + 21 * nb_d) / nb_d
+        out["diloco_outer_step"] = {
+            "workload": f"W={W_d} simulated workers of {n_d} fp32 parameters each ({nb_d} chunks of 2^26): pseudo-gradient, "
+                        "uint8 ring all-reduce (both phases), SGD-Nesterov outer step and copy to the inner model",
+            "separate_kernels": {"ms": round(t_plain * 1e3, 3), "bytes_per_element_per_worker": round(plain_b, 2),
+                                 "GBps": round(plain_b * n_d * W_d / t_plain / 1e9, 1)},
+            "fused": {"ms": round(t_fused * 1e3, 3), "bytes_per_element_per_worker": round(fused_b, 2),
+                      "GBps": round(fused_b * n_d * W_d / t_fused / 1e9, 1),
+                      "what": "pseudo-gradient formed at a chunk's first visit, all-gather in the code domain, outer step from codes"},
+            "speedup": round(t_plain / t_fused, 3),
+            "parameters_per_s_fused": round(n_d * W_d / t_fused, 1),
+        }
+        del outers, inners, grads, moms
         torch.cuda.empty_cache()
 
     if not args.no_cpu_baseline:

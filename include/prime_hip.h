@@ -148,6 +148,16 @@ int prime_ring_reduce_div_step(float* acc, const uint8_t* codes_in, const float*
                                uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out, void* ws,
                                prime_stream_t stream);
 
+/* (codes_out, lut_out) = uniform_8bit_quantize(t) for t[i] = lut_in[codes_in[i]], without t: the
+ * quantization that forwards a chunk in the all-gather (collectives.cpp:204-215) when the fp32
+ * chunk itself is not needed yet.  t holds at most 256 distinct values, so the statistics
+ * follow from the population of each code, codes_out[i] is a 256-entry map of codes_in[i] and
+ * lut_out is the population-weighted mean of the old entries that share a new code.  Codes are
+ * those of the two-pass path bit for bit; 3 bytes per element instead of 10.  codes_out must
+ * not overlap codes_in. */
+int prime_requantize_codes(const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out,
+                           float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream);
+
 /* One hop of the ring's all-gather as ring_allreduce runs it, collectives.cpp:200-215:
  * chunk[i] = lut_in[codes_in[i]] (fast_index_set_omp), then (codes_out, lut_out) =
  * uniform_8bit_quantize(chunk) for forwarding.  The statistics are taken while the chunk is

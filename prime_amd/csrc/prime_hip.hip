@@ -33,6 +33,9 @@ namespace {
 #ifndef PRIME_THREADS
 #define PRIME_THREADS 1024               // workgroup size of the streaming kernels
 #endif
+#ifndef PRIME_COUNT_REPLICAS
+#define PRIME_COUNT_REPLICAS 16          // LDS copies of each counter in the code-population kernel
+#endif
 #ifndef PRIME_BLOCKS_PER_CU
 #define PRIME_BLOCKS_PER_CU 2            // resident workgroups per compute unit (32 wavefronts)
 #endif
@@ -61,18 +64,25 @@ struct BinAcc {
 // boundary makes them visible to the second stage.  Nothing has to be zero between calls.
 struct Workspace {
     prime_qparams qp;                    // scale of the tensor in flight
+    uint32_t code_map[kBins / 4];        // old code -> new code of a requantization in the code domain
+    unsigned long long code_total[kBins];   // population of each code over the whole tensor
     double part_sum[kMaxGrid];
     double part_sq[kMaxGrid];
-    BinAcc hist[kMaxGrid][kBins];        // 4 KiB per workgroup
+    union {
+        BinAcc hist[kMaxGrid][kBins];    // 4 KiB per workgroup
+        uint32_t code_cnt[kMaxGrid][kBins];   // per-workgroup populations of each code value
+    };
 };
 
 typedef float f4a __attribute__((ext_vector_type(4)));   // 16-byte aligned
+typedef uint32_t u4a __attribute__((ext_vector_type(4)));   // 16 codes, 16-byte aligned
 
 // Under-aligned views for buffers that are only element aligned (a chunk or a view that
 // starts at an odd element).  They are distinct struct types, so the alignment survives
 // template deduction; the compiler picks accesses that are legal for that alignment.
 struct __attribute__((packed, aligned(4))) F4U { float x, y, z, w; };
 struct __attribute__((packed)) U32U { uint32_t v; };
+struct __attribute__((packed)) U4U { uint32_t x, y, z, w; };
 
 // Streamed accesses, 4 floats / 4 codes at vector index i.  ALIGNED means the float buffer is
 // 16-byte aligned and the code buffer 4-byte aligned.  NT adds the non-temporal hint to loads:
@@ -437,6 +447,220 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
     }
     if (blockIdx.x == 0)
         for (int64_t b = kBins + threadIdx.x; b < n_bins; b += kFinalThreads) lut[b] = 0.0f;
+}
+
+// ---- requantization in the code domain ----------------------------------------------------
+// The all-gather forwards uniform_8bit_quantize(chunk) of a chunk that was just set to
+// lut_in[codes_in] (collectives.cpp:204-215).  Such a chunk holds at most 256 distinct values, so
+// its quantization is a function of the received codes alone: the statistics follow from the
+// population of each code, the new code of an element from a 256-entry map, and a new lookup
+// entry is the population-weighted mean of the old entries that map to it.  3 bytes per element
+// (codes read twice, written once) instead of a pass over the fp32 chunk.
+
+// 16 codes at vector index i; ALIGNED means both code buffers are 16-byte aligned.
+template <bool ALIGNED>
+__device__ __forceinline__ u4a ld_codes16(const uint8_t* p, int64_t i) {
+    if (ALIGNED) return reinterpret_cast<const u4a*>(p)[i];
+    const U4U t = reinterpret_cast<const U4U*>(p)[i];
+    return u4a{t.x, t.y, t.z, t.w};
+}
+
+template <bool ALIGNED>
+__device__ __forceinline__ void st_codes16(uint8_t* p, int64_t i, u4a v) {
+    if (ALIGNED) __builtin_nontemporal_store(v, reinterpret_cast<u4a*>(p) + i);
+    else reinterpret_cast<U4U*>(p)[i] = U4U{v.x, v.y, v.z, v.w};
+}
+
+// Pass 1: population of each code value, one partial per workgroup.  1 byte per element.
+template <bool ALIGNED, int R>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_count_kernel(const uint8_t* __restrict__ codes, int64_t n,
+                                                                              Workspace* ws) {
+    __shared__ unsigned cnt[kBins * R];
+    for (int i = threadIdx.x; i < kBins * R; i += kThreads) cnt[i] = 0u;
+    __syncthreads();
+    const int rep = threadIdx.x & (R - 1);
+    auto bump = [&](uint32_t code) {
+        __hip_atomic_fetch_add(&cnt[code * R + rep], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    const int64_t nvec = n >> 4;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        u4a v[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            v[j] = (full || i < nvec) ? ld_codes16<ALIGNED>(codes, i) : u4a{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t w = v[j][k];
+                    bump(w & 255);
+                    bump((w >> 8) & 255);
+                    bump((w >> 16) & 255);
+                    bump(w >> 24);
+                }
+            }
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 15)) bump(codes[(nvec << 4) + threadIdx.x]);
+    __syncthreads();
+    for (int b = threadIdx.x; b < kBins; b += kThreads) {
+        unsigned c = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) c += cnt[b * R + r];
+        ws->code_cnt[blockIdx.x][b] = c;
+    }
+}
+
+// Between the passes, first kernel: total population of each code.  Workgroup j owns codes
+// 4j .. 4j+3 (16 contiguous bytes of every partial); lane (row, code) adds partials row,
+// row + 256, ..., then the rows are added by a tree of fixed shape.
+__global__ __launch_bounds__(kFinalThreads) void code_total_kernel(Workspace* ws, int nparts) {
+    constexpr int kRows = kFinalThreads / kLutBinsPerBlock;
+    __shared__ unsigned long long sh_cnt[kFinalThreads];
+    const int bl = threadIdx.x % kLutBinsPerBlock;
+    const int row = threadIdx.x / kLutBinsPerBlock;
+    const int bin = blockIdx.x * kLutBinsPerBlock + bl;
+    constexpr int kIters = kMaxGrid / kRows;
+    uint32_t part[kIters];
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) {          // all loads in flight at once
+        const int p = row + k * kRows;
+        part[k] = p < nparts ? ws->code_cnt[p][bin] : 0u;
+    }
+    unsigned long long c = 0;
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) c += part[k];
+    sh_cnt[threadIdx.x] = c;
+    __syncthreads();
+    for (int half = kRows / 2; half > 0; half >>= 1) {
+        if (row < half) sh_cnt[threadIdx.x] += sh_cnt[threadIdx.x + half * kLutBinsPerBlock];
+        __syncthreads();
+    }
+    if (row == 0) ws->code_total[bin] = sh_cnt[threadIdx.x];
+}
+
+// Between the passes, second kernel, one workgroup: the statistics
+// sum = sum_c count_c * lut_in[c] and sumsq = sum_c count_c * lut_in[c]^2 in fp64, the scale
+// (compression.cpp:113-116), the map old code -> new code (:23-24 applied to lut_in[c]) and the
+// new lookup table (:99-101).  Entries of lut_in whose code does not occur are ignored.
+__global__ __launch_bounds__(kFinalThreads) void requant_plan_kernel(Workspace* ws, const float* __restrict__ lut_in, int64_t n,
+                                                                      float* __restrict__ lut_out, prime_qparams* qp_out) {
+    struct Rec {
+        double term;                 // count * value
+        unsigned long long count;
+        int target;                  // new code, -1 when the old code does not occur
+        int pad;
+    };
+    constexpr int kGroups = kFinalThreads / kBins;
+    constexpr int kSpan = kBins / kGroups;
+    __shared__ Rec rec[kBins];
+    __shared__ double sh_s[kBins / 64], sh_q[kBins / 64];
+    __shared__ float sh_inv;
+    __shared__ double g_sum[kGroups][kBins];
+    __shared__ unsigned long long g_cnt[kGroups][kBins];
+    const int bin = threadIdx.x & (kBins - 1);
+    float v = 0.0f;
+    unsigned long long t = 0;
+    if (threadIdx.x < kBins) {
+        t = ws->code_total[bin];
+        v = lut_in[bin];
+        double s = 0.0, q = 0.0;
+        if (t) {
+            const double dv = v, dc = static_cast<double>(t);
+            s = dc * dv;
+            q = dc * (dv * dv);
+        }
+        rec[bin].term = s;
+        rec[bin].count = t;
+        s = wave_sum(s);
+        q = wave_sum(q);
+        if ((threadIdx.x & 63) == 0) { sh_s[threadIdx.x >> 6] = s; sh_q[threadIdx.x >> 6] = q; }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double S = sh_s[0], Q = sh_q[0];
+#pragma unroll
+        for (int w = 1; w < kBins / 64; ++w) { S += sh_s[w]; Q += sh_q[w]; }
+        prime_qparams qp;
+        finalize_qparams(S, Q, n, &qp);
+        sh_inv = qp.inv_scale;
+        ws->qp = qp;
+        if (qp_out) *qp_out = qp;
+    }
+    __syncthreads();
+    int target = 0;
+    if (threadIdx.x < kBins) {
+        target = quantize_code(v, sh_inv, kZeroPoint);
+        rec[bin].target = t ? target : -1;
+    }
+    __syncthreads();
+    {
+        // new entry `bin`: population-weighted mean of the old entries that map to it; the 256 old
+        // codes are split over kGroups groups of lanes, joined in a fixed order
+        const int group = threadIdx.x / kBins;
+        double sum = 0.0;
+        unsigned long long k = 0;
+#pragma unroll 16
+        for (int j = 0; j < kSpan; ++j) {
+            const Rec r = rec[group * kSpan + j];
+            const bool hit = r.target == bin;
+            sum += hit ? r.term : 0.0;
+            k += hit ? r.count : 0ull;
+        }
+        g_sum[group][bin] = sum;
+        g_cnt[group][bin] = k;
+    }
+    __syncthreads();
+    if (threadIdx.x < kBins) {
+        double sum = g_sum[0][bin];
+        unsigned long long k = g_cnt[0][bin];
+#pragma unroll
+        for (int g = 1; g < kGroups; ++g) { sum += g_sum[g][bin]; k += g_cnt[g][bin]; }
+        lut_out[bin] = k ? static_cast<float>(sum / static_cast<double>(k)) : 0.0f;
+        // four adjacent lanes pack their new codes into one word of the map
+        uint32_t word = static_cast<uint32_t>(target) << (8 * (bin & 3));
+        word |= __shfl_xor(word, 1, 64);
+        word |= __shfl_xor(word, 2, 64);
+        if ((bin & 3) == 0) ws->code_map[bin >> 2] = word;
+    }
+}
+
+// Pass 2: codes_out[i] = map[codes_in[i]].  2 bytes per element.
+template <bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_remap_kernel(const uint8_t* __restrict__ in, uint8_t* __restrict__ out,
+                                                                              int64_t n, const Workspace* __restrict__ ws) {
+    __shared__ uint32_t map_words[kBins / 4];
+    if (threadIdx.x < kBins / 4) map_words[threadIdx.x] = ws->code_map[threadIdx.x];
+    __syncthreads();
+    const uint8_t* map = reinterpret_cast<const uint8_t*>(map_words);
+    auto remap = [&](uint32_t w) {
+        return static_cast<uint32_t>(map[w & 255]) | (static_cast<uint32_t>(map[(w >> 8) & 255]) << 8) |
+               (static_cast<uint32_t>(map[(w >> 16) & 255]) << 16) | (static_cast<uint32_t>(map[w >> 24]) << 24);
+    };
+    const int64_t nvec = n >> 4;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        u4a v[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            v[j] = (full || i < nvec) ? ld_codes16<ALIGNED>(in, i) : u4a{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) st_codes16<ALIGNED>(out, i, u4a{remap(v[j].x), remap(v[j].y), remap(v[j].z), remap(v[j].w)});
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 15)) {
+        const int64_t i = (nvec << 4) + threadIdx.x;
+        out[i] = map[in[i]];
+    }
 }
 
 __global__ void lut_zero_kernel(float* __restrict__ lut, int64_t n_bins, unsigned long long* __restrict__ counts) {
@@ -897,13 +1121,13 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouch, kIdFirstTouchCodes, kIdCount
+    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouch, kIdFirstTouchCodes, kIdCodeCount, kIdCodeTotal, kIdRequantPlan, kIdCodeRemap, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
     "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
     "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>", "div_kernel",
-    "first_touch_kernel", "first_touch_kernel<codes>"};
+    "first_touch_kernel", "first_touch_kernel<codes>", "code_count_kernel", "code_total_kernel", "requant_plan_kernel", "code_remap_kernel"};
 
 struct TimedLaunch {
     int id;
@@ -1020,6 +1244,30 @@ int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, W
         launch(id, bytes, dequant_kernel<ADD, STATS, true, false, DIV>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
     if (grid_out) *grid_out = grid;
     return launch_check("dequant_kernel");
+}
+
+// Workgroups for a kernel that streams 16 codes per lane and step.
+int grid_for_codes(int64_t n) { return grid_for((n + 3) / 4); }
+
+// (codes_out, lut_out) = uniform_8bit_quantize(lut_in[codes_in]) without the fp32 tensor.
+int run_requantize_codes(const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out, float* lut_out,
+                         prime_qparams* qp_out, Workspace* ws, hipStream_t st) {
+    const int grid = grid_for_codes(n);
+    const bool al = aligned_to(codes_in, 16) && aligned_to(codes_out, 16);
+    if (al)
+        launch(kIdCodeCount, 1.0 * n, code_count_kernel<true, PRIME_COUNT_REPLICAS>, grid, kThreads, st, codes_in, n, ws);
+    else
+        launch(kIdCodeCount, 1.0 * n, code_count_kernel<false, PRIME_COUNT_REPLICAS>, grid, kThreads, st, codes_in, n, ws);
+    if (int rc = launch_check("code_count_kernel")) return rc;
+    launch(kIdCodeTotal, 4.0 * kBins * grid, code_total_kernel, kBins / kLutBinsPerBlock, kFinalThreads, st, ws, grid);
+    if (int rc = launch_check("code_total_kernel")) return rc;
+    launch(kIdRequantPlan, 0.0, requant_plan_kernel, 1, kFinalThreads, st, ws, lut_in, n, lut_out, qp_out);
+    if (int rc = launch_check("requant_plan_kernel")) return rc;
+    if (al)
+        launch(kIdCodeRemap, 2.0 * n, code_remap_kernel<true>, grid, kThreads, st, codes_in, codes_out, n, ws);
+    else
+        launch(kIdCodeRemap, 2.0 * n, code_remap_kernel<false>, grid, kThreads, st, codes_in, codes_out, n, ws);
+    return launch_check("code_remap_kernel");
 }
 
 bool bad_n(int64_t n) { return n < 0 || n > kMaxElems; }
@@ -1218,6 +1466,20 @@ int prime_dequant_add(float* out, const float* lut, const uint8_t* codes, int64_
     if (bad_n(n) || (n > 0 && (!out || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_dequant_add: bad argument");
     if (n == 0) return 0;
     return run_dequant<true, false>(out, lut, codes, n, nullptr, static_cast<hipStream_t>(stream), nullptr);
+}
+
+int prime_requantize_codes(const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out, float* lut_out,
+                           prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
+    if (bad_n(n) || (n > 0 && (!codes_in || !codes_out)) || !lut_in || !lut_out)
+        return fail(PRIME_EINVAL, "prime_requantize_codes: bad argument");
+    if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Workspace* w = static_cast<Workspace*>(ws);
+    if (n == 0) {
+        if (int rc = run_stats(lut_in, 0, qparams_out, w, st)) return rc;
+        return run_lut_finalize(w, 0, lut_out, kBins, nullptr, st);
+    }
+    return run_requantize_codes(codes_in, lut_in, n, codes_out, lut_out, qparams_out, w, st);
 }
 
 }  // extern "C"

@@ -155,7 +155,8 @@ class Diloco:
 
 
 @torch.no_grad()
-def step_simulated_workers(workers: Sequence[Diloco], models: Sequence[nn.Module], fake: bool = False) -> None:
+def step_simulated_workers(workers: Sequence[Diloco], models: Sequence[nn.Module], fake: bool = False,
+                           coded_gather: bool = True) -> None:
     """The outer step of W workers that live in one process on one GPU: every worker forms its
     pseudo-gradient, each layer bucket goes through the ring all-reduce of W simulated ranks, and
     every worker applies the outer optimizer."""
@@ -166,15 +167,26 @@ def step_simulated_workers(workers: Sequence[Diloco], models: Sequence[nn.Module
             and all(w._inner_is_flat(m) for w, m in zip(workers, models))
             and all((j - i) % (2 * W) == 0 for i, j in workers[0].bucket_bounds))
     if lazy:
-        # the pseudo-gradient of a chunk is formed in the ring pass that first visits it
+        # the pseudo-gradient of a chunk is formed in the ring pass that first visits it; with
+        # coded_gather the all-gather stays in the code domain and the outer step dequantizes
         from . import ring
 
         for b, (i, j) in enumerate(workers[0].bucket_bounds):
-            ring.ring_allreduce_simulated([w.grad_buckets[b] for w in workers], avg=False,
-                                          sources=[(w.outer_data_flat[i:j], w.inner_flat[i:j]) for w in workers],
-                                          world_size=float(W))
+            final = ring.ring_allreduce_simulated([w.grad_buckets[b] for w in workers], avg=False,
+                                                  sources=[(w.outer_data_flat[i:j], w.inner_flat[i:j]) for w in workers],
+                                                  world_size=float(W), keep_codes=coded_gather)
+            if coded_gather:
+                csz = (j - i) // (2 * W)
+                for w, chunks in zip(workers, final):
+                    for c, (codes, lut) in enumerate(chunks):
+                        sl = slice(i + c * csz, i + (c + 1) * csz)
+                        ops.outer_sgd_nesterov_codes_(w.outer_data_flat[sl], w.momentum_flat[sl], codes, lut, w.inner_flat[sl],
+                                                      w.outer_lr, OUTER_MOMENTUM, w._first_step)
         for w, m in zip(workers, models):
-            w.outer_step(m)
+            if coded_gather:
+                w._first_step = False
+            else:
+                w.outer_step(m)
         return
     for w, m in zip(workers, models):
         w.compute_pseudo_gradient(m, W, fake=fake)

@@ -11,6 +11,7 @@ Schemas mirror the Python signatures of the reference's wrappers
     prime::dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()
     prime::ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
     prime::ring_gather_step(Tensor(a!) chunk, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
+    prime::requantize_codes(Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
     prime::ring_reduce_div_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in, float divisor) -> (Tensor, Tensor)
     prime::uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)
     prime::uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)
@@ -40,6 +41,7 @@ _LIB.define("dequantize(Tensor codes, Tensor lut) -> Tensor")
 _LIB.define("dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()")
 _LIB.define("ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
 _LIB.define("ring_gather_step(Tensor(a!) chunk, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
+_LIB.define("requantize_codes(Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
 _LIB.define("ring_reduce_div_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in, float divisor) -> (Tensor, Tensor)")
 _LIB.define("uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)")
 _LIB.define("uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)")
@@ -172,6 +174,23 @@ def _ring_gather_step(chunk: torch.Tensor, codes_in: torch.Tensor, lut_in: torch
     return _ring_step(chunk, codes_in, lut_in, "ring_gather_step")
 
 
+def _requantize_codes(codes_in: torch.Tensor, lut_in: torch.Tensor):
+    """uniform_8bit_quantize(lut_in[codes_in]) computed from the codes alone: what the all-gather
+    forwards (collectives.cpp:204-215) when the fp32 chunk is not needed yet."""
+    _need_u8(codes_in, "requantize_codes")
+    lut_in = _need_lut(lut_in, "requantize_codes")
+    lib = _lib.load()
+    c = codes_in.contiguous()
+    dev = c.device
+    with torch.cuda.device(dev):
+        codes = torch.empty(c.shape, dtype=torch.uint8, device=dev)
+        lut = torch.empty(N_BINS, dtype=torch.float32, device=dev)
+        ws = workspace(dev)
+        _lib.check(lib.prime_requantize_codes(c.data_ptr(), lut_in.data_ptr(), c.numel(), codes.data_ptr(), lut.data_ptr(), None,
+                                              ws.data_ptr(), _stream(dev)), "prime_requantize_codes")
+    return codes, lut
+
+
 def _ring_reduce_div_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, divisor: float):
     """acc = (acc + lut_in[codes_in]) / divisor, then its quantization: the last accumulation into
     a rank's own chunk with ReduceOp::AVG's division (collectives.cpp:124-133, :155-162)."""
@@ -234,6 +253,7 @@ _LIB.impl("dequantize", _dequantize, "CUDA")
 _LIB.impl("dequantize_", _dequantize_, "CUDA")
 _LIB.impl("ring_reduce_step", _ring_reduce_step, "CUDA")
 _LIB.impl("ring_gather_step", _ring_gather_step, "CUDA")
+_LIB.impl("requantize_codes", _requantize_codes, "CUDA")
 _LIB.impl("ring_reduce_div_step", _ring_reduce_div_step, "CUDA")
 _LIB.impl("uniform_8bit_quantize_stats", _uniform_8bit_quantize_stats, "CUDA")
 _LIB.impl("uniform_8bit_quantize_batched", _uniform_8bit_quantize_batched, "CUDA")
@@ -270,6 +290,11 @@ def _(chunk, codes_in, lut_in):
     return chunk.new_empty(chunk.shape, dtype=torch.uint8), chunk.new_empty(N_BINS, dtype=torch.float32)
 
 
+@torch.library.register_fake("prime::requantize_codes")
+def _(codes_in, lut_in):
+    return codes_in.new_empty(codes_in.shape), codes_in.new_empty(N_BINS, dtype=torch.float32)
+
+
 @torch.library.register_fake("prime::ring_reduce_div_step")
 def _(acc, codes_in, lut_in, divisor):
     return acc.new_empty(acc.shape, dtype=torch.uint8), acc.new_empty(N_BINS, dtype=torch.float32)
@@ -290,6 +315,7 @@ dequantize_ = torch.ops.prime.dequantize_
 ring_reduce_step = torch.ops.prime.ring_reduce_step
 ring_gather_step = torch.ops.prime.ring_gather_step
 ring_reduce_div_step = torch.ops.prime.ring_reduce_div_step
+requantize_codes = torch.ops.prime.requantize_codes
 uniform_8bit_quantize_stats = torch.ops.prime.uniform_8bit_quantize_stats
 uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched
 

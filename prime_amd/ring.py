@@ -52,7 +52,8 @@ def _check_ring_inputs(tensors: Sequence[torch.Tensor]) -> int:
 
 def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
                              sources: Optional[Sequence[Tuple[torch.Tensor, torch.Tensor]]] = None,
-                             world_size: Optional[float] = None) -> None:
+                             world_size: Optional[float] = None,
+                             keep_codes: bool = False) -> Optional[List[List[Tuple[torch.Tensor, torch.Tensor]]]]:
     """The whole of ``ring_allreduce`` for ``len(tensors)`` ranks, in place, in lock step.
 
     A message posted at step s is consumed at step s + 2 (BUFFER_COUNT receive slots,
@@ -61,7 +62,14 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
     With ``sources`` = one (outer, inner) pair of flat tensors per rank, ``tensors[r]`` need not
     hold anything yet: rank r's pseudo-gradient (outer - inner) / world_size (diloco.py:93-101) is
     formed chunk by chunk in the reduce-scatter, where every chunk of a rank is visited exactly
-    once, and the result is what the all-reduce of the materialized pseudo-gradients gives."""
+    once, and the result is what the all-reduce of the materialized pseudo-gradients gives.
+
+    With ``keep_codes`` the all-gather stays in the code domain: a rank's final value of a chunk
+    is ``lut[codes]`` of the message it received (or of its own quantization), so the fp32 chunk is
+    not written; what is forwarded, ``uniform_8bit_quantize(lut[codes])`` (:215), is computed from
+    the codes alone (``ops.requantize_codes``).  Returns ``result[r][c] = (codes, lut)`` for every
+    rank r and chunk c; ``tensors`` then hold stale reduce-scatter values and the caller
+    dequantizes where it needs fp32 (``ops.dequantize_``, ``ops.outer_sgd_nesterov_codes_``)."""
     W = len(tensors)
     n = _check_ring_inputs(tensors)
     if sources is not None:
@@ -87,6 +95,7 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
                                      None if msg is None else msg[0], None if msg is None else msg[1], divisor)
 
     own: dict = {}     # (rank, chunk) -> (codes, lut) of the rank's reduced chunk, not yet written back
+    final: List[List] = [[None] * nb for _ in range(W)]
     for phase in (1, 2):
         inbox: List[dict] = [dict() for _ in range(W)]
         for step in range(1, nb + 1):
@@ -105,6 +114,12 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
                         posted.append(((r + 1) % W, step, pair[0], pair[1]))
                     else:
                         own[(r, c)] = pair
+                elif phase == 2 and keep_codes and (msg is not None or (r, c) in own):
+                    pair = msg if msg is not None else own.pop((r, c))
+                    final[r][c] = pair
+                    if sending:
+                        codes, lut = ops.requantize_codes(pair[0], pair[1])     # :215 without the fp32 chunk
+                        posted.append(((r + 1) % W, step, codes, lut))
                 elif msg is not None and sending:
                     if phase == 1:
                         codes, lut = ops.ring_reduce_step(ch, msg[0], msg[1])   # :128-138 fused
@@ -135,8 +150,12 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
                     codes, lut = touch(0, i, None, 1.0)
                 else:
                     codes, lut = ops.uniform_8bit_quantize(ch, True)        # :162 (dividing by 1 changes nothing)
-                ops.dequantize_(ch, codes, lut, False)                      # :167-172
+                if keep_codes:
+                    final[0][i] = (codes, lut)
+                else:
+                    ops.dequantize_(ch, codes, lut, False)                  # :167-172
     assert not own
+    return final if keep_codes else None
 
 
 def ring_allreduce_single(tensor: torch.Tensor, avg: bool = False) -> None:

@@ -83,6 +83,15 @@ class Abi:
         _lib.check(rc, "ring_step")
         return codes, lut, qp
 
+    def requantize_codes(self, codes_in: torch.Tensor, lut_in: torch.Tensor, codes_out: torch.Tensor = None):
+        n = codes_in.numel()
+        codes = torch.empty(n, dtype=torch.uint8, device=self.dev) if codes_out is None else codes_out
+        lut = torch.empty(256, dtype=torch.float32, device=self.dev)
+        qp = torch.empty(4, dtype=torch.float64, device=self.dev)
+        _lib.check(self.lib.prime_requantize_codes(codes_in.data_ptr(), lut_in.data_ptr(), n, codes.data_ptr(), lut.data_ptr(),
+                                                   qp.data_ptr(), self.ws.data_ptr(), self.st), "requantize_codes")
+        return codes, lut, qp
+
     def batched(self, flat: torch.Tensor, offsets: torch.Tensor):
         count = offsets.numel() - 1
         codes = torch.empty(flat.numel(), dtype=torch.uint8, device=self.dev)

@@ -264,7 +264,7 @@ def test_flat_inner_workers_with_lazy_pseudo_gradient_equal_the_plain_ones(dev, 
                 f.data.add_(delta)
         announce(f"flat-inner diloco W={W} outer step {outer}")
         step_simulated_workers(wp, plain)
-        step_simulated_workers(wf, flat)
+        step_simulated_workers(wf, flat, coded_gather=False)
         torch.cuda.synchronize()
         for mp, mf, w in zip(plain, flat, wf):
             assert w._inner_is_flat(mf)
@@ -275,6 +275,40 @@ def test_flat_inner_workers_with_lazy_pseudo_gradient_equal_the_plain_ones(dev, 
     # a model can still be used as a module: forward through the flat views
     y = flat[0].output(torch.randn(2, 64, device=dev))
     assert y.shape == (2, 256)
+
+
+@pytest.mark.parametrize("W", [1, 2, 4])
+def test_flat_inner_workers_with_coded_all_gather_track_the_plain_ones(dev, W):
+    # the fastest arrangement: lazy pseudo-gradient, all-gather in the code domain, outer step straight
+    # from codes.  Same codes everywhere; lookup entries of forwarded chunks agree to rounding only, so
+    # parameters agree to rounding except where an element crossed a bin edge
+    from prime_amd.diloco import Diloco, step_simulated_workers
+
+    torch.manual_seed(2)
+    base = TinyLlama()
+    plain = [TinyLlama().to(dev) for _ in range(W)]
+    flat = [TinyLlama().to(dev) for _ in range(W)]
+    for m in plain + flat:
+        m.load_state_dict(base.state_dict())
+    wp = [Diloco(0.7, m) for m in plain]
+    wf = [Diloco(0.7, m, flat_inner=True) for m in flat]
+    for outer in range(2):
+        gen = torch.Generator().manual_seed(300 + outer)
+        for mp, mf in zip(plain, flat):
+            for p, f in zip(mp.parameters(), mf.parameters()):
+                delta = (torch.randn(p.shape, generator=gen) * 1e-3).to(dev)
+                p.data.add_(delta)
+                f.data.add_(delta)
+        announce(f"coded diloco W={W} outer step {outer}")
+        step_simulated_workers(wp, plain)
+        step_simulated_workers(wf, flat)                  # coded_gather is the default
+        torch.cuda.synchronize()
+        for a, b, mf in zip(wp, wf, flat):
+            assert b._inner_is_flat(mf) and not b._first_step
+            assert torch.equal(b.inner_flat, b.outer_data_flat)
+            diff = (a.outer_data_flat - b.outer_data_flat).abs()
+            assert float(diff.max()) < 6e-5 and float(diff.mean()) < 3e-7
+            assert float((a.momentum_flat - b.momentum_flat).abs().max()) < 6e-5
 
 
 def test_uncompressed_simulated_all_reduce_and_fake_step(dev):

@@ -508,6 +508,88 @@ def test_ring_reduce_div_step_rejects_a_zero_or_nan_divisor(abi):
     assert bool((acc == 1).all())
 
 
+def _check_requantized(abi, oracle, codes_in, lut_in, codes, lut, qp):
+    ci, li = codes_in.cpu().numpy(), lut_in.cpu().numpy()
+    want = np.empty(ci.size, np.float32)
+    oracle.index_set(want, li, ci)                       # the chunk the reference would quantize
+    q = abi.qparams(qp)
+    assert q["n"] == ci.size
+    assert np.array_equal(np.array([q["scale"]]), np.array([oracle.scale_exact(want)]), equal_nan=True)
+    oc, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q["scale"]))
+    assert np.array_equal(codes.cpu().numpy(), oc)
+    mean, _ = oracle.average_buckets_f64(want, oc)
+    floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+    assert lut_rel_err(lut.cpu().numpy(), mean, floor) <= LUT_TOL
+
+
+@pytest.mark.parametrize("n", [1, 2, 15, 16, 17, 4097, 65536, 1 << 20, 3_000_001])
+def test_requantize_codes_equals_quantizing_the_dequantized_chunk(abi, oracle, n):
+    # uniform_8bit_quantize(lut[codes]) of the all-gather (collectives.cpp:204-215) computed from the
+    # codes alone: same scale, same codes, lookup within the bar; also against the gather step
+    rng = np.random.default_rng(n + 3)
+    src = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    if n > 1000:
+        src[rng.integers(0, n, 5)] *= 40                  # a few outliers: outer bins saturate and merge
+    announce(f"requantize codes n={n}")
+    codes_in, lut_in, _ = abi.uniform(abi.to_dev(src))
+    codes, lut, qp = abi.requantize_codes(codes_in, lut_in)
+    chunk = torch.empty(n, device=abi.dev)
+    codes2, lut2, qp2 = abi.ring_step(chunk, codes_in, lut_in, gather=True)
+    torch.cuda.synchronize()
+    _check_requantized(abi, oracle, codes_in, lut_in, codes, lut, qp)
+    assert torch.equal(codes, codes2)
+    assert abi.qparams(qp)["scale"] == abi.qparams(qp2)["scale"] or n == 1
+    a, b = lut.cpu().numpy(), lut2.cpu().numpy()
+    assert np.allclose(a, b, rtol=2e-6, atol=0, equal_nan=True)
+
+
+def test_requantize_codes_misaligned_special_values_and_foreign_tables(abi, oracle):
+    rng = np.random.default_rng(77)
+    n = 100_003
+    src = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    codes_in, lut_in, _ = abi.uniform(abi.to_dev(src))
+    # code buffers that start at odd addresses take the element-aligned kernels
+    announce("requantize codes misaligned")
+    big_in = torch.zeros(n + 32, dtype=torch.uint8, device=abi.dev)
+    big_out = torch.zeros(n + 32, dtype=torch.uint8, device=abi.dev)
+    for shift_in, shift_out in ((1, 0), (0, 3), (5, 7)):
+        vin, vout = big_in[shift_in:shift_in + n], big_out[shift_out:shift_out + n]
+        vin.copy_(codes_in)
+        big_out.fill_(9)
+        codes, lut, qp = abi.requantize_codes(vin, lut_in, vout)
+        torch.cuda.synchronize()
+        _check_requantized(abi, oracle, codes_in, lut_in, codes, lut, qp)
+        assert bool((big_out[:shift_out] == 9).all()) and bool((big_out[shift_out + n:] == 9).all())
+    # a table with an infinite and a NaN entry that occur, and garbage in entries that do not occur
+    announce("requantize codes special tables")
+    for special in (np.inf, np.nan):
+        li = lut_in.cpu().numpy().copy()
+        ci = codes_in.cpu().numpy().copy()
+        used = np.unique(ci)
+        li[used[0]] = special
+        unused = np.setdiff1d(np.arange(256), used)
+        if unused.size:
+            li[unused] = np.nan                                      # must be ignored
+        codes, lut, qp = abi.requantize_codes(abi.to_dev(ci), abi.to_dev(li))
+        torch.cuda.synchronize()
+        want = li[ci]
+        q = abi.qparams(qp)
+        assert np.array_equal(np.array([q["scale"]]), np.array([oracle.scale_exact(want)]), equal_nan=True)
+        oc, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q["scale"]))
+        assert np.array_equal(codes.cpu().numpy(), oc)
+    # all elements in one code
+    ci = np.full(5000, 200, np.uint8)
+    li = np.zeros(256, np.float32)
+    li[200] = 0.25
+    codes, lut, qp = abi.requantize_codes(abi.to_dev(ci), abi.to_dev(li))
+    torch.cuda.synchronize()
+    assert bool((codes == 171).all()) and float(lut[171]) == 0.25 and float(lut.sum()) == 0.25
+    # empty
+    codes, lut, qp = abi.requantize_codes(torch.empty(0, dtype=torch.uint8, device=abi.dev), abi.to_dev(li))
+    torch.cuda.synchronize()
+    assert codes.numel() == 0 and bool((lut == 0).all())
+
+
 def test_entry_points_replay_from_a_hip_graph(abi, oracle):
     # nothing in the library allocates, synchronises or records a memset: a sequence of calls can be
     # captured once and replayed; every replay must reproduce the eager result on fresh inputs

@@ -120,6 +120,38 @@ def test_whole_schedule_tracks_the_cpu_ring_element_by_element(dev, oracle, W, a
         assert np.abs(gpu[r].cpu().numpy() - ref_t).max() < 2.5 * bin_width
 
 
+@pytest.mark.parametrize("W,avg", [(1, False), (2, True), (4, False), (8, True)])
+def test_all_gather_in_the_code_domain_gives_the_same_tensors(dev, W, avg):
+    # keep_codes: what is forwarded is requantized from the received codes alone and the fp32 chunk is
+    # never written; a rank's result is lut[codes] of what it received.  Codes are identical to the
+    # plain schedule's; lookup entries agree to rounding, which can move an element across a bin edge
+    from prime_amd import ops, ring
+
+    n = 2 * W * 30_000
+    xs = _inputs(W, n, 200 + W)
+    plain = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    coded = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    announce(f"ring keep_codes W={W} avg={avg}")
+    ring.ring_allreduce_simulated(plain, avg=avg)
+    final = ring.ring_allreduce_simulated(coded, avg=avg, keep_codes=True)
+    torch.cuda.synchronize()
+    assert len(final) == W and all(len(f) == 2 * W for f in final)
+    bin_width = 6 * 10 * math.sqrt(W) / 256 / (W if avg else 1)
+    for r in range(W):
+        got = torch.cat([ops.dequantize(c, l) for c, l in final[r]])
+        d = (got - plain[r]).abs().cpu().numpy()
+        assert d.max() < 2.5 * bin_width
+        assert (d > 1e-2 * bin_width).mean() < 2e-3
+        for c, l in final[r]:
+            assert c.dtype == torch.uint8 and c.numel() == n // (2 * W) and l.shape == (256,)
+    # a rank's own chunks never travelled: bit-identical
+    csz = n // (2 * W)
+    for r in range(W):
+        for i in range(2):
+            c = 2 * r + i
+            assert torch.equal(ops.dequantize(*final[r][c]), plain[r][c * csz:(c + 1) * csz])
+
+
 def test_ops_layer_checks_on_device_tensors(dev):
     from prime_amd.C import compression as C
     from prime_amd import ops
