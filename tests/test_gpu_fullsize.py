@@ -114,3 +114,64 @@ def test_config4_shard_all_42_buckets(abi):
         mean = torch.where(cnt > 0, sums / cnt.clamp(min=1), torch.zeros_like(sums))
         floor = torch.tensor(float(q["scale"]), device=abi.dev, dtype=torch.float64)
         assert float(((lut.double() - mean).abs() / torch.maximum(mean.abs(), floor)).max()) <= 1e-6
+
+
+def test_all_gather_requantization_2p26_chunk_in_the_code_domain(abi):
+    # config 3's chunk: what the all-gather forwards, from codes alone, against the fp32 route
+    n = 1 << 26
+    g = torch.Generator(device=abi.dev).manual_seed(5)
+    src = torch.randn(n, device=abi.dev, generator=g) * 1e-3
+    announce("2^26 requantize codes")
+    codes_in, lut_in, _ = abi.uniform(src)
+    codes, lut, qp = abi.requantize_codes(codes_in, lut_in)
+    chunk = torch.empty(n, device=abi.dev)
+    codes2, lut2, qp2 = abi.ring_step(chunk, codes_in, lut_in, gather=True)
+    torch.cuda.synchronize()
+    assert torch.equal(chunk, lut_in[codes_in.long()])
+    assert torch.equal(codes, codes2)
+    q, q2 = abi.qparams(qp), abi.qparams(qp2)
+    assert q["scale"] == q2["scale"] and q["n"] == n
+    assert abs(q["sumsq"] - q2["sumsq"]) <= 1e-12 * q2["sumsq"]
+    assert torch.allclose(lut, lut2, rtol=1e-6, atol=0)
+    # exact population-weighted means, spelled with torch
+    cnt = torch.bincount(codes_in.int(), minlength=256).double()
+    new = torch.zeros(256, dtype=torch.float64, device=abi.dev)
+    pop = torch.zeros(256, dtype=torch.float64, device=abi.dev)
+    mapping = torch.zeros(256, dtype=torch.long, device=abi.dev)
+    mapping[codes_in.long()] = codes.long()               # a function of the old code
+    assert torch.equal(mapping[codes_in.long()], codes.long())
+    new.index_add_(0, mapping, cnt * lut_in.double())
+    pop.index_add_(0, mapping, cnt)
+    want = torch.where(pop > 0, new / pop.clamp(min=1), torch.zeros_like(new)).float()
+    assert torch.allclose(lut, want, rtol=1e-6, atol=0)
+
+
+def test_ring_first_touch_2p26_chunk_equals_separate_calls(abi):
+    from prime_amd import _lib
+
+    n = 1 << 26
+    g = torch.Generator(device=abi.dev).manual_seed(6)
+    outer = torch.randn(n, device=abi.dev, generator=g)
+    inner = outer + torch.randn(n, device=abi.dev, generator=g) * 1e-3
+    msg_c, msg_l, _ = abi.uniform(torch.randn(n, device=abi.dev, generator=g) * 1e-4)
+    for with_msg, divisor in ((False, 1.0), (True, 1.0), (True, 8.0)):
+        announce(f"2^26 first touch msg={with_msg} divisor={divisor}")
+        grad = torch.empty(n, device=abi.dev)
+        codes = torch.empty(n, dtype=torch.uint8, device=abi.dev)
+        lut = torch.empty(256, device=abi.dev)
+        qp = torch.empty(4, dtype=torch.float64, device=abi.dev)
+        _lib.check(abi.lib.prime_ring_first_touch(outer.data_ptr(), inner.data_ptr(), n, 8.0,
+                                                  msg_c.data_ptr() if with_msg else None, msg_l.data_ptr() if with_msg else None,
+                                                  divisor, grad.data_ptr(), codes.data_ptr(), lut.data_ptr(), qp.data_ptr(),
+                                                  abi.ws.data_ptr(), abi.st), "first touch")
+        want = (outer - inner) / 8.0
+        if with_msg:
+            want = want + msg_l[msg_c.long()]
+            if divisor != 1.0:
+                want = want / divisor
+        codes2, lut2, qp2 = abi.uniform(want)
+        torch.cuda.synchronize()
+        assert torch.equal(grad, want)
+        assert torch.equal(codes, codes2)
+        assert abi.qparams(qp)["scale"] == abi.qparams(qp2)["scale"]
+        assert torch.allclose(lut, lut2, rtol=1e-6, atol=0)

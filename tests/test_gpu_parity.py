@@ -607,7 +607,8 @@ def test_entry_points_replay_from_a_hip_graph(abi, oracle):
             for x, acc in zip(xs, accs):
                 c, l, qp = g_abi.uniform(x)
                 c2, l2, qp2 = g_abi.ring_step(acc, c, l)
-                res.append((c, l, qp, c2, l2, qp2))
+                c3, l3, qp3 = g_abi.requantize_codes(c2, l2)
+                res.append((c, l, qp, c2, l2, qp2, c3, l3, qp3))
             return res
 
         for x, acc in zip(xs, accs):
@@ -629,7 +630,7 @@ def test_entry_points_replay_from_a_hip_graph(abi, oracle):
         announce(f"graph replay {replay}")
         graph.replay()
         torch.cuda.synchronize()
-        for (c, l, qp, c2, l2, qp2), a, b, acc in zip(outs, hx, ha, accs):
+        for (c, l, qp, c2, l2, qp2, c3, l3, qp3), a, b, acc in zip(outs, hx, ha, accs):
             q = abi.qparams(qp)
             assert q["scale"] == oracle.scale_exact(a)
             oc, _, _ = oracle.uniform_8bit_quantize(a, "given", scale=float(q["scale"]))
@@ -640,6 +641,7 @@ def test_entry_points_replay_from_a_hip_graph(abi, oracle):
             q2 = abi.qparams(qp2)
             oc2, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q2["scale"]))
             assert q2["scale"] == oracle.scale_exact(want) and np.array_equal(c2.cpu().numpy(), oc2)
+            _check_requantized(abi, oracle, c2, l2, c3, l3, qp3)
 
 
 @pytest.mark.parametrize("shift", [0, 1, 3])
