@@ -99,6 +99,23 @@ int prime_quantize_lookup_u8(const float* x, int64_t n, float scale, uint8_t* co
 int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float* lut,
                                 prime_qparams* qparams_out, void* ws, prime_stream_t stream);
 
+/* The norm as the reference receives it from libtorch's CPU kernel at compression.cpp:113
+ * (eight serial fp32 fused-multiply-add lanes, lanes added in order, scalar tail, sqrtf: the
+ * order observed in libtorch 2.10 on x86-64 with 256-bit vectors), and the scale of :113-116
+ * derived from it.  The exact entry points above differ from this value by libtorch's
+ * accumulation error (-7e-4 relative at 2^24 elements, -3.7e-2 at 2^28).  The chains are
+ * serial, so this runs in one workgroup at about 1.9 G elements/s: a compatibility path, for
+ * bit-for-bit reproduction of the reference.  qparams_out: scale, inv_scale, n; sum is NaN and
+ * sumsq the square of the norm. */
+int prime_norm_literal_f32(const float* x, int64_t n, prime_qparams* qparams_out, void* ws,
+                           prime_stream_t stream);
+
+/* uniform_8bit_quantize with that norm: scale and codes equal the compiled reference's bit for
+ * bit; the lookup table is the fp64 bin mean (the reference's fp32 table depends on its thread
+ * count). */
+int prime_uniform_8bit_quantize_literal(const float* x, int64_t n, uint8_t* codes, float* lut,
+                                        prime_qparams* qparams_out, void* ws, prime_stream_t stream);
+
 /* Large buckets, pipelined: bucket i is quantized as prime_uniform_8bit_quantize would, on
  * streams[i % n_streams] with workspaces[i % n_streams], so that the statistics pass of one
  * bucket overlaps the quantize pass and the launch ramps of its neighbours (three streams

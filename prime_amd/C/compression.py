@@ -12,6 +12,26 @@ from .. import _lib, ops
 
 _lib.load()
 
+_NORM_MODE = "exact"
+
+
+def set_norm_mode(mode: str) -> None:
+    """How ``uniform_8bit_quantize`` obtains ``tensor.norm()`` (compression.cpp:113).
+
+    ``"exact"`` (default): the fp64 sum of squares, rounded once, at full memory bandwidth.
+    ``"libtorch"``: the fp32 value the reference actually receives from libtorch's CPU kernel
+    (eight serial lanes; 7e-4 below the exact norm at 2^24 elements, 3.7 % at 2^28), so that
+    scale and codes equal a CPU run of the reference bit for bit; the accumulation is serial by
+    definition and runs at about 1.9 G elements/s."""
+    global _NORM_MODE
+    if mode not in ("exact", "libtorch"):
+        raise ValueError("norm mode must be 'exact' or 'libtorch'")
+    _NORM_MODE = mode
+
+
+def get_norm_mode() -> str:
+    return _NORM_MODE
+
 
 def uniform_8bit_quantize(tensor: torch.Tensor, inplace: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
     """Quantize a tensor to 8-bit codes and build the 256-entry lookup table.
@@ -22,6 +42,8 @@ def uniform_8bit_quantize(tensor: torch.Tensor, inplace: bool = True) -> Tuple[t
     Returns:
         (uint8 codes shaped like ``tensor``, float32 lookup table of 256 bin means)
     """
+    if _NORM_MODE == "libtorch":
+        return ops.uniform_8bit_quantize_literal(tensor)
     return ops.uniform_8bit_quantize(tensor, inplace)
 
 

@@ -63,6 +63,8 @@ SIGNATURES = {
     "prime_uniform_8bit_quantize_batched": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp]),
     "prime_dequant_set": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp]),
     "prime_dequant_add": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp]),
+    "prime_norm_literal_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp, _vp]),
+    "prime_uniform_8bit_quantize_literal": (ctypes.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "prime_requantize_codes": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "prime_ring_reduce_step": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "prime_ring_gather_step": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),

@@ -144,8 +144,13 @@ __device__ __forceinline__ int quantize_code(float x, float inv_scale, int zero_
 // compression.cpp:113-116: std = double(norm) / sqrt(numel - 1), scale = 6 * std / 256,
 // narrowed to float at the quantizer's argument (:119).  norm() returns an fp32 tensor, so
 // the fp64 sum of squares is rounded to float once after the square root.
+__device__ __forceinline__ void finalize_from_norm(float norm, double sum, double sumsq, int64_t n, prime_qparams* qp);
+
 __device__ __forceinline__ void finalize_qparams(double sum, double sumsq, int64_t n, prime_qparams* qp) {
-    const float norm = static_cast<float>(sqrt(sumsq));
+    finalize_from_norm(static_cast<float>(sqrt(sumsq)), sum, sumsq, n, qp);
+}
+
+__device__ __forceinline__ void finalize_from_norm(float norm, double sum, double sumsq, int64_t n, prime_qparams* qp) {
     const double std_unbiased = static_cast<double>(norm) / sqrt(static_cast<double>(n - 1));
     const double scale = 6.0 * std_unbiased / 256.0;
     const float sf = static_cast<float>(scale);
@@ -277,6 +282,77 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const fl
     block_stats_store(s0 + s1, q0 + q1, ws);
 }
 
+// The norm as libtorch's CPU kernel accumulates it (the value compression.cpp:113 actually
+// receives): eight fp32 lanes, lane j taking elements j, j + 8, ... by fused multiply-add, lanes
+// added 0..7, then the n % 8 tail in order (a group of four as separately rounded products, the
+// rest by fused multiply-add) and a float square root.  The chains are serial by definition, so
+// this is one workgroup: fifteen wavefronts stage tiles in LDS, eight lanes of the first accumulate.  It exists
+// to reproduce the reference's output bit for bit; the streaming kernels compute the exact sum.
+constexpr int kLiteralTile = 8192;                       // floats per stage (two stages in LDS)
+constexpr int kLiteralRow = kLiteralTile / 8 + 8;        // lane j's elements, padded: conflict-free stores
+__global__ __launch_bounds__(kFinalThreads) void norm_literal_kernel(const float* __restrict__ x, int64_t n, Workspace* ws,
+                                                                      prime_qparams* out) {
+    // tile[buf][j * kLiteralRow + k] = element 8 k + j of the stage: lane j reads its chain in order,
+    // four elements per LDS access.  Wavefront 0 accumulates stage s while the others load stage s + 1.
+    __shared__ __attribute__((aligned(16))) float tile[2][8 * kLiteralRow];
+    const int64_t m = n - (n % 8);
+    const int64_t stages = (m + kLiteralTile - 1) / kLiteralTile;
+    auto load_stage = [&](int64_t s, int first, int step) {
+        const int64_t base = s * kLiteralTile;
+        const int count = static_cast<int>(m - base < kLiteralTile ? m - base : kLiteralTile);   // a multiple of 8
+        float* t = tile[s & 1];
+        for (int i = first; i < count; i += step) t[(i & 7) * kLiteralRow + (i >> 3)] = x[base + i];
+    };
+    float acc = 0.0f;
+    if (stages > 0) load_stage(0, threadIdx.x, kFinalThreads);
+    __syncthreads();
+    for (int64_t s = 0; s < stages; ++s) {
+        if (threadIdx.x >= 64) {
+            if (s + 1 < stages) load_stage(s + 1, threadIdx.x - 64, kFinalThreads - 64);
+        } else if (threadIdx.x < 8) {
+            const int64_t base = s * kLiteralTile;
+            const int per_lane = static_cast<int>(m - base < kLiteralTile ? m - base : kLiteralTile) >> 3;
+            const float* t = tile[s & 1] + threadIdx.x * kLiteralRow;
+            int k = 0;
+            for (; k + 16 <= per_lane; k += 16) {
+                f4a v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f4a*>(t + k + 4 * u);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    acc = __builtin_fmaf(v[u].x, v[u].x, acc);
+                    acc = __builtin_fmaf(v[u].y, v[u].y, acc);
+                    acc = __builtin_fmaf(v[u].z, v[u].z, acc);
+                    acc = __builtin_fmaf(v[u].w, v[u].w, acc);
+                }
+            }
+            for (; k < per_lane; ++k) acc = __builtin_fmaf(t[k], t[k], acc);
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x < 64) {
+        float total = __shfl(acc, 0, 64);
+#pragma unroll
+        for (int j = 1; j < 8; ++j) total += __shfl(acc, j, 64);
+        if (threadIdx.x == 0) {
+            int64_t i = m;
+            if (n - i >= 4) {
+                for (int k = 0; k < 4; ++k) {
+                    const float sq = x[i + k] * x[i + k];     // rounded on its own (contraction is off)
+                    total += sq;
+                }
+                i += 4;
+            }
+            for (; i < n; ++i) total = __builtin_fmaf(x[i], x[i], total);
+            const float norm = __builtin_sqrtf(total);
+            prime_qparams qp;
+            finalize_from_norm(norm, __builtin_nan(""), static_cast<double>(norm) * static_cast<double>(norm), n, &qp);
+            ws->qp = qp;
+            if (out) *out = qp;
+        }
+    }
+}
+
 // LDS histogram: R copies of each bin, chosen by lane, so that lanes of one wavefront that
 // hit the same bin mostly hit different addresses (and banks).  Sums are fp64, counts u32
 // (a workgroup never sees 2^32 elements: n is capped at 2^40 and the grid is at least one
@@ -321,7 +397,10 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
     __shared__ LdsHist<HIST ? R : 1> hist;
     if (HIST) hist_zero(hist);
     // the scale: given by value, or derived here from the statistics partials of the pass before
-    const float inv = stats_parts > 0 ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out) : 1.0f / scale_val;
+    // (stats_parts < 0: the record a preceding kernel left in the workspace)
+    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out)
+                      : stats_parts < 0 ? ws->qp.inv_scale
+                                        : 1.0f / scale_val;
     if (HIST) __syncthreads();
     const int64_t nvec = n >> 2;
     sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
@@ -1121,13 +1200,13 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouch, kIdFirstTouchCodes, kIdCodeCount, kIdCodeTotal, kIdRequantPlan, kIdCodeRemap, kIdCount
+    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouch, kIdFirstTouchCodes, kIdCodeCount, kIdCodeTotal, kIdRequantPlan, kIdCodeRemap, kIdNormLiteral, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
     "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
     "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>", "div_kernel",
-    "first_touch_kernel", "first_touch_kernel<codes>", "code_count_kernel", "code_total_kernel", "requant_plan_kernel", "code_remap_kernel"};
+    "first_touch_kernel", "first_touch_kernel<codes>", "code_count_kernel", "code_total_kernel", "requant_plan_kernel", "code_remap_kernel", "norm_literal_kernel"};
 
 struct TimedLaunch {
     int id;
@@ -1423,6 +1502,26 @@ int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float
     int parts = 0, grid = 0;
     if (int rc = run_stats_partials(x, n, w, st, &parts)) return rc;
     if (int rc = run_quantize(x, n, 0.0f, parts, qparams_out, kZeroPoint, codes, w, true, st, &grid)) return rc;
+    return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
+}
+
+int prime_norm_literal_f32(const float* x, int64_t n, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
+    if (bad_n(n) || (n > 0 && !x)) return fail(PRIME_EINVAL, "prime_norm_literal_f32: bad argument");
+    if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
+    launch(kIdNormLiteral, 4.0 * n, norm_literal_kernel, 1, kFinalThreads, static_cast<hipStream_t>(stream), x, n,
+           static_cast<Workspace*>(ws), qparams_out);
+    return launch_check("norm_literal_kernel");
+}
+
+int prime_uniform_8bit_quantize_literal(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out,
+                                        void* ws, prime_stream_t stream) {
+    if (bad_n(n) || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_literal: bad argument");
+    if (int rc = prime_norm_literal_f32(x, n, qparams_out, ws, stream)) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Workspace* w = static_cast<Workspace*>(ws);
+    int grid = 0;
+    if (n > 0)
+        if (int rc = run_quantize(x, n, 0.0f, -1, nullptr, kZeroPoint, codes, w, true, st, &grid)) return rc;
     return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
 }
 

@@ -12,6 +12,7 @@ Schemas mirror the Python signatures of the reference's wrappers
     prime::ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
     prime::ring_gather_step(Tensor(a!) chunk, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
     prime::requantize_codes(Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)
+    prime::uniform_8bit_quantize_literal(Tensor tensor) -> (Tensor, Tensor)
     prime::ring_reduce_div_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in, float divisor) -> (Tensor, Tensor)
     prime::uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)
     prime::uniform_8bit_quantize_batched(Tensor flat, Tensor offsets) -> (Tensor, Tensor, Tensor)
@@ -41,6 +42,7 @@ _LIB.define("dequantize(Tensor codes, Tensor lut) -> Tensor")
 _LIB.define("dequantize_(Tensor(a!) out, Tensor codes, Tensor lut, bool accumulate) -> ()")
 _LIB.define("ring_reduce_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
 _LIB.define("ring_gather_step(Tensor(a!) chunk, Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
+_LIB.define("uniform_8bit_quantize_literal(Tensor tensor) -> (Tensor, Tensor)")
 _LIB.define("requantize_codes(Tensor codes_in, Tensor lut_in) -> (Tensor, Tensor)")
 _LIB.define("ring_reduce_div_step(Tensor(a!) acc, Tensor codes_in, Tensor lut_in, float divisor) -> (Tensor, Tensor)")
 _LIB.define("uniform_8bit_quantize_stats(Tensor tensor) -> (Tensor, Tensor, Tensor)")
@@ -92,9 +94,19 @@ def _uniform_8bit_quantize(tensor: torch.Tensor, inplace: bool = True):
     return codes, lut
 
 
+def _uniform_8bit_quantize_literal(tensor: torch.Tensor):
+    """uniform_8bit_quantize with the norm accumulated as libtorch's CPU kernel does it, so that
+    scale and codes are the reference's bit for bit (compression.cpp:113); slow by design."""
+    return _uniform_8bit_quantize_with(tensor, True)[:2]
+
+
 def _uniform_8bit_quantize_stats(tensor: torch.Tensor):
     """(codes, lut, qparams): qparams is the 32-byte ``prime_qparams`` record as 4 float64
     words; view it with ``unpack_qparams``."""
+    return _uniform_8bit_quantize_with(tensor, False)
+
+
+def _uniform_8bit_quantize_with(tensor: torch.Tensor, literal: bool):
     _need_f32(tensor, "uniform_8bit_quantize")
     lib = _lib.load()
     x = tensor.contiguous()
@@ -104,10 +116,9 @@ def _uniform_8bit_quantize_stats(tensor: torch.Tensor):
         lut = torch.empty(N_BINS, dtype=torch.float32, device=dev)
         qp = torch.empty(4, dtype=torch.float64, device=dev)
         ws = workspace(dev)
-        _lib.check(
-            lib.prime_uniform_8bit_quantize(x.data_ptr(), x.numel(), codes.data_ptr(), lut.data_ptr(), qp.data_ptr(),
-                                            ws.data_ptr(), _stream(dev)),
-            "prime_uniform_8bit_quantize")
+        fn = lib.prime_uniform_8bit_quantize_literal if literal else lib.prime_uniform_8bit_quantize
+        _lib.check(fn(x.data_ptr(), x.numel(), codes.data_ptr(), lut.data_ptr(), qp.data_ptr(), ws.data_ptr(), _stream(dev)),
+                   "prime_uniform_8bit_quantize")
     return codes, lut, qp
 
 
@@ -253,6 +264,7 @@ _LIB.impl("dequantize", _dequantize, "CUDA")
 _LIB.impl("dequantize_", _dequantize_, "CUDA")
 _LIB.impl("ring_reduce_step", _ring_reduce_step, "CUDA")
 _LIB.impl("ring_gather_step", _ring_gather_step, "CUDA")
+_LIB.impl("uniform_8bit_quantize_literal", _uniform_8bit_quantize_literal, "CUDA")
 _LIB.impl("requantize_codes", _requantize_codes, "CUDA")
 _LIB.impl("ring_reduce_div_step", _ring_reduce_div_step, "CUDA")
 _LIB.impl("uniform_8bit_quantize_stats", _uniform_8bit_quantize_stats, "CUDA")
@@ -290,6 +302,11 @@ def _(chunk, codes_in, lut_in):
     return chunk.new_empty(chunk.shape, dtype=torch.uint8), chunk.new_empty(N_BINS, dtype=torch.float32)
 
 
+@torch.library.register_fake("prime::uniform_8bit_quantize_literal")
+def _(tensor):
+    return tensor.new_empty(tensor.shape, dtype=torch.uint8), tensor.new_empty(N_BINS, dtype=torch.float32)
+
+
 @torch.library.register_fake("prime::requantize_codes")
 def _(codes_in, lut_in):
     return codes_in.new_empty(codes_in.shape), codes_in.new_empty(N_BINS, dtype=torch.float32)
@@ -316,6 +333,7 @@ ring_reduce_step = torch.ops.prime.ring_reduce_step
 ring_gather_step = torch.ops.prime.ring_gather_step
 ring_reduce_div_step = torch.ops.prime.ring_reduce_div_step
 requantize_codes = torch.ops.prime.requantize_codes
+uniform_8bit_quantize_literal = torch.ops.prime.uniform_8bit_quantize_literal
 uniform_8bit_quantize_stats = torch.ops.prime.uniform_8bit_quantize_stats
 uniform_8bit_quantize_batched = torch.ops.prime.uniform_8bit_quantize_batched
 

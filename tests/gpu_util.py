@@ -36,6 +36,15 @@ class Abi:
                                                         self.ws.data_ptr(), self.st), "uniform")
         return codes, lut, qp
 
+    def uniform_literal(self, x: torch.Tensor):
+        n = x.numel()
+        codes = torch.empty(n, dtype=torch.uint8, device=self.dev)
+        lut = torch.empty(256, dtype=torch.float32, device=self.dev)
+        qp = torch.empty(4, dtype=torch.float64, device=self.dev)
+        _lib.check(self.lib.prime_uniform_8bit_quantize_literal(x.data_ptr(), n, codes.data_ptr(), lut.data_ptr(), qp.data_ptr(),
+                                                                self.ws.data_ptr(), self.st), "uniform_literal")
+        return codes, lut, qp
+
     def quantize_lookup(self, x: torch.Tensor, scale: float):
         n = x.numel()
         codes = torch.empty(n, dtype=torch.uint8, device=self.dev)

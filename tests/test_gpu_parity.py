@@ -335,6 +335,10 @@ def test_golden_fixtures_of_the_compiled_reference(abi, oracle, golden, name):
         assert lut_rel_err(lut.cpu().numpy(), golden[f"{key}/lut"].astype(np.float64), ref_scale) < 2e-5
         mean, _ = oracle.average_buckets_f64(x, golden[f"{key}/codes"])
         assert lut_rel_err(lut.cpu().numpy(), mean, ref_scale) <= LUT_TOL
+    # the libtorch-order norm on the GPU: scale and codes are the reference's, bit for bit, end to end
+    codes, lut, qp = abi.uniform_literal(xt)
+    assert np.array_equal(np.array([abi.qparams(qp)["scale"]]), golden[f"{key}/scale"], equal_nan=True)
+    assert np.array_equal(codes.cpu().numpy(), golden[f"{key}/codes"])
     # end to end with the GPU's own scale
     codes, lut, qp = abi.uniform(xt)
     q = abi.qparams(qp)
@@ -351,6 +355,50 @@ def test_golden_fixtures_of_the_compiled_reference(abi, oracle, golden, name):
     else:
         assert np.array_equal(np.array([q["scale"]]), golden[f"{key}/scale"], equal_nan=True)
         assert np.array_equal(codes.cpu().numpy(), golden[f"{key}/codes"])
+
+
+@pytest.mark.parametrize("n", list(range(1, 40)) + [4097, 16384, 16385, 100_003, (1 << 20) + 7, 1 << 24])
+def test_literal_norm_is_libtorch_order_bit_for_bit(abi, oracle, n):
+    # the norm as the reference receives it from libtorch (compression.cpp:113): the oracle's emulation
+    # is pinned against torch itself on the CPU; the GPU kernel must give the same float at every size
+    # (vector body, lane sum, both kinds of tail, several 64 KiB tiles)
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    announce(f"literal norm n={n}")
+    codes, lut, qp = abi.uniform_literal(abi.to_dev(x))
+    torch.cuda.synchronize()
+    q = abi.qparams(qp)
+    want_scale = oracle.scale_literal(x)
+    assert np.array_equal(np.array([q["scale"]]), np.array([want_scale]), equal_nan=True), (q["scale"], want_scale)
+    assert q["n"] == n and np.isnan(q["sum"])
+    assert np.float32(np.sqrt(q["sumsq"])) == oracle.norm_literal(x)
+    oc, _, _ = oracle.uniform_8bit_quantize(x, "literal")
+    assert np.array_equal(codes.cpu().numpy(), oc)
+    if np.isfinite(want_scale) and want_scale > 0:
+        mean, _ = oracle.average_buckets_f64(x, oc)
+        assert lut_rel_err(lut.cpu().numpy(), mean, float(want_scale)) <= LUT_TOL
+
+
+def test_literal_norm_against_the_compiled_reference_at_2p24(abi, oracle):
+    # BASELINE config 1 as the reference itself computes it: same scale, same codes, every element
+    if not oracle.ref_available():
+        pytest.skip("oracle/_ref is not built")
+    import torch as _t
+
+    n = 1 << 24
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    ref_codes, ref_lut = oracle.ref().uniform_8bit_quantize(_t.from_numpy(x), False)
+    announce("literal 2^24 against the compiled reference")
+    codes, lut, qp = abi.uniform_literal(abi.to_dev(x))
+    torch.cuda.synchronize()
+    assert np.array_equal(codes.cpu().numpy(), ref_codes.numpy())
+    q = abi.qparams(qp)
+    assert lut_rel_err(lut.cpu().numpy(), ref_lut.numpy().astype(np.float64), float(q["scale"])) < 2e-5
+    # and the exact path differs from it by libtorch's accumulation error only
+    _, _, qp_exact = abi.uniform(abi.to_dev(x))
+    rel = float(q["scale"]) / float(abi.qparams(qp_exact)["scale"]) - 1
+    assert -2e-3 < rel < -1e-4
 
 
 def test_results_do_not_depend_on_scheduling(abi):

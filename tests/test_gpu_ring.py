@@ -179,6 +179,29 @@ def test_ops_layer_checks_on_device_tensors(dev):
     assert torch.equal(d, l1[c1.long()])
 
 
+def test_norm_mode_switch_of_the_compression_module(dev, oracle):
+    # set_norm_mode("libtorch"): uniform_8bit_quantize gives the scale-dependent codes of a CPU run of the
+    # reference (oracle in literal mode, itself pinned against torch's norm and the compiled reference)
+    from prime_amd.C import compression as C
+
+    rng = np.random.default_rng(12)
+    x = (rng.standard_normal(3_000_003) * 1e-3).astype(np.float32)
+    t = torch.from_numpy(x).to(dev)
+    assert C.get_norm_mode() == "exact"
+    announce("norm mode switch")
+    try:
+        C.set_norm_mode("libtorch")
+        c_lit, _ = C.uniform_8bit_quantize(t)
+    finally:
+        C.set_norm_mode("exact")
+    c_exact, _ = C.uniform_8bit_quantize(t)
+    assert np.array_equal(c_lit.cpu().numpy(), oracle.uniform_8bit_quantize(x, "literal")[0])
+    assert np.array_equal(c_exact.cpu().numpy(), oracle.uniform_8bit_quantize(x, "exact")[0])
+    assert not torch.equal(c_lit, c_exact)          # libtorch's norm is off by 1e-4 here: a few codes move
+    with pytest.raises(ValueError):
+        C.set_norm_mode("fast")
+
+
 def test_div_kernel_is_fp32_division(dev, oracle):
     # chunk.div_(world_size) of ReduceOp::AVG (collectives.cpp:155-159)
     from prime_amd import ops
