@@ -375,6 +375,63 @@ __device__ __forceinline__ void hist_add(LdsHist<R>& h, int code, float x) {
     __hip_atomic_fetch_add(&h.cnt[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
+// Register-side accumulators for a tensor whose values crowd into a few codes (a constant, or
+// weights near 1 whose spread is a fraction of a bin): LDS atomics of a wavefront on one address
+// serialize, so the three codes around the code of the mean are summed per lane and reach LDS
+// once per wavefront.  Used only when the statistics say the tensor is that narrow.
+struct HotCodes {
+    int base;                 // hot codes are base, base + 1, base + 2
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0;
+    unsigned c0 = 0, c1 = 0, c2 = 0;
+};
+
+template <int R>
+__device__ __forceinline__ void hist_add_hot(LdsHist<R>& h, HotCodes& hot, int code, float x) {
+    const unsigned d = static_cast<unsigned>(code - hot.base);
+    if (d < 3u) {
+        const double v = x;
+        hot.s0 += d == 0 ? v : 0.0;
+        hot.s1 += d == 1 ? v : 0.0;
+        hot.s2 += d == 2 ? v : 0.0;
+        hot.c0 += d == 0;
+        hot.c1 += d == 1;
+        hot.c2 += d == 2;
+    } else {
+        hist_add(h, code, x);
+    }
+}
+
+// Every lane of the wavefront must call this (it shuffles); lane 0 adds the wavefront's totals.
+template <int R>
+__device__ __forceinline__ void hist_flush_hot(LdsHist<R>& h, const HotCodes& hot) {
+    const double s[3] = {wave_sum(hot.s0), wave_sum(hot.s1), wave_sum(hot.s2)};
+    unsigned c[3] = {hot.c0, hot.c1, hot.c2};
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) c[k] += __shfl_down(c[k], off, 64);
+    if ((threadIdx.x & 63) == 0) {
+        const int rep = (threadIdx.x >> 6) & (R - 1);
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const int code = hot.base + k;
+            if (c[k] && code >= 0 && code < kBins) {
+                __hip_atomic_fetch_add(&h.sum[code * R + rep], s[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&h.cnt[code * R + rep], c[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+    }
+}
+
+// True when the tensor's spread is below about two bins: std < 0.05 rms, from the fp64 sums.
+__device__ __forceinline__ bool narrow_distribution(double sum, double sumsq, int64_t n) {
+    if (n < 2) return false;
+    const double mean = sum / static_cast<double>(n);
+    const double ms = sumsq / static_cast<double>(n);
+    const double var = ms - mean * mean;
+    return var * 400.0 <= ms;            // also true for an all-zero tensor; false when a sum is NaN
+}
+
 // Store the workgroup's histogram (copies added in a fixed order) as its partial: one
 // 16-byte store per lane, 4 KiB contiguous per workgroup.
 template <int R>
@@ -823,6 +880,7 @@ __global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __r
     __shared__ double sh_s[kBatchThreads / 64];
     __shared__ double sh_q[kBatchThreads / 64];
     __shared__ prime_qparams sh_qp;
+    __shared__ int sh_hot_base;          // >= -1: the tensor is narrow, hot codes start here; INT_MIN: it is not
     const int64_t t = blockIdx.x;
     const int64_t lo = offsets[t];
     const int64_t hi = offsets[t + 1];
@@ -868,10 +926,21 @@ __global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __r
         for (int w = 1; w < kBatchThreads / 64; ++w) { S += sh_s[w]; Q += sh_q[w]; }
         finalize_qparams(S, Q, n, &sh_qp);
         if (qps) qps[t] = sh_qp;
+        sh_hot_base = narrow_distribution(S, Q, n)
+                          ? quantize_code(static_cast<float>(S / static_cast<double>(n)), sh_qp.inv_scale, kZeroPoint) - 1
+                          : INT_MIN;
     }
     __syncthreads();
     const float inv = sh_qp.inv_scale;
     uint32_t* __restrict__ c4 = reinterpret_cast<uint32_t*>(codes);
+    auto second_pass = [&](auto narrow_t) {
+    constexpr bool narrow = decltype(narrow_t)::value;
+    HotCodes hot;
+    hot.base = sh_hot_base;
+    auto add = [&](int code, float xv) {
+        if (narrow) hist_add_hot(hist, hot, code, xv);
+        else hist_add(hist, code, xv);
+    };
     for (int64_t v0 = (a >> 2) + threadIdx.x; v0 < (b >> 2); v0 += kBatchThreads * U) {
         f4a v[U];
 #pragma unroll
@@ -889,10 +958,10 @@ __global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __r
                 const int cd = quantize_code(v[j].w, inv, kZeroPoint);
                 c4[i] = static_cast<uint32_t>(ca) | (static_cast<uint32_t>(cb) << 8) | (static_cast<uint32_t>(cc) << 16) |
                         (static_cast<uint32_t>(cd) << 24);
-                hist_add(hist, ca, v[j].x);
-                hist_add(hist, cb, v[j].y);
-                hist_add(hist, cc, v[j].z);
-                hist_add(hist, cd, v[j].w);
+                add(ca, v[j].x);
+                add(cb, v[j].y);
+                add(cc, v[j].z);
+                add(cd, v[j].w);
             }
         }
     }
@@ -902,9 +971,13 @@ __global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __r
             const float v = x[i];
             const int c = quantize_code(v, inv, kZeroPoint);
             codes[i] = static_cast<uint8_t>(c);
-            hist_add(hist, c, v);
+            add(c, v);
         }
     }
+    if (narrow) hist_flush_hot(hist, hot);
+    };
+    if (sh_hot_base != INT_MIN) second_pass(std::true_type{});
+    else second_pass(std::false_type{});
     __syncthreads();
     for (int bin = threadIdx.x; bin < kBins; bin += kBatchThreads) {
         double sum = 0.0;
