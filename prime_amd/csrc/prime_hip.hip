@@ -180,15 +180,26 @@ __device__ __forceinline__ void block_stats_store(double s, double q, Workspace*
     }
 }
 
+// True when the tensor's spread is below about two bins: std < 0.05 rms, from the fp64 sums.
+__device__ __forceinline__ bool narrow_distribution(double sum, double sumsq, int64_t n) {
+    if (n < 2) return false;
+    const double mean = sum / static_cast<double>(n);
+    const double ms = sumsq / static_cast<double>(n);
+    const double var = ms - mean * mean;
+    return var * 400.0 <= ms;            // also true for an all-zero tensor; false when a sum is NaN
+}
+
 // Second stage of the statistics run by a whole workgroup of the consuming kernel: every
 // workgroup adds the same partials in the same order, so all of them derive the same scale
 // bit for bit and no separate launch is needed.  Returns 1 / scale; workgroup 0 publishes
 // the record.
 template <int THREADS>
-__device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int nparts, int64_t n, prime_qparams* out) {
+__device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
+                                                           int* hot_base = nullptr) {
     __shared__ double sh_s[THREADS / 64];
     __shared__ double sh_q[THREADS / 64];
     __shared__ float sh_inv;
+    __shared__ int sh_hot;
     constexpr int kIters = (kMaxGrid + THREADS - 1) / THREADS;
     double ps[kIters], pq[kIters];
 #pragma unroll
@@ -212,12 +223,15 @@ __device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int np
         prime_qparams qp;
         finalize_qparams(S, Q, n, &qp);
         sh_inv = qp.inv_scale;
+        sh_hot = narrow_distribution(S, Q, n) ? quantize_code(static_cast<float>(S / static_cast<double>(n)), qp.inv_scale, kZeroPoint) - 1
+                                              : INT_MIN;
         if (blockIdx.x == 0) {
             ws->qp = qp;
             if (out) *out = qp;
         }
     }
     __syncthreads();
+    if (hot_base) *hot_base = sh_hot;
     return sh_inv;
 }
 
@@ -423,15 +437,6 @@ __device__ __forceinline__ void hist_flush_hot(LdsHist<R>& h, const HotCodes& ho
     }
 }
 
-// True when the tensor's spread is below about two bins: std < 0.05 rms, from the fp64 sums.
-__device__ __forceinline__ bool narrow_distribution(double sum, double sumsq, int64_t n) {
-    if (n < 2) return false;
-    const double mean = sum / static_cast<double>(n);
-    const double ms = sumsq / static_cast<double>(n);
-    const double var = ms - mean * mean;
-    return var * 400.0 <= ms;            // also true for an all-zero tensor; false when a sum is NaN
-}
-
 // Store the workgroup's histogram (copies added in a fixed order) as its partial: one
 // 16-byte store per lane, 4 KiB contiguous per workgroup.
 template <int R>
@@ -455,45 +460,58 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
     if (HIST) hist_zero(hist);
     // the scale: given by value, or derived here from the statistics partials of the pass before
     // (stats_parts < 0: the record a preceding kernel left in the workspace)
-    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out)
+    int hot_base = INT_MIN;              // set when the statistics show a tensor crowded into a few codes
+    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &hot_base)
                       : stats_parts < 0 ? ws->qp.inv_scale
                                         : 1.0f / scale_val;
     if (HIST) __syncthreads();
     const int64_t nvec = n >> 2;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
-        constexpr bool full = decltype(full_t)::value;
-        f4a v[kUnroll];
+    auto pass = [&](auto narrow_t) {
+        constexpr bool narrow = decltype(narrow_t)::value;
+        HotCodes hot;
+        hot.base = hot_base;
+        auto add = [&](int code, float xv) {
+            if (narrow) hist_add_hot(hist, hot, code, xv);
+            else hist_add(hist, code, xv);
+        };
+        sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+            constexpr bool full = decltype(full_t)::value;
+            f4a v[kUnroll];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = i0 + j * stride;
-            v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
-        }
+            for (int j = 0; j < kUnroll; ++j) {
+                const int64_t i = i0 + j * stride;
+                v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            }
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
-            const int64_t i = i0 + j * stride;
-            if (full || i < nvec) {
-                const int a = quantize_code(v[j].x, inv, zero_point);
-                const int b = quantize_code(v[j].y, inv, zero_point);
-                const int c = quantize_code(v[j].z, inv, zero_point);
-                const int d = quantize_code(v[j].w, inv, zero_point);
-                M::stu32(codes, i, static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) |
-                                       (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24));
-                if (HIST) {
-                    hist_add(hist, a, v[j].x);
-                    hist_add(hist, b, v[j].y);
-                    hist_add(hist, c, v[j].z);
-                    hist_add(hist, d, v[j].w);
+            for (int j = 0; j < kUnroll; ++j) {
+                const int64_t i = i0 + j * stride;
+                if (full || i < nvec) {
+                    const int a = quantize_code(v[j].x, inv, zero_point);
+                    const int b = quantize_code(v[j].y, inv, zero_point);
+                    const int c = quantize_code(v[j].z, inv, zero_point);
+                    const int d = quantize_code(v[j].w, inv, zero_point);
+                    M::stu32(codes, i, static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) |
+                                           (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24));
+                    if (HIST) {
+                        add(a, v[j].x);
+                        add(b, v[j].y);
+                        add(c, v[j].z);
+                        add(d, v[j].w);
+                    }
                 }
             }
+        });
+        if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+            const int64_t i = (nvec << 2) + threadIdx.x;
+            const float v = x[i];
+            const int a = quantize_code(v, inv, zero_point);
+            codes[i] = static_cast<uint8_t>(a);
+            if (HIST) add(a, v);
         }
-    });
-    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
-        const int64_t i = (nvec << 2) + threadIdx.x;
-        const float v = x[i];
-        const int a = quantize_code(v, inv, zero_point);
-        codes[i] = static_cast<uint8_t>(a);
-        if (HIST) hist_add(hist, a, v);
-    }
+        if (HIST && narrow) hist_flush_hot(hist, hot);
+    };
+    if (HIST && hot_base != INT_MIN) pass(std::true_type{});
+    else pass(std::false_type{});
     if (HIST) {
         __syncthreads();
         hist_store(hist, ws);
