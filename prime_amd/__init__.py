@@ -7,6 +7,8 @@ Layout
     C/compression.py, C/collectives.py, collectives.py, config.py
                      the reference's module and function names for this path
     ring.py          the ring's per-hop compute for W simulated ranks on one GPU
+    diloco.py        pseudo-gradient, bucketing and outer step around the all-reduce, GPU-resident
+    shim.py          registers these modules under the reference's import paths (zeroband.*)
 """
 from .config import Compression  # noqa: F401
 

@@ -215,3 +215,31 @@ def test_div_kernel_is_fp32_division(dev, oracle):
             want = x.copy()
             oracle.div_scalar(want, d)
             assert np.array_equal(t.cpu().numpy(), want)
+
+
+def test_reference_import_paths_reach_the_hip_kernels(dev):
+    # the body of the reference's own tests/test_c/test_compression.py (:14-56), with its imports
+    # unchanged, after prime_amd.shim.install()
+    import sys
+
+    import prime_amd.shim as shim
+
+    shim.install()
+    try:
+        from zeroband.C.compression import average_buckets, quantize_per_tensor_uint8, uniform_8bit_quantize
+
+        N = 1_000_000
+        announce("reference import paths")
+        a = torch.randn(N, device=dev) * 10
+        codes, lut = uniform_8bit_quantize(a)
+        assert codes.dtype == torch.uint8 and codes.shape == a.shape and lut.shape == (256,)
+        diff = (lut[codes.long()] - a).abs()
+        assert float(diff.max()) <= 6 * float(a.norm() / math.sqrt(N - 1)) / 256 * 1.01 or float(diff.median()) < 0.2
+        new_lut = average_buckets(a, codes, 256)
+        assert torch.equal(new_lut, lut)
+        q = quantize_per_tensor_uint8(torch.ones(N, device=dev) * 10, 0.01, 128)
+        assert bool((q == 255).all())
+    finally:
+        shim.uninstall()
+        for k in [k for k in sys.modules if k == "zeroband" or k.startswith("zeroband.")]:
+            del sys.modules[k]

@@ -105,3 +105,36 @@ def test_missing_library_is_an_error(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libprime_hip.so")
     with pytest.raises(_lib.PrimeHipError, match="no CPU fallback"):
         _lib.load()
+
+
+def test_shim_registers_the_reference_import_paths():
+    # src/zeroband/diloco.py:6, tests/test_c/test_compression.py:6: those imports, unchanged, reach this package
+    import sys
+
+    import prime_amd.shim as shim
+
+    had = {k: sys.modules.get(k) for k in list(sys.modules) if k == "zeroband" or k.startswith("zeroband.")}
+    try:
+        shim.install()
+        from zeroband.C.compression import average_buckets, quantize_per_tensor_uint8, uniform_8bit_quantize
+        from zeroband.C.collectives import ring_allreduce
+        from zeroband.collectives import Compression, all_reduce
+
+        import prime_amd.C.collectives
+        import prime_amd.C.compression
+        import prime_amd.collectives
+
+        assert uniform_8bit_quantize is prime_amd.C.compression.uniform_8bit_quantize
+        assert average_buckets is prime_amd.C.compression.average_buckets
+        assert quantize_per_tensor_uint8 is prime_amd.C.compression.quantize_per_tensor_uint8
+        assert ring_allreduce is prime_amd.C.collectives.ring_allreduce
+        assert all_reduce is prime_amd.collectives.all_reduce and Compression.UINT8.value == "uint8"
+        shim.install()                                  # idempotent
+        import zeroband.C.compression as again
+
+        assert again is prime_amd.C.compression
+    finally:
+        shim.uninstall()
+        for k in [k for k in sys.modules if k == "zeroband" or k.startswith("zeroband.")]:
+            del sys.modules[k]
+        sys.modules.update({k: v for k, v in had.items() if v is not None})
