@@ -47,6 +47,7 @@ constexpr int kBins = 256;               // compression.cpp:5
 constexpr int kZeroPoint = 128;          // compression.cpp:107
 constexpr int kMaxGrid = 2048;           // per-workgroup partial slots in the workspace
 constexpr int kUnroll = PRIME_UNROLL;
+constexpr int kDivUnroll = PRIME_UNROLL > 2 ? 2 : PRIME_UNROLL;   // vectors per step in the kernels that divide
 // wavefronts per SIMD the streaming kernels are compiled for (4 SIMDs per compute unit, at
 // most 8 wavefronts each): bounds their register use so that PRIME_BLOCKS_PER_CU workgroups fit
 constexpr int kWavesPerSimd = (PRIME_THREADS / 64) * PRIME_BLOCKS_PER_CU / 4 > 8 ? 8
@@ -248,16 +249,18 @@ __global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace
 // as one sliding window of contiguous 64 KiB pieces and every access of the main part is
 // unguarded.  Tail (fewer than G tiles): single rows dealt round-robin, so no workgroup
 // streams more than one row beyond the average.  body(i0, stride, full) handles the kUnroll
-// vectors i0 + j * stride of the calling lane; `full` is a compile-time flag (true_type in the
+// vectors i0 + j * stride (j < U) of the calling lane; `full` is a compile-time flag (true_type in the
 // main part): unless it is set, each vector needs the check i < nvec.
-template <typename Body>
+// U is the number of vectors body handles per call (kUnroll unless the kernel needs the registers:
+// the kernels that divide keep two operands per vector and a division sequence live).
+template <int U = kUnroll, typename Body>
 __device__ __forceinline__ void sweep(int64_t nvec, Body&& body) {
     const int64_t G = gridDim.x;
     const int64_t rows = (nvec + kThreads - 1) / kThreads;
-    const int64_t rounds = (nvec / kThreads) / (G * kUnroll);
+    const int64_t rounds = (nvec / kThreads) / (G * U);
     for (int64_t k = 0; k < rounds; ++k)
-        body(((k * G + blockIdx.x) * kUnroll) * kThreads + threadIdx.x, static_cast<int64_t>(kThreads), std::true_type{});
-    const int64_t r0 = rounds * G * kUnroll + blockIdx.x;
+        body(((k * G + blockIdx.x) * U) * kThreads + threadIdx.x, static_cast<int64_t>(kThreads), std::true_type{});
+    const int64_t r0 = rounds * G * U + blockIdx.x;
     if (r0 < rows) body(r0 * kThreads + threadIdx.x, G * kThreads, std::false_type{});
 }
 
@@ -838,20 +841,21 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float*
     for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
     __syncthreads();
     const int64_t nvec = n >> 2;
+    constexpr int U = DIV ? kDivUnroll : kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
-        uint32_t c[kUnroll];
-        f4a a[kUnroll];
+        uint32_t c[U];
+        f4a a[U];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             const bool ok = full || i < nvec;
             c[j] = ok ? M::ldu32(codes, i) : 0u;
             if (ADD) a[j] = ok ? M::ldf4(out, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             f4a v;
             v.x = s_lut[c[j] & 255];
@@ -1017,16 +1021,17 @@ template <bool ALIGNED>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void div_kernel(float* __restrict__ x, int64_t n, float d) {
     using M = Mem<ALIGNED, false>;
     const int64_t nvec = n >> 2;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    constexpr int U = kDivUnroll;
+    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
-        f4a v[kUnroll];
+        f4a v[U];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             if (full || i < nvec) M::stf4(x, i, v[j] / d, false);
         }
@@ -1047,18 +1052,19 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void pseudo_gradient_kerne
                                                                                    float world_size, float* __restrict__ out) {
     using M = Mem<ALIGNED, false>;
     const int64_t nvec = n >> 2;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    constexpr int U = kDivUnroll;
+    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
-        f4a a[kUnroll], b[kUnroll];
+        f4a a[U], b[U];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             const bool ok = full || i < nvec;
             a[j] = ok ? M::ldf4(outer, i) : f4a{0.f, 0.f, 0.f, 0.f};
             b[j] = ok ? M::ldf4(inner, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             if (full || i < nvec) M::stf4(out, i, (a[j] - b[j]) / world_size, false);
         }
@@ -1090,13 +1096,14 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
     }
     const bool div = divisor != 1.0f;
     const int64_t nvec = n >> 2;
+    constexpr int U = kDivUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
-        f4a a[kUnroll], b[kUnroll];
-        uint32_t c[kUnroll];
+        f4a a[U], b[U];
+        uint32_t c[U];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             const bool ok = full || i < nvec;
             a[j] = ok ? M::ldf4(outer, i) : f4a{0.f, 0.f, 0.f, 0.f};
@@ -1104,7 +1111,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
             if (CODES) c[j] = ok ? M::ldu32(codes, i) : 0u;
         }
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             f4a v = (a[j] - b[j]) / world_size;
             if (CODES) {
