@@ -39,6 +39,35 @@ def build(verbose: bool = True, defines: dict | None = None, out: Path | None = 
     return out
 
 
+def kernel_resources() -> dict:
+    """Registers and scratch of every kernel as the production flags compile it: a device-only
+    compile with the compiler's resource remarks.  Returns {mangled name: {"vgprs", "scratch",
+    "occupancy", "lds"}}.  A streaming kernel that needs scratch has spilled registers: its spill
+    traffic competes with the data it streams."""
+    import re
+    import tempfile
+
+    flags = [f for f in HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    with tempfile.TemporaryDirectory() as tmp:
+        cmd = ["hipcc", *flags, "--cuda-device-only", "-c", *map(str, SOURCES), "-o", str(Path(tmp) / "device.o"),
+               "-Rpass-analysis=kernel-resource-usage"]
+        res = subprocess.run(cmd, check=True, capture_output=True, text=True)
+    out, name = {}, None
+    keys = {"VGPRs": "vgprs", "ScratchSize [bytes/lane]": "scratch", "Occupancy [waves/SIMD]": "occupancy",
+            "LDS Size [bytes/block]": "lds"}
+    for line in res.stderr.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            out[name] = {}
+            continue
+        for label, key in keys.items():
+            m = re.search(re.escape(label) + r": (\d+)", line)
+            if m and name:
+                out[name][key] = int(m.group(1))
+    return out
+
+
 if __name__ == "__main__":
     build()
     sys.exit(0)

@@ -68,3 +68,19 @@ def test_options_round_trip():
         assert "unknown option" in str(e)
     else:
         raise AssertionError("unknown option accepted")
+
+
+def test_no_kernel_spills_and_streaming_kernels_keep_full_occupancy():
+    # a spilled register in a bandwidth-bound kernel shows up as extra HBM traffic (scratch); the
+    # streaming kernels are compiled for 8 wavefronts per SIMD, so two 1024-thread workgroups fit a CU
+    from prime_amd.build import kernel_resources
+
+    res = kernel_resources()
+    assert len(res) >= 40
+    spilled = {k: v["scratch"] for k, v in res.items() if v.get("scratch", 0) > 0}
+    assert not spilled, spilled
+    streaming = ("stats_kernel", "quantize_kernel", "hist_kernel", "dequant_kernel", "first_touch_kernel", "outer_step_kernel",
+                 "pseudo_gradient_kernel", "div_kernel", "code_count_kernel", "code_remap_kernel", "copy_kernel")
+    for name, v in res.items():
+        if any(s in name for s in streaming):
+            assert v["occupancy"] == 8 and v["vgprs"] <= 64, (name, v)
