@@ -20,6 +20,9 @@ The single JSON line printed at the end carries
   ring_step      BASELINE config 3: W = 8 chunks of 2^26 elements; quantize chunk 0, then 7 hops of
                  dequantize-add + requantize (14 bytes per element per hop)
   tensor_2p28    uniform_8bit_quantize on one 2^28-element tensor, the size the target is quoted on
+  other_configs  BASELINE configs 1, 4 and 5 (round trip on 2^24 elements; 42 buckets of a 10B model's
+                 shard with outliers, quantize + dequantize; 2,000 small tensors in one launch and the
+                 edge tensors), each as algorithmic GB/s
   cpu_baseline   the reference's own compression.cpp (compiled into oracle/_ref) on this box's
                  host cores, on a bounded sample (one bucket, a few repetitions)
 """
@@ -167,8 +170,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--streams", type=int, default=3,
                     help="HIP streams the buckets are spread over in the timed region (1 = strictly one after another)")
-    ap.add_argument("--legs", default="buckets,ring,t28,outer,diloco",
-                    help="comma list of buckets (always run: it carries value and roofline), ring, t28, outer, diloco")
+    ap.add_argument("--legs", default="buckets,ring,t28,outer,diloco,configs",
+                    help="comma list of buckets (always run: it carries value and roofline), ring, t28, outer, diloco, configs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -507,6 +510,99 @@ def main() -> int:
         }
         del outers, inners, grads, moms
         torch.cuda.empty_cache()
+
+    if "configs" in legs:
+        # ---- the other BASELINE configurations, one figure each ---------------------------------------
+        import numpy as np
+
+        cfgs = {}
+
+        def dequant(o, lut_t, codes_t):
+            _lib.check(lib.prime_dequant_set(o.data_ptr(), lut_t.data_ptr(), codes_t.data_ptr(), o.numel(), st), "dequant_set")
+
+        # config 1: 2^24 elements N(0, 1e-3), quantize -> dequantize round trip (14 B/element; 64 MiB:
+        # the tensor stays in the 256 MB last-level cache between the passes)
+        n1 = 1 << 24
+        g = torch.Generator(device=dev).manual_seed(0)
+        x1 = torch.randn(n1, device=dev, generator=g) * 1e-3
+        c1 = torch.empty(n1, dtype=torch.uint8, device=dev)
+        o1 = torch.empty(n1, device=dev)
+        l1 = torch.empty(256, device=dev)
+        q1 = torch.empty(4, dtype=torch.float64, device=dev)
+
+        def cfg1():
+            uniform(x1, c1, l1, q1)
+            dequant(o1, l1, c1)
+
+        t1 = timed(cfg1, args.steps * 5, args.warmup)
+        cfgs["config_1_round_trip_2p24"] = {"us": round(t1 * 1e6, 2), "bytes_per_element": 14, "GBps": round(14.0 * n1 / t1 / 1e9, 1),
+                                           "frac_of_hbm_peak": round(14.0 * n1 / t1 / 1e9 / HBM_PEAK_GBS, 4),
+                                           "note": "cache-assisted: 64 MiB fits the last-level cache"}
+        del x1, c1, o1
+
+        # config 4: 1.25e9 elements in 42 buckets (29,761,904 each, the last 32 longer), N(0, 5e-4) with
+        # 0.01 % of entries at +-50 sigma; quantize + lookup over three streams, then dequantize
+        sizes4 = [29_761_904] * 41 + [29_761_904 + 32]
+        xs4 = []
+        for b, nb4 in enumerate(sizes4):
+            g = torch.Generator(device=dev).manual_seed(400 + b)
+            x = torch.randn(nb4, device=dev, generator=g) * 5e-4
+            pos = torch.randint(0, nb4, (nb4 // 10000,), device=dev, generator=g)
+            sign = torch.randint(0, 2, (nb4 // 10000,), device=dev, generator=g).float() * 2 - 1
+            x[pos] = sign * (50 * 5e-4)
+            xs4.append(x)
+        cs4 = [torch.empty(nb4, dtype=torch.uint8, device=dev) for nb4 in sizes4]
+        os4 = [torch.empty(nb4, device=dev) for nb4 in sizes4]
+        l4 = torch.empty((42, 256), device=dev)
+        q4 = torch.empty((42, 4), dtype=torch.float64, device=dev)
+        plan4 = ops.BucketPlan(xs4, cs4, l4, q4, n_streams=args.streams)
+
+        def cfg4():
+            plan4.run()
+            for b in range(42):
+                dequant(os4[b], l4[b], cs4[b])
+
+        steps4 = max(2, args.steps // 3)
+        t4 = timed(cfg4, steps4, 1)
+        cfgs["config_4_shard_42_buckets"] = {"ms": round(t4 * 1e3, 3), "bytes_per_element": 14, "elements": sum(sizes4),
+                                            "GBps": round(14.0 * sum(sizes4) / t4 / 1e9, 1),
+                                            "frac_of_hbm_peak": round(14.0 * sum(sizes4) / t4 / 1e9 / HBM_PEAK_GBS, 4)}
+        del xs4, cs4, os4, plan4
+        torch.cuda.empty_cache()
+
+        # config 5: 2,000 small tensors N(1, 1e-2), sizes U[1, 65536], in one launch; the edge tensors
+        rng = np.random.default_rng(5)
+        sizes5 = rng.integers(1, 65536, 2000, endpoint=True)
+        off5 = torch.from_numpy(np.concatenate([[0], np.cumsum(sizes5)]).astype(np.int64)).to(dev)
+        tot5 = int(sizes5.sum())
+        g = torch.Generator(device=dev).manual_seed(5)
+        x5 = torch.randn(tot5, device=dev, generator=g) * 1e-2 + 1
+        c5 = torch.empty(tot5, dtype=torch.uint8, device=dev)
+        l5 = torch.empty((2000, 256), device=dev)
+        q5 = torch.empty((2000, 4), dtype=torch.float64, device=dev)
+
+        def cfg5():
+            _lib.check(lib.prime_uniform_8bit_quantize_batched(x5.data_ptr(), off5.data_ptr(), 2000, c5.data_ptr(), l5.data_ptr(),
+                                                               q5.data_ptr(), st), "batched")
+
+        t5 = timed(cfg5, args.steps * 3, args.warmup)
+        edge = {}
+        n20 = 1 << 20
+        g = torch.Generator(device=dev).manual_seed(50)
+        half = torch.randn(n20, device=dev, generator=g) * 1e-3
+        half[torch.rand(n20, device=dev, generator=g) < 0.5] = 0
+        tail = torch.randn((1 << 24) + 7, device=dev, generator=g) * 1e-3
+        for name, x in (("constant_2p20", torch.full((n20,), 0.25, device=dev)), ("zeros_2p20", torch.zeros(n20, device=dev)),
+                        ("half_zeros_2p20", half), ("tail_2p24_plus_7", tail)):
+            ce = torch.empty(x.numel(), dtype=torch.uint8, device=dev)
+            te = timed(lambda: uniform(x, ce, l1, q1), args.steps * 5, args.warmup)
+            edge[name] = {"us": round(te * 1e6, 2), "GBps": round(9.0 * x.numel() / te / 1e9, 1)}
+        cfgs["config_5_small_and_edge_tensors"] = {
+            "batched_2000_tensors": {"us": round(t5 * 1e6, 2), "elements": tot5, "bytes_per_element": 9,
+                                     "GBps": round(9.0 * tot5 / t5 / 1e9, 1),
+                                     "frac_of_hbm_peak": round(9.0 * tot5 / t5 / 1e9 / HBM_PEAK_GBS, 4)},
+            "edge": edge, "note": "the 2^20-element tensors (4 MiB) run from cache and are bound by launch latency"}
+        out["other_configs"] = cfgs
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(BUCKET_ELEMS, RING_CHUNK, reps=5)
