@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One "step" is one pass of the hot path over the workload of BASELINE config 2: the 22
+One "step" is one pass of the hot path over the workload of benchmark configuration 2: the 22
 per-layer pseudo-gradient buckets of a 1B Llama-style model (51,380,224 fp32 elements each,
 Student-t(3) * 1e-4), each run through uniform_8bit_quantize (statistics pass, then the
 fused quantize + 256-bin lookup build).  Inputs are generated on the GPU with a seeded torch
@@ -17,10 +17,10 @@ The single JSON line printed at the end carries
   roofline       the dominant kernel (quantize + histogram, 5 bytes per element) priced against
                  the 8 TB/s HBM peak from per-launch HIP-event times taken in a second pass over
                  the same workload
-  ring_step      BASELINE config 3: W = 8 chunks of 2^26 elements; quantize chunk 0, then 7 hops of
+  ring_step      benchmark configuration 3: W = 8 chunks of 2^26 elements; quantize chunk 0, then 7 hops of
                  dequantize-add + requantize (14 bytes per element per hop)
   tensor_2p28    uniform_8bit_quantize on one 2^28-element tensor, the size the target is quoted on
-  other_configs  BASELINE configs 1, 4 and 5 (round trip on 2^24 elements; 42 buckets of a 10B model's
+  other_configs  benchmark configurations 1, 4 and 5 (round trip on 2^24 elements; 42 buckets of a 10B model's
                  shard with outliers, quantize + dequantize; 2,000 small tensors in one launch and the
                  edge tensors), each as algorithmic GB/s
   cpu_baseline   the reference's own compression.cpp (compiled into oracle/_ref) on this box's
@@ -293,7 +293,7 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE config 2: 22 per-layer pseudo-gradient buckets x 51,380,224 fp32 elements, "
+            "workload": "benchmark configuration 2: 22 per-layer pseudo-gradient buckets x 51,380,224 fp32 elements, "
                         "Student-t(3)*1e-4 (torch cuda generator, seed = layer), uniform_8bit_quantize bucket by bucket",
             "elements_per_step": elems,
             "streams": args.streams,
@@ -345,7 +345,7 @@ def main() -> int:
         rprof = _lib.profile_end()
         ring_gbs = 14.0 * RING_CHUNK / hop / 1e9
         out["ring_step"] = {
-            "workload": "BASELINE config 3: W=8 ranks, 2^26-element chunks N(0,1e-3) (seed = rank); per hop: "
+            "workload": "benchmark configuration 3: W=8 ranks, 2^26-element chunks N(0,1e-3) (seed = rank); per hop: "
                         "acc += lut[codes]; uniform_8bit_quantize(acc)",
             "value": round(ring_gbs, 1),
             "unit": "GB/s",
@@ -512,7 +512,7 @@ def main() -> int:
         torch.cuda.empty_cache()
 
     if "configs" in legs:
-        # ---- the other BASELINE configurations, one figure each ---------------------------------------
+        # ---- the other benchmark configurations, one figure each ---------------------------------------
         import numpy as np
 
         cfgs = {}

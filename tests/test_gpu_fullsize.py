@@ -55,7 +55,7 @@ def test_uniform_8bit_quantize_2p28_properties(abi):
 
 
 def test_ring_reduce_step_2p26_chunks(abi):
-    # BASELINE config 3 shape: 2^26-element chunks; three ranks' worth to bound memory and time
+    # benchmark configuration 3 shape: 2^26-element chunks; three ranks' worth to bound memory and time
     n = 1 << 26
     g = torch.Generator(device=abi.dev).manual_seed(1)
     x0 = torch.randn(n, device=abi.dev, generator=g) * 1e-3
@@ -78,7 +78,7 @@ def test_ring_reduce_step_2p26_chunks(abi):
 
 
 def test_config4_shard_all_42_buckets(abi):
-    # BASELINE config 4 in full: 1.25e9 elements (5 GB) as 42 buckets, the last 32 longer, N(0, 5e-4)
+    # benchmark configuration 4 in full: 1.25e9 elements (5 GB) as 42 buckets, the last 32 longer, N(0, 5e-4)
     # with 0.01 % of entries at +-50 sigma; quantize + lookup + dequantize per bucket, checked through
     # properties that hold at any size
     base, extra, nb = 29_761_904, 32, 42

@@ -1,4 +1,4 @@
-"""Parity of the HIP path with the CPU oracle, through the C ABI, on the BASELINE
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on the benchmark
 configurations at sizes the oracle finishes in seconds.
 
 Bars: uint8 codes, dequantized values and accumulators bit-exact; scale equal to the float
@@ -50,7 +50,7 @@ def check_uniform(abi, oracle, x: np.ndarray, label: str):
 
 
 def test_cfg1_round_trip_2p24(abi, oracle):
-    # BASELINE config 1: 2^24 elements, N(0, 1e-3), seed 0; quantize then dequantize
+    # benchmark configuration 1: 2^24 elements, N(0, 1e-3), seed 0; quantize then dequantize
     x = (np.random.default_rng(0).standard_normal(1 << 24) * 1e-3).astype(np.float32)
     xt, codes, lut, q = check_uniform(abi, oracle, x, "cfg1")
     out = torch.empty_like(xt)
@@ -74,7 +74,7 @@ def test_cfg1_round_trip_2p24(abi, oracle):
 
 
 def test_cfg2_llama_1b_layer_bucket(abi, oracle):
-    # BASELINE config 2: one per-layer bucket, 4*2048*2048 + 3*2048*5632 elements, Student-t(3) * 1e-4
+    # benchmark configuration 2: one per-layer bucket, 4*2048*2048 + 3*2048*5632 elements, Student-t(3) * 1e-4
     n = 4 * 2048 * 2048 + 3 * 2048 * 5632
     assert n == 51_380_224
     x = (np.random.default_rng(0).standard_t(3, n) * 1e-4).astype(np.float32)
@@ -84,7 +84,7 @@ def test_cfg2_llama_1b_layer_bucket(abi, oracle):
 
 
 def test_cfg3_ring_hops_w8(abi, oracle):
-    # BASELINE config 3 at chunk 2^20: W = 8 ranks, hop by hop with identical inputs on both sides
+    # benchmark configuration 3 at chunk 2^20: W = 8 ranks, hop by hop with identical inputs on both sides
     W, n = 8, 1 << 20
     chunks = [(np.random.default_rng(r).standard_normal(n) * 1e-3).astype(np.float32) for r in range(W)]
     xt, codes, lut, q = check_uniform(abi, oracle, chunks[0], "cfg3 rank 0")
@@ -118,7 +118,7 @@ def test_cfg3_ring_hops_w8(abi, oracle):
 
 
 def test_cfg4_fsdp_shard_bucket_with_outliers(abi, oracle):
-    # BASELINE config 4: 1.25e9 elements in 42 buckets of 29,761,904, the last one 32 longer;
+    # benchmark configuration 4: 1.25e9 elements in 42 buckets of 29,761,904, the last one 32 longer;
     # N(0, 5e-4) with 0.01 % of entries at +-50 sigma.  The last bucket is checked in full.
     n = 29_761_904 + 32
     assert 41 * 29_761_904 + n == 1_250_000_000
@@ -136,7 +136,7 @@ def test_cfg4_fsdp_shard_bucket_with_outliers(abi, oracle):
 
 
 def test_cfg5_two_thousand_small_tensors_batched(abi, oracle):
-    # BASELINE config 5: 2,000 tensors of sizes U[1, 65536], N(1, 1e-2), one launch
+    # benchmark configuration 5: 2,000 tensors of sizes U[1, 65536], N(1, 1e-2), one launch
     rng = np.random.default_rng(5)
     sizes = rng.integers(1, 65536, 2000, endpoint=True)
     off = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
@@ -380,7 +380,7 @@ def test_literal_norm_is_libtorch_order_bit_for_bit(abi, oracle, n):
 
 
 def test_literal_norm_against_the_compiled_reference_at_2p24(abi, oracle):
-    # BASELINE config 1 as the reference itself computes it: same scale, same codes, every element
+    # benchmark configuration 1 as the reference itself computes it: same scale, same codes, every element
     if not oracle.ref_available():
         pytest.skip("oracle/_ref is not built")
     import torch as _t
