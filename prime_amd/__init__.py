@@ -1,7 +1,8 @@
 """prime_amd: the int8 pseudo-gradient compression path of prime (ZeroBand) on MI355X.
 
 Layout
-    csrc/            HIP kernels and the C ABI (libprime_hip.so; include/prime_hip.h)
+    csrc/            HIP kernels (kernels_*.h, device_common.h) and the C ABI (prime_hip.hip ->
+                     libprime_hip.so; include/prime_hip.h)
     _lib.py          ctypes binding of the C ABI
     ops.py           torch.library ops over it
     C/compression.py, C/collectives.py, collectives.py, config.py

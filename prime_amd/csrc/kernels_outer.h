@@ -1,0 +1,231 @@
+// Either side of the all-reduce: division, pseudo-gradient, a chunk's first touch in the ring,
+// the SGD-Nesterov outer step (from fp32 or from codes), and the plain copy and fill kernels.
+//
+// Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
+
+__global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < nwords;
+         i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+        p[i] = 0u;
+}
+
+// chunk /= world_size for ReduceOp::AVG (collectives.cpp:155-159): an fp32 division in place.
+template <bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void div_kernel(float* __restrict__ x, int64_t n, float d) {
+    using M = Mem<ALIGNED, false>;
+    const int64_t nvec = n >> 2;
+    constexpr int U = kDivUnroll;
+    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a v[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = i0 + j * stride;
+            v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) M::stf4(x, i, v[j] / d, false);
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        x[i] = x[i] / d;
+    }
+}
+
+// The pseudo-gradient of one bucket as Diloco.sync_pseudo_gradient forms it
+// (src/zeroband/diloco.py:93-101): grad = outer_param - inner_param, then the whole flat buffer
+// divided by the world size; an fp32 subtraction and an fp32 division per element.
+// 12 bytes per element.
+template <bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer,
+                                                                                   const float* __restrict__ inner, int64_t n,
+                                                                                   float world_size, float* __restrict__ out) {
+    using M = Mem<ALIGNED, false>;
+    const int64_t nvec = n >> 2;
+    constexpr int U = kDivUnroll;
+    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a a[U], b[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = i0 + j * stride;
+            const bool ok = full || i < nvec;
+            a[j] = ok ? M::ldf4(outer, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            b[j] = ok ? M::ldf4(inner, i) : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) M::stf4(out, i, (a[j] - b[j]) / world_size, false);
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        out[i] = (outer[i] - inner[i]) / world_size;
+    }
+}
+
+// A chunk's first touch in the ring when the pseudo-gradient has not been written yet: every
+// chunk of a rank is visited exactly once in the reduce-scatter (collectives.cpp:115-116), so
+// grad = (outer - inner) / world_size (diloco.py:93-101) can be formed in the pass that would
+// otherwise read it back.  With CODES the received message is accumulated,
+// acc = grad + lut[codes] (collectives.cpp:128-133), and with a divisor other than 1 the sum is
+// divided (ReduceOp::AVG, :155-159).  The fp64 sum and sum of squares of what is stored are the
+// statistics of the quantization that follows.  12 bytes per element, 13 with codes.
+template <bool CODES, bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(const float* __restrict__ outer,
+                                                                               const float* __restrict__ inner, int64_t n,
+                                                                               float world_size, const uint8_t* __restrict__ codes,
+                                                                               const float* __restrict__ lut, float divisor,
+                                                                               float* __restrict__ out, Workspace* ws) {
+    using M = Mem<ALIGNED, false>;
+    __shared__ float s_lut[kBins];
+    if (CODES) {
+        for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
+        __syncthreads();
+    }
+    const bool div = divisor != 1.0f;
+    const int64_t nvec = n >> 2;
+    constexpr int U = kDivUnroll;
+    double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
+    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a a[U], b[U];
+        uint32_t c[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = i0 + j * stride;
+            const bool ok = full || i < nvec;
+            a[j] = ok ? M::ldf4(outer, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            b[j] = ok ? M::ldf4(inner, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            if (CODES) c[j] = ok ? M::ldu32(codes, i) : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = i0 + j * stride;
+            f4a v = (a[j] - b[j]) / world_size;
+            if (CODES) {
+                f4a l;
+                l.x = s_lut[c[j] & 255];
+                l.y = s_lut[(c[j] >> 8) & 255];
+                l.z = s_lut[(c[j] >> 16) & 255];
+                l.w = s_lut[c[j] >> 24];
+                v += l;
+                if (div) v = v / divisor;
+            }
+            if (full || i < nvec) {
+                M::stf4(out, i, v, false);       // the quantize pass reads it again: no streaming hint
+                if (j & 1) stats_add4(v, s1, q1); else stats_add4(v, s0, q0);
+            }
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        float v = (outer[i] - inner[i]) / world_size;
+        if (CODES) {
+            v += s_lut[codes[i]];
+            if (div) v = v / divisor;
+        }
+        out[i] = v;
+        const double d = v;
+        s0 += d;
+        q0 = fma(d, d, q0);
+    }
+    block_stats_store(s0 + s1, q0 + q1, ws);
+}
+
+// One element of the outer optimizer, torch.optim.SGD(lr, momentum, nesterov=True) as the
+// reference builds it (src/zeroband/diloco.py:72-74) and libtorch's CPU kernels round it:
+//   buf = buf * mu + g     (a product and a sum, each rounded; buf = g on the first step)
+//   d   = fma(buf, mu, g)  (add with alpha: one rounding)
+//   p   = fma(d, -lr, p)
+__device__ __forceinline__ void outer_sgd_one(float& p, float& buf, float g, float neg_lr, float mu, bool first) {
+    buf = first ? g : buf * mu + g;
+    const float d = fmaf(buf, mu, g);
+    p = fmaf(d, neg_lr, p);
+}
+
+// Outer step of DiLoCo on one bucket (diloco.py:212-215): SGD with Nesterov momentum on the
+// outer parameters with the reduced pseudo-gradient, and the copy of the new parameters to
+// the inner model (sync_inner_model, :137-144) in the same pass.  The gradient is fp32
+// (24 bytes per element) or, with CODES, uint8 codes and their lookup table (21 bytes per
+// element, and the dequantize pass is saved).
+template <bool CODES, bool ALIGNED>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom,
+                                                                              const float* __restrict__ grad,
+                                                                              const uint8_t* __restrict__ codes,
+                                                                              const float* __restrict__ lut,
+                                                                              float* __restrict__ inner, int64_t n, float neg_lr,
+                                                                              float mu, int first) {
+    using M = Mem<ALIGNED, false>;
+    __shared__ float s_lut[kBins];
+    if (CODES) {
+        for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
+        __syncthreads();
+    }
+    const int64_t nvec = n >> 2;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a p[kUnroll], m[kUnroll], g[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            const bool ok = full || i < nvec;
+            p[j] = ok ? M::ldf4(param, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            m[j] = (ok && !first) ? M::ldf4(mom, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            if (CODES) {
+                const uint32_t c = ok ? M::ldu32(codes, i) : 0u;
+                g[j] = f4a{s_lut[c & 255], s_lut[(c >> 8) & 255], s_lut[(c >> 16) & 255], s_lut[c >> 24]};
+            } else {
+                g[j] = ok ? M::ldf4(grad, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float pc = p[j][c], mc = m[j][c];
+                    outer_sgd_one(pc, mc, g[j][c], neg_lr, mu, first);
+                    p[j][c] = pc;
+                    m[j][c] = mc;
+                }
+                M::stf4(param, i, p[j], false);
+                M::stf4(mom, i, m[j], false);
+                if (inner) M::stf4(inner, i, p[j], true);
+            }
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        float p = param[i];
+        float m = first ? 0.f : mom[i];
+        const float g = CODES ? s_lut[codes[i]] : grad[i];
+        outer_sgd_one(p, m, g, neg_lr, mu, first);
+        param[i] = p;
+        mom[i] = m;
+        if (inner) inner[i] = p;
+    }
+}
+
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
+    using M = Mem<true, false>;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a v[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) v[j] = M::ldf4(reinterpret_cast<const float*>(src), i);
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) M::stf4(reinterpret_cast<float*>(dst), i, v[j], true);
+        }
+    });
+}

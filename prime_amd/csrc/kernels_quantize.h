@@ -1,0 +1,289 @@
+// Quantization to uint8 codes with the 256-bin sum / count histogram, the lookup-table second
+// stage, the histogram under given codes (average_buckets) and the one-workgroup-per-tensor
+// kernel for many small tensors.
+//
+// Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
+
+// K2 (+K3 when HIST): quantize to uint8, 4 codes packed per 32-bit store, and the 256-bin
+// sum / count histogram of the same elements.  5 bytes per element.
+template <bool ALIGNED, bool NT, bool HIST, int R>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
+                                                            int stats_parts, prime_qparams* qp_out, int zero_point,
+                                                            uint8_t* __restrict__ codes, Workspace* ws) {
+    using M = Mem<ALIGNED, NT>;
+    __shared__ LdsHist<HIST ? R : 1> hist;
+    if (HIST) hist_zero(hist);
+    // the scale: given by value, or derived here from the statistics partials of the pass before
+    // (stats_parts < 0: the record a preceding kernel left in the workspace)
+    int hot_base = INT_MIN;              // set when the statistics show a tensor crowded into a few codes
+    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &hot_base)
+                      : stats_parts < 0 ? ws->qp.inv_scale
+                                        : 1.0f / scale_val;
+    if (HIST) __syncthreads();
+    const int64_t nvec = n >> 2;
+    auto pass = [&](auto narrow_t) {
+        constexpr bool narrow = decltype(narrow_t)::value;
+        HotCodes hot;
+        hot.base = hot_base;
+        auto add = [&](int code, float xv) {
+            if (narrow) hist_add_hot(hist, hot, code, xv);
+            else hist_add(hist, code, xv);
+        };
+        sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+            constexpr bool full = decltype(full_t)::value;
+            f4a v[kUnroll];
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) {
+                const int64_t i = i0 + j * stride;
+                v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int j = 0; j < kUnroll; ++j) {
+                const int64_t i = i0 + j * stride;
+                if (full || i < nvec) {
+                    const int a = quantize_code(v[j].x, inv, zero_point);
+                    const int b = quantize_code(v[j].y, inv, zero_point);
+                    const int c = quantize_code(v[j].z, inv, zero_point);
+                    const int d = quantize_code(v[j].w, inv, zero_point);
+                    M::stu32(codes, i, static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) |
+                                           (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24));
+                    if (HIST) {
+                        add(a, v[j].x);
+                        add(b, v[j].y);
+                        add(c, v[j].z);
+                        add(d, v[j].w);
+                    }
+                }
+            }
+        });
+        if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+            const int64_t i = (nvec << 2) + threadIdx.x;
+            const float v = x[i];
+            const int a = quantize_code(v, inv, zero_point);
+            codes[i] = static_cast<uint8_t>(a);
+            if (HIST) add(a, v);
+        }
+        if (HIST && narrow) hist_flush_hot(hist, hot);
+    };
+    if (HIST && hot_base != INT_MIN) pass(std::true_type{});
+    else pass(std::false_type{});
+    if (HIST) {
+        __syncthreads();
+        hist_store(hist, ws);
+    }
+}
+
+// K3 alone: histogram of x under caller-supplied codes (average_buckets).  5 bytes per element.
+template <bool ALIGNED, int R>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const float* __restrict__ x, const uint8_t* __restrict__ codes,
+                                                        int64_t n, int n_bins, Workspace* ws) {
+    using M = Mem<ALIGNED, false>;
+    __shared__ LdsHist<R> hist;
+    hist_zero(hist);
+    __syncthreads();
+    const int64_t nvec = n >> 2;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a v[kUnroll];
+        uint32_t c[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            const bool ok = full || i < nvec;
+            v[j] = ok ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            c[j] = ok ? M::ldu32(codes, i) : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) {
+                const int a = c[j] & 255, b = (c[j] >> 8) & 255, cc = (c[j] >> 16) & 255, d = c[j] >> 24;
+                if (a < n_bins) hist_add(hist, a, v[j].x);     // compression.cpp:70
+                if (b < n_bins) hist_add(hist, b, v[j].y);
+                if (cc < n_bins) hist_add(hist, cc, v[j].z);
+                if (d < n_bins) hist_add(hist, d, v[j].w);
+            }
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        const int a = codes[i];
+        if (a < n_bins) hist_add(hist, a, x[i]);
+    }
+    __syncthreads();
+    hist_store(hist, ws);
+}
+
+// Second stage of the lookup build.  Workgroup j owns bins 4j .. 4j+3 (64 contiguous bytes
+// of every partial): lane (row, bin) adds partials row, row + 256, ... in order, the 256
+// rows are then added by a tree of fixed shape.  Mean = fp64 sum / count rounded to float
+// once; an empty bin gives 0.0f (compression.cpp:100).  Entries >= 256 of a longer table
+// are 0.0f.
+__global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Workspace* __restrict__ ws, int nparts,
+                                                                      float* __restrict__ lut, int64_t n_bins,
+                                                                      unsigned long long* __restrict__ counts) {
+    constexpr int kRows = kFinalThreads / kLutBinsPerBlock;
+    __shared__ double sh_sum[kFinalThreads];
+    __shared__ unsigned long long sh_cnt[kFinalThreads];
+    const int bl = threadIdx.x % kLutBinsPerBlock;
+    const int row = threadIdx.x / kLutBinsPerBlock;
+    const int bin = blockIdx.x * kLutBinsPerBlock + bl;
+    constexpr int kIters = kMaxGrid / kRows;
+    BinAcc part[kIters];
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) {          // all loads in flight at once
+        const int p = row + k * kRows;
+        part[k] = p < nparts ? ws->hist[p][bin] : BinAcc{0.0, 0ull};
+    }
+    double s = 0.0;
+    unsigned long long c = 0;
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) { s += part[k].sum; c += part[k].cnt; }
+    sh_sum[threadIdx.x] = s;
+    sh_cnt[threadIdx.x] = c;
+    __syncthreads();
+    for (int half = kRows / 2; half > 0; half >>= 1) {
+        if (row < half) {
+            sh_sum[threadIdx.x] += sh_sum[threadIdx.x + half * kLutBinsPerBlock];
+            sh_cnt[threadIdx.x] += sh_cnt[threadIdx.x + half * kLutBinsPerBlock];
+        }
+        __syncthreads();
+    }
+    if (row == 0 && bin < n_bins) {
+        const unsigned long long cc = sh_cnt[threadIdx.x];
+        lut[bin] = cc ? static_cast<float>(sh_sum[threadIdx.x] / static_cast<double>(cc)) : 0.0f;
+        if (counts) counts[bin] = cc;
+    }
+    if (blockIdx.x == 0)
+        for (int64_t b = kBins + threadIdx.x; b < n_bins; b += kFinalThreads) lut[b] = 0.0f;
+}
+
+__global__ void lut_zero_kernel(float* __restrict__ lut, int64_t n_bins, unsigned long long* __restrict__ counts) {
+    for (int64_t b = threadIdx.x; b < n_bins; b += blockDim.x) {
+        lut[b] = 0.0f;
+        if (counts && b < kBins) counts[b] = 0ull;
+    }
+}
+
+// Small tensors: one workgroup per tensor of a flat buffer does the whole of
+// uniform_8bit_quantize (statistics, scale, codes, lookup) without touching the workspace.
+// With VEC (flat buffer 16-byte aligned, code buffer 4-byte aligned) the part of the tensor
+// between its first and last multiple-of-4 global index is read as 16-byte vectors and its
+// codes stored 4 at a time; the ragged ends, which share vectors with the neighbouring
+// tensors, go element by element.  The second read of a tensor comes from L2.
+template <bool VEC>
+__global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __restrict__ x, const int64_t* __restrict__ offsets,
+                                                                uint8_t* __restrict__ codes, float* __restrict__ luts,
+                                                                prime_qparams* __restrict__ qps) {
+    constexpr int R = 4;
+    __shared__ LdsHist<R> hist;
+    __shared__ double sh_s[kBatchThreads / 64];
+    __shared__ double sh_q[kBatchThreads / 64];
+    __shared__ prime_qparams sh_qp;
+    __shared__ int sh_hot_base;          // >= -1: the tensor is narrow, hot codes start here; INT_MIN: it is not
+    const int64_t t = blockIdx.x;
+    const int64_t lo = offsets[t];
+    const int64_t hi = offsets[t + 1];
+    const int64_t n = hi - lo;
+    // [lo, a) and [b, hi) element by element, [a, b) as vectors
+    int64_t a = VEC ? (lo + 3) & ~int64_t(3) : hi;
+    int64_t b = VEC ? hi & ~int64_t(3) : hi;
+    if (a > b) { a = hi; b = hi; }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < kBins * R; i += kBatchThreads) { hist.sum[i] = 0.0; hist.cnt[i] = 0u; }
+    double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
+    const f4a* __restrict__ x4 = reinterpret_cast<const f4a*>(x);
+    constexpr int U = 4;
+    for (int64_t v0 = (a >> 2) + threadIdx.x; v0 < (b >> 2); v0 += kBatchThreads * U) {
+        f4a v[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = v0 + j * kBatchThreads;
+            v[j] = i < (b >> 2) ? x4[i] : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if (j & 1) stats_add4(v[j], s1, q1); else stats_add4(v[j], s0, q0);
+        }
+    }
+    for (int64_t i = lo + threadIdx.x; i < a; i += kBatchThreads) {        // ragged head (everything without VEC)
+        const double v = x[i];
+        s0 += v;
+        q0 = fma(v, v, q0);
+    }
+    for (int64_t i = b + threadIdx.x; i < hi; i += kBatchThreads) {        // ragged tail
+        const double v = x[i];
+        s1 += v;
+        q1 = fma(v, v, q1);
+    }
+    double s = wave_sum(s0 + s1);
+    double q = wave_sum(q0 + q1);
+    if (lane == 0) { sh_s[wave] = s; sh_q[wave] = q; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double S = sh_s[0], Q = sh_q[0];
+#pragma unroll
+        for (int w = 1; w < kBatchThreads / 64; ++w) { S += sh_s[w]; Q += sh_q[w]; }
+        finalize_qparams(S, Q, n, &sh_qp);
+        if (qps) qps[t] = sh_qp;
+        sh_hot_base = narrow_distribution(S, Q, n)
+                          ? quantize_code(static_cast<float>(S / static_cast<double>(n)), sh_qp.inv_scale, kZeroPoint) - 1
+                          : INT_MIN;
+    }
+    __syncthreads();
+    const float inv = sh_qp.inv_scale;
+    uint32_t* __restrict__ c4 = reinterpret_cast<uint32_t*>(codes);
+    auto second_pass = [&](auto narrow_t) {
+    constexpr bool narrow = decltype(narrow_t)::value;
+    HotCodes hot;
+    hot.base = sh_hot_base;
+    auto add = [&](int code, float xv) {
+        if (narrow) hist_add_hot(hist, hot, code, xv);
+        else hist_add(hist, code, xv);
+    };
+    for (int64_t v0 = (a >> 2) + threadIdx.x; v0 < (b >> 2); v0 += kBatchThreads * U) {
+        f4a v[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = v0 + j * kBatchThreads;
+            v[j] = i < (b >> 2) ? x4[i] : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t i = v0 + j * kBatchThreads;
+            if (i < (b >> 2)) {
+                const int ca = quantize_code(v[j].x, inv, kZeroPoint);
+                const int cb = quantize_code(v[j].y, inv, kZeroPoint);
+                const int cc = quantize_code(v[j].z, inv, kZeroPoint);
+                const int cd = quantize_code(v[j].w, inv, kZeroPoint);
+                c4[i] = static_cast<uint32_t>(ca) | (static_cast<uint32_t>(cb) << 8) | (static_cast<uint32_t>(cc) << 16) |
+                        (static_cast<uint32_t>(cd) << 24);
+                add(ca, v[j].x);
+                add(cb, v[j].y);
+                add(cc, v[j].z);
+                add(cd, v[j].w);
+            }
+        }
+    }
+    for (int part = 0; part < 2; ++part) {
+        const int64_t from = part ? b : lo, to = part ? hi : a;
+        for (int64_t i = from + threadIdx.x; i < to; i += kBatchThreads) {
+            const float v = x[i];
+            const int c = quantize_code(v, inv, kZeroPoint);
+            codes[i] = static_cast<uint8_t>(c);
+            add(c, v);
+        }
+    }
+    if (narrow) hist_flush_hot(hist, hot);
+    };
+    if (sh_hot_base != INT_MIN) second_pass(std::true_type{});
+    else second_pass(std::false_type{});
+    __syncthreads();
+    for (int bin = threadIdx.x; bin < kBins; bin += kBatchThreads) {
+        double sum = 0.0;
+        unsigned long long cnt = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) { sum += hist.sum[bin * R + r]; cnt += hist.cnt[bin * R + r]; }
+        luts[t * kBins + bin] = cnt ? static_cast<float>(sum / static_cast<double>(cnt)) : 0.0f;
+    }
+}

@@ -1,0 +1,109 @@
+// Statistics: fp64 sum and sum of squares (first stage per workgroup, second stage in one
+// workgroup), and the norm accumulated in libtorch's order for bit-for-bit reproduction.
+//
+// Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
+
+// Second stage of the statistics: one workgroup adds the partials (tree of fixed shape) and
+// derives the scale.
+__global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace* ws, int nparts, int64_t n,
+                                                                        prime_qparams* out) {
+    (void)block_scale_from_partials<kFinalThreads>(ws, nparts, n, out);
+}
+
+// K1: sum and sum of squares in fp64.  4 bytes per element.
+template <bool ALIGNED, bool NT>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
+    using M = Mem<ALIGNED, NT>;
+    const int64_t nvec = n >> 2;
+    double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
+    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        f4a v[kUnroll];
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < kUnroll; ++j) {
+            if (j & 1) stats_add4(v[j], s1, q1); else stats_add4(v[j], s0, q0);
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const double v = x[(nvec << 2) + threadIdx.x];
+        s0 += v;
+        q0 = fma(v, v, q0);
+    }
+    block_stats_store(s0 + s1, q0 + q1, ws);
+}
+
+// The norm as libtorch's CPU kernel accumulates it (the value compression.cpp:113 actually
+// receives): eight fp32 lanes, lane j taking elements j, j + 8, ... by fused multiply-add, lanes
+// added 0..7, then the n % 8 tail in order (a group of four as separately rounded products, the
+// rest by fused multiply-add) and a float square root.  The chains are serial by definition, so
+// this is one workgroup: fifteen wavefronts stage tiles in LDS, eight lanes of the first accumulate.  It exists
+// to reproduce the reference's output bit for bit; the streaming kernels compute the exact sum.
+constexpr int kLiteralTile = 8192;                       // floats per stage (two stages in LDS)
+constexpr int kLiteralRow = kLiteralTile / 8 + 8;        // lane j's elements, padded: conflict-free stores
+__global__ __launch_bounds__(kFinalThreads) void norm_literal_kernel(const float* __restrict__ x, int64_t n, Workspace* ws,
+                                                                      prime_qparams* out) {
+    // tile[buf][j * kLiteralRow + k] = element 8 k + j of the stage: lane j reads its chain in order,
+    // four elements per LDS access.  Wavefront 0 accumulates stage s while the others load stage s + 1.
+    __shared__ __attribute__((aligned(16))) float tile[2][8 * kLiteralRow];
+    const int64_t m = n - (n % 8);
+    const int64_t stages = (m + kLiteralTile - 1) / kLiteralTile;
+    auto load_stage = [&](int64_t s, int first, int step) {
+        const int64_t base = s * kLiteralTile;
+        const int count = static_cast<int>(m - base < kLiteralTile ? m - base : kLiteralTile);   // a multiple of 8
+        float* t = tile[s & 1];
+        for (int i = first; i < count; i += step) t[(i & 7) * kLiteralRow + (i >> 3)] = x[base + i];
+    };
+    float acc = 0.0f;
+    if (stages > 0) load_stage(0, threadIdx.x, kFinalThreads);
+    __syncthreads();
+    for (int64_t s = 0; s < stages; ++s) {
+        if (threadIdx.x >= 64) {
+            if (s + 1 < stages) load_stage(s + 1, threadIdx.x - 64, kFinalThreads - 64);
+        } else if (threadIdx.x < 8) {
+            const int64_t base = s * kLiteralTile;
+            const int per_lane = static_cast<int>(m - base < kLiteralTile ? m - base : kLiteralTile) >> 3;
+            const float* t = tile[s & 1] + threadIdx.x * kLiteralRow;
+            int k = 0;
+            for (; k + 16 <= per_lane; k += 16) {
+                f4a v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f4a*>(t + k + 4 * u);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    acc = __builtin_fmaf(v[u].x, v[u].x, acc);
+                    acc = __builtin_fmaf(v[u].y, v[u].y, acc);
+                    acc = __builtin_fmaf(v[u].z, v[u].z, acc);
+                    acc = __builtin_fmaf(v[u].w, v[u].w, acc);
+                }
+            }
+            for (; k < per_lane; ++k) acc = __builtin_fmaf(t[k], t[k], acc);
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x < 64) {
+        float total = __shfl(acc, 0, 64);
+#pragma unroll
+        for (int j = 1; j < 8; ++j) total += __shfl(acc, j, 64);
+        if (threadIdx.x == 0) {
+            int64_t i = m;
+            if (n - i >= 4) {
+                for (int k = 0; k < 4; ++k) {
+                    const float sq = x[i + k] * x[i + k];     // rounded on its own (contraction is off)
+                    total += sq;
+                }
+                i += 4;
+            }
+            for (; i < n; ++i) total = __builtin_fmaf(x[i], x[i], total);
+            const float norm = __builtin_sqrtf(total);
+            prime_qparams qp;
+            finalize_from_norm(norm, __builtin_nan(""), static_cast<double>(norm) * static_cast<double>(norm), n, &qp);
+            ws->qp = qp;
+            if (out) *out = qp;
+        }
+    }
+}
