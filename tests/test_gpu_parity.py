@@ -469,6 +469,73 @@ def test_random_sizes_offsets_and_distributions(abi, oracle):
         assert np.array_equal(view.cpu().numpy(), ref), case
 
 
+def test_random_sizes_and_offsets_through_the_fused_ring_entry_points(abi, oracle):
+    # seeded sweep over length and the start offset of every buffer (element-aligned variants of the
+    # kernels included) for the reduce step with division, the first touch and the code-domain requantize
+    rng = np.random.default_rng(777)
+    cap = 1_200_000
+    f_big = [torch.empty(cap + 16, dtype=torch.float32, device=abi.dev) for _ in range(3)]
+    c_big = [torch.empty(cap + 16, dtype=torch.uint8, device=abi.dev) for _ in range(2)]
+
+    def check(want, codes, lut, qp, case):
+        q = abi.qparams(qp)
+        assert np.array_equal(np.array([q["scale"]]), np.array([oracle.scale_exact(want)]), equal_nan=True), case
+        oc, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q["scale"]))
+        assert np.array_equal(codes.cpu().numpy(), oc), case
+        mean, _ = oracle.average_buckets_f64(want, oc)
+        floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
+        assert lut_rel_err(lut.cpu().numpy(), mean, floor) <= LUT_TOL, case
+
+    for case in range(30):
+        n = int(rng.integers(2, cap)) if case % 3 else int(rng.integers(2, 5000))
+        offs = [int(o) for o in rng.integers(0, 9, 5)]
+        divisor = float(rng.choice([1.0, 2.0, 3.0, 8.0]))
+        W = float(rng.choice([1.0, 2.0, 4.0, 14.0]))
+        outer = rng.standard_normal(n).astype(np.float32)
+        inner = (outer + rng.standard_normal(n).astype(np.float32) * 1e-3).astype(np.float32)
+        msg_src = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+        announce(f"fused sweep case {case}: n={n} offs={offs} divisor={divisor} W={W}")
+        vo, vi, vg = (b[o:o + n] for b, o in zip(f_big, offs[:3]))
+        vc_in, vc_out = (b[o:o + n] for b, o in zip(c_big, offs[3:]))
+        vo.copy_(abi.to_dev(outer))
+        vi.copy_(abi.to_dev(inner))
+        m_codes, m_lut, _ = abi.uniform(abi.to_dev(msg_src))
+        vc_in.copy_(m_codes)
+        li, ci = m_lut.cpu().numpy(), m_codes.cpu().numpy()
+        lut = torch.empty(256, device=abi.dev)
+        qp = torch.empty(4, dtype=torch.float64, device=abi.dev)
+        # first touch with a message and a divisor
+        _lib.check(abi.lib.prime_ring_first_touch(vo.data_ptr(), vi.data_ptr(), n, W, vc_in.data_ptr(), m_lut.data_ptr(), divisor,
+                                                  vg.data_ptr(), vc_out.data_ptr(), lut.data_ptr(), qp.data_ptr(), abi.ws.data_ptr(),
+                                                  abi.st), "first touch")
+        want = oracle.pseudo_gradient(outer, inner, W)
+        oracle.index_add(want, li, ci)
+        oracle.div_scalar(want, divisor)
+        assert np.array_equal(vg.cpu().numpy(), want), case
+        check(want, vc_out, lut, qp, case)
+        # first touch without a message
+        _lib.check(abi.lib.prime_ring_first_touch(vo.data_ptr(), vi.data_ptr(), n, W, None, None, 1.0, vg.data_ptr(),
+                                                  vc_out.data_ptr(), lut.data_ptr(), qp.data_ptr(), abi.ws.data_ptr(), abi.st),
+                   "first touch")
+        want = oracle.pseudo_gradient(outer, inner, W)
+        assert np.array_equal(vg.cpu().numpy(), want), case
+        check(want, vc_out, lut, qp, case)
+        # reduce step with division onto the pseudo-gradient just written
+        _lib.check(abi.lib.prime_ring_reduce_div_step(vg.data_ptr(), vc_in.data_ptr(), m_lut.data_ptr(), n, divisor, vc_out.data_ptr(),
+                                                      lut.data_ptr(), qp.data_ptr(), abi.ws.data_ptr(), abi.st), "reduce div")
+        oracle.index_add(want, li, ci)
+        oracle.div_scalar(want, divisor)
+        assert np.array_equal(vg.cpu().numpy(), want), case
+        check(want, vc_out, lut, qp, case)
+        # what the all-gather would forward for the message, from its codes alone
+        _lib.check(abi.lib.prime_requantize_codes(vc_in.data_ptr(), m_lut.data_ptr(), n, vc_out.data_ptr(), lut.data_ptr(),
+                                                  qp.data_ptr(), abi.ws.data_ptr(), abi.st), "requantize")
+        deq = np.empty(n, np.float32)
+        oracle.index_set(deq, li, ci)
+        check(deq, vc_out, lut, qp, case)
+        assert np.array_equal(vo.cpu().numpy(), outer) and np.array_equal(vi.cpu().numpy(), inner), case
+
+
 def test_layer_buckets_as_views_of_one_flat_buffer(abi, oracle):
     # the caller's layout (src/zeroband/diloco.py:147-201): one flat fp32 buffer, one view per layer
     # bucket; bucket sizes need not be multiples of four, so most views start misaligned
