@@ -82,6 +82,39 @@ def test_outer_step_from_codes_equals_dequantize_then_step(dev, n):
     assert torch.equal(p1, p2)
 
 
+@pytest.mark.parametrize("shift", [1, 2, 3])
+def test_outer_step_kernels_on_element_aligned_views(dev, oracle, shift):
+    # parameters of a model are views at arbitrary element offsets of the flat buffers: the
+    # element-aligned variants of both outer-step kernels against the oracle (itself pinned on torch's SGD)
+    from prime_amd import ops
+
+    n = 100_003
+    rng = np.random.default_rng(shift)
+    p0 = rng.standard_normal(n).astype(np.float32)
+    b0 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    g0 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    pad = 16
+    bufs = [torch.zeros(n + pad, device=dev) for _ in range(4)]
+    p, b, g, inner = (t[shift + k:shift + k + n] for k, t in enumerate(bufs))
+    p.copy_(torch.from_numpy(p0)); b.copy_(torch.from_numpy(b0)); g.copy_(torch.from_numpy(g0))
+    announce(f"outer step misaligned shift={shift}")
+    ops.outer_sgd_nesterov_(p, b, g, inner, 0.7, 0.9, False)
+    wp, wb = p0.copy(), b0.copy()
+    oracle.outer_sgd_nesterov(wp, wb, g0, 0.7, 0.9, first_step=False)
+    assert np.array_equal(p.cpu().numpy(), wp) and np.array_equal(b.cpu().numpy(), wb) and torch.equal(inner, p)
+    for t, lo in zip(bufs, (shift, shift + 1, shift + 2, shift + 3)):
+        assert bool((t[:lo] == 0).all()) and bool((t[lo + n:] == 0).all())         # nothing written outside the views
+    # from codes held in a byte buffer at an odd address
+    codes, lut = ops.uniform_8bit_quantize(g)
+    cbuf = torch.zeros(n + pad, dtype=torch.uint8, device=dev)
+    cv = cbuf[shift:shift + n]
+    cv.copy_(codes)
+    ops.outer_sgd_nesterov_codes_(p, b, cv, lut, inner, 0.7, 0.9, False)
+    deq = lut.cpu().numpy()[codes.cpu().numpy()]
+    oracle.outer_sgd_nesterov(wp, wb, deq, 0.7, 0.9, first_step=False)
+    assert np.array_equal(p.cpu().numpy(), wp) and np.array_equal(b.cpu().numpy(), wb) and torch.equal(inner, p)
+
+
 class TinyLlama(nn.Module):
     """Parameter names shaped like the reference model's (layers.<i>.*), so the layer bucketing of
     get_offloaded_param (diloco.py:165-167) has something to group."""
