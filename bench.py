@@ -372,13 +372,33 @@ def main() -> int:
         for _ in range(args.steps):
             uniform(x28, c28, l28, qp28)
         tprof = _lib.profile_end()
+        # the ring's reduce step at the same size: acc += lut[codes]; (codes, lut) = uniform_8bit_quantize(acc)
+        acc28 = torch.randn(n28, device=dev, generator=g) * 1e-3
+        keep28 = acc28.clone()
+        co28 = torch.empty(n28, dtype=torch.uint8, device=dev)
+        lo28 = torch.empty(256, dtype=torch.float32, device=dev)
+        r28 = []
+        for it in range(args.warmup + args.steps):
+            acc28.copy_(keep28)                 # every step accumulates onto the rank's own data
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ring_step(acc28, c28, l28, co28, lo28)
+            torch.cuda.synchronize()
+            if it >= args.warmup:
+                r28.append(time.perf_counter() - t0)
+        rs28 = statistics.mean(r28)
+        rg28 = 14.0 * n28 / rs28 / 1e9
         out["tensor_2p28"] = {
             "workload": "uniform_8bit_quantize on one 2^28-element fp32 tensor N(0,1e-3)",
             "value": round(gbs28, 1), "unit": "GB/s", "ms": round(s28 * 1e3, 4),
             "elements_per_s": round(n28 / s28, 1), "frac_of_hbm_peak": round(gbs28 / HBM_PEAK_GBS, 4),
             "kernels": kernel_table(tprof, event_overhead_us),
+            "ring_reduce_step": {"workload": "one ring reduce step on a 2^28-element accumulator (14 bytes per element), "
+                                             "timed call by call with a host synchronisation either side",
+                                 "value": round(rg28, 1), "unit": "GB/s", "ms": round(rs28 * 1e3, 4),
+                                 "frac_of_hbm_peak": round(rg28 / HBM_PEAK_GBS, 4)},
         }
-        del x28, c28
+        del x28, c28, acc28, keep28, co28
         torch.cuda.empty_cache()
 
     if "outer" in legs:
