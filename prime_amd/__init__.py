@@ -9,6 +9,7 @@ Layout
                      the reference's module and function names for this path
     ring.py          the ring's per-hop compute for W simulated ranks on one GPU
     diloco.py        pseudo-gradient, bucketing and outer step around the all-reduce, GPU-resident
+    wire.py          message layout and pinned host staging between the GPU and a host transport
     shim.py          registers these modules under the reference's import paths (zeroband.*)
 """
 from .config import Compression  # noqa: F401

@@ -1,0 +1,197 @@
+"""What crosses the wire in the ring, and the pinned host buffers between the GPU and a host
+transport.
+
+The reference sends, per step, two tensors to the next rank (src/zeroband/C/csrc/collectives.cpp:140-150):
+
+    lookup   float32[256]            tag step + 1000
+    codes    uint8[chunk numel]      tag step
+
+through ``group->send`` / ``group->recv`` of a c10d process group (Gloo: host memory), with
+BUFFER_COUNT = 2 slots in flight (:6, :118-122).  Its tensors already live in host memory.  Here
+codes and lookup are produced on the GPU, so each rank keeps
+
+    send slots   pinned host memory, filled by asynchronous device-to-host copies on a copy stream
+    recv slots   pinned host memory the transport writes into, drained by host-to-device copies
+    device recv  the buffers the ring-step kernels read
+
+and only uint8 codes + 1 KiB cross PCIe (a quarter of the fp32 chunk).  Copies run on their own
+HIP stream of default priority and are ordered against the compute stream with events, so the
+copy of step s overlaps the kernels of step s + 1, as the reference overlaps its sends with
+the next quantization.
+
+No transport is built here (one GPU, no process group): ``Loopback`` stands in for the pair of
+``send`` / ``recv`` calls between neighbours by copying host slot to host slot, which is enough
+to run the whole schedule through the staging path and to time the PCIe side.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from . import ops
+from .ring import BUFFER_COUNT, _check_ring_inputs
+
+LOOKUP_TAG_OFFSET = 1000      # collectives.cpp:141,144
+N_BINS = ops.N_BINS
+
+
+def message_tags(step: int) -> Tuple[int, int]:
+    """(tag of the lookup table, tag of the codes) for one step (collectives.cpp:141,147)."""
+    return step + LOOKUP_TAG_OFFSET, step
+
+
+class HostStage:
+    """One rank's staging buffers for chunks of ``chunk_numel`` elements."""
+
+    def __init__(self, device: torch.device, chunk_numel: int, depth: int = BUFFER_COUNT):
+        self.device = torch.device(device)
+        self.chunk_numel = int(chunk_numel)
+        self.depth = int(depth)
+        self.copy_stream = torch.cuda.Stream(self.device)
+
+        def pinned(shape, dtype):
+            return torch.empty(shape, dtype=dtype, pin_memory=True)
+
+        with torch.cuda.device(self.device):
+            self.send_codes = [pinned(self.chunk_numel, torch.uint8) for _ in range(self.depth)]
+            self.send_lut = [pinned(N_BINS, torch.float32) for _ in range(self.depth)]
+            self.recv_codes = [pinned(self.chunk_numel, torch.uint8) for _ in range(self.depth)]
+            self.recv_lut = [pinned(N_BINS, torch.float32) for _ in range(self.depth)]
+            self.dev_codes = [torch.empty(self.chunk_numel, dtype=torch.uint8, device=self.device) for _ in range(self.depth)]
+            self.dev_lut = [torch.empty(N_BINS, dtype=torch.float32, device=self.device) for _ in range(self.depth)]
+        self._d2h_done: List[Optional[torch.cuda.Event]] = [None] * self.depth
+        self._h2d_done: List[Optional[torch.cuda.Event]] = [None] * self.depth
+        self._consumed: List[Optional[torch.cuda.Event]] = [None] * self.depth
+        self._keep: List[tuple] = [()] * self.depth       # device tensors a copy in flight still reads
+
+    # ---- sending -------------------------------------------------------------------------------
+    def post_send(self, step: int, codes: torch.Tensor, lut: torch.Tensor) -> None:
+        """Start the device-to-host copy of one message; the kernels that produced it are on the
+        current stream.  The slot must have been taken by the transport (``take_send``) before it is
+        reused, BUFFER_COUNT steps later."""
+        if codes.numel() != self.chunk_numel or codes.dtype != torch.uint8 or lut.numel() != N_BINS or lut.dtype != torch.float32:
+            raise RuntimeError("post_send: a message is uint8 codes of the chunk size and 256 float32 lookup entries")
+        slot = step % self.depth
+        ready = torch.cuda.current_stream(self.device).record_event()
+        self.copy_stream.wait_event(ready)
+        with torch.cuda.stream(self.copy_stream):
+            self.send_lut[slot].copy_(lut.view(-1), non_blocking=True)
+            self.send_codes[slot].copy_(codes.view(-1), non_blocking=True)
+            self._d2h_done[slot] = self.copy_stream.record_event()
+        self._keep[slot] = (codes, lut)
+
+    def take_send(self, step: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Block until the message of ``step`` is in host memory; returns (lookup, codes), the two
+        host tensors to hand to ``send`` with ``message_tags(step)``."""
+        slot = step % self.depth
+        ev = self._d2h_done[slot]
+        if ev is None:
+            raise RuntimeError(f"no message was posted for step {step}")
+        ev.synchronize()
+        self._keep[slot] = ()
+        return self.send_lut[slot], self.send_codes[slot]
+
+    # ---- receiving -----------------------------------------------------------------------------
+    def recv_buffers(self, step: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(lookup, codes) host tensors for ``recv`` with ``message_tags(step)``.  Blocks until the
+        host-to-device copy that last read this slot has finished."""
+        slot = step % self.depth
+        if self._h2d_done[slot] is not None:
+            self._h2d_done[slot].synchronize()
+        return self.recv_lut[slot], self.recv_codes[slot]
+
+    def to_device(self, step: int) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Start the host-to-device copy of the received message of ``step`` and order the current
+        stream after it; returns (codes, lookup) on the device."""
+        slot = step % self.depth
+        if self._consumed[slot] is not None:
+            self.copy_stream.wait_event(self._consumed[slot])      # the kernels that read this device slot last
+        with torch.cuda.stream(self.copy_stream):
+            self.dev_lut[slot].copy_(self.recv_lut[slot], non_blocking=True)
+            self.dev_codes[slot].copy_(self.recv_codes[slot], non_blocking=True)
+            self._h2d_done[slot] = self.copy_stream.record_event()
+        torch.cuda.current_stream(self.device).wait_event(self._h2d_done[slot])
+        return self.dev_codes[slot], self.dev_lut[slot]
+
+    def release(self, step: int) -> None:
+        """The kernels reading the device slot of ``step`` have been enqueued on the current stream."""
+        self._consumed[step % self.depth] = torch.cuda.current_stream(self.device).record_event()
+
+
+class Loopback:
+    """Stand-in for the neighbour-to-neighbour ``send`` / ``recv`` pair: host memory to host
+    memory inside one process.  ``bytes_moved`` counts what a real transport would carry."""
+
+    def __init__(self):
+        self.bytes_moved = 0
+        self.messages = 0
+
+    def deliver(self, src: HostStage, dst: HostStage, step: int) -> None:
+        lut, codes = src.take_send(step)
+        rl, rc = dst.recv_buffers(step)
+        rl.copy_(lut)
+        rc.copy_(codes)
+        self.bytes_moved += lut.numel() * 4 + codes.numel()
+        self.messages += 2            # two tensors per step, tags step + 1000 and step
+
+
+def ring_allreduce_staged(tensors: Sequence[torch.Tensor], avg: bool = False, transport: Optional[Loopback] = None,
+                          stages: Optional[Sequence[HostStage]] = None) -> Loopback:
+    """``ring_allreduce`` (collectives.cpp:76-230) for ``len(tensors)`` simulated ranks with every
+    message taking the path of a host transport: GPU -> pinned host (sender) -> transport ->
+    pinned host (receiver) -> GPU.  Same kernels and schedule as
+    ``prime_amd.ring.ring_allreduce_simulated``, so the results are identical to it."""
+    W = len(tensors)
+    n = _check_ring_inputs(tensors)
+    nb = BUFFER_COUNT * W
+    csz = n // nb
+    flats = [t.view(-1) for t in tensors]
+    dev = flats[0].device
+    transport = transport or Loopback()
+    if stages is None:
+        stages = [HostStage(dev, csz) for _ in range(W)]
+    if len(stages) != W or any(s.chunk_numel != csz for s in stages):
+        raise ValueError("one HostStage per rank, sized for the chunk, is needed")
+
+    def chunk(r: int, c: int) -> torch.Tensor:
+        return flats[r][c * csz:(c + 1) * csz]
+
+    own: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
+    for phase in (1, 2):
+        arrived = [set() for _ in range(W)]
+        for step in range(1, nb + 1):
+            posted = []
+            for r in range(W):
+                c = ((r * BUFFER_COUNT - step) if phase == 1 else (r * BUFFER_COUNT + BUFFER_COUNT - step)) % nb   # :116 / :192
+                ch = chunk(r, c)
+                got = (step - BUFFER_COUNT) in arrived[r]
+                sending = step <= (W - 1) * BUFFER_COUNT                                                        # :136 / :212
+                out = None
+                if got:
+                    arrived[r].discard(step - BUFFER_COUNT)
+                    codes_in, lut_in = stages[r].to_device(step - BUFFER_COUNT)
+                    if sending:
+                        out = (ops.ring_reduce_step if phase == 1 else ops.ring_gather_step)(ch, codes_in, lut_in)
+                    elif phase == 1:
+                        own[(r, c)] = ops.ring_reduce_div_step(ch, codes_in, lut_in, float(W) if avg else 1.0)
+                    else:
+                        ops.dequantize_(ch, codes_in, lut_in, False)
+                    stages[r].release(step - BUFFER_COUNT)
+                elif sending and (r, c) in own:
+                    out = ops.ring_gather_step(ch, *own.pop((r, c)))
+                elif sending:
+                    out = ops.uniform_8bit_quantize(ch, False)
+                if out is not None:
+                    stages[r].post_send(step, out[0], out[1])
+                    posted.append(r)
+            for r in posted:                       # the transport: rank r -> rank r + 1
+                transport.deliver(stages[r], stages[(r + 1) % W], step)
+                arrived[(r + 1) % W].add(step)
+        if phase == 1 and W == 1:
+            for i in range(BUFFER_COUNT):
+                ch = chunk(0, i)
+                codes, lut = ops.uniform_8bit_quantize(ch, True)
+                ops.dequantize_(ch, codes, lut, False)
+    assert not own
+    return transport

@@ -1,0 +1,83 @@
+"""Wire format and host staging of the ring's messages (src/zeroband/C/csrc/collectives.cpp:140-150):
+uint8 codes with tag ``step`` and a 256-entry float32 lookup with tag ``step + 1000``, through pinned
+host double buffers, with a host-to-host loopback in place of the neighbour's send / recv."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import announce
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(W, n, seed):
+    rng = np.random.default_rng(seed)
+    return [(rng.standard_normal(n) * 10).astype(np.float32) for _ in range(W)]
+
+
+def test_message_tags_and_slot_contents(dev):
+    from prime_amd import ops, wire
+
+    assert wire.message_tags(7) == (1007, 7) and wire.BUFFER_COUNT == 2
+    n = 50_000
+    stage = wire.HostStage(dev, n)
+    x = torch.randn(n, device=dev)
+    announce("host stage round trip")
+    codes, lut = ops.uniform_8bit_quantize(x)
+    stage.post_send(3, codes, lut)
+    h_lut, h_codes = stage.take_send(3)
+    assert h_lut.is_pinned() and h_codes.is_pinned() and not h_lut.is_cuda
+    assert h_lut.dtype == torch.float32 and h_lut.shape == (256,) and h_codes.dtype == torch.uint8 and h_codes.shape == (n,)
+    assert torch.equal(h_codes, codes.cpu()) and torch.equal(h_lut, lut.cpu())
+    # the receiving side: host slot -> device slot, usable by a ring step on the current stream
+    r_lut, r_codes = stage.recv_buffers(3)
+    r_lut.copy_(h_lut)
+    r_codes.copy_(h_codes)
+    d_codes, d_lut = stage.to_device(3)
+    acc = torch.zeros(n, device=dev)
+    ops.dequantize_(acc, d_codes, d_lut, True)
+    stage.release(3)
+    torch.cuda.synchronize()
+    assert torch.equal(acc, lut[codes.long()])
+    with pytest.raises(RuntimeError, match="posted"):
+        wire.HostStage(dev, n).take_send(1)
+    with pytest.raises(RuntimeError, match="uint8 codes"):
+        stage.post_send(4, codes[:10], lut)
+
+
+@pytest.mark.parametrize("W,avg", [(1, False), (2, False), (3, True), (4, True), (8, False)])
+def test_staged_ring_equals_the_simulated_ring(dev, W, avg):
+    # same kernels, same schedule; every message goes GPU -> pinned host -> loopback -> pinned host -> GPU
+    from prime_amd import ring, wire
+
+    n = 2 * W * 25_000
+    xs = _inputs(W, n, 300 + W)
+    direct = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    staged = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    announce(f"staged ring W={W} avg={avg}")
+    ring.ring_allreduce_simulated(direct, avg=avg)
+    transport = wire.ring_allreduce_staged(staged, avg=avg)
+    torch.cuda.synchronize()
+    for a, b in zip(direct, staged):
+        assert torch.equal(a, b)
+    # per rank and phase (W - 1) * BUFFER_COUNT steps send two tensors each
+    steps = 2 * W * (W - 1) * 2
+    assert transport.messages == 2 * steps
+    assert transport.bytes_moved == steps * (n // (2 * W) + 1024)
+
+
+def test_staged_ring_reuses_its_stages_across_calls(dev):
+    from prime_amd import ring, wire
+
+    W, n = 2, 4 * 60_000
+    stages = [wire.HostStage(dev, n // (2 * W)) for _ in range(W)]
+    for seed in (1, 2, 3):
+        xs = _inputs(W, n, seed)
+        direct = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+        staged = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+        ring.ring_allreduce_simulated(direct)
+        wire.ring_allreduce_staged(staged, stages=stages)
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip(direct, staged))
+    with pytest.raises(ValueError, match="HostStage"):
+        wire.ring_allreduce_staged(staged, stages=stages[:1])
