@@ -359,3 +359,48 @@ def test_uncompressed_simulated_all_reduce_and_fake_step(dev):
     d.step(model, group=SimulatedRing([d.grad_flat]), world_size=1, fake=True)     # fake: zero pseudo-gradient (:95-96)
     for p, q in zip(model.parameters(), before):
         assert torch.equal(p.detach(), q)
+
+
+def test_outer_step_with_a_real_process_group_of_one_rank(dev, oracle, tmp_path):
+    # the reference's call site unchanged: all_reduce(Compression.UINT8, bucket, SUM, group) on the default
+    # process group; with one rank no message is sent, but every bucket's two chunks still take the lossy
+    # quantize / dequantize round trip (collectives.cpp:161-173)
+    import torch.distributed as dist
+
+    from prime_amd.collectives import Compression, all_reduce
+    from prime_amd.diloco import Diloco
+
+    assert not dist.is_initialized()
+    dist.init_process_group("gloo", init_method=f"file://{tmp_path}/rendezvous", rank=0, world_size=1)
+    try:
+        rng = np.random.default_rng(8)
+        x = (rng.standard_normal(40_000) * 1e-3).astype(np.float32)
+        t = torch.from_numpy(x.copy()).to(dev)
+        announce("one-rank process group: all_reduce")
+        all_reduce(Compression.UINT8, t, dist.ReduceOp.SUM)              # group=None: the default group
+        want = [x.copy()]
+        oracle.ring_allreduce_sim(want)
+        assert np.allclose(t.cpu().numpy(), want[0], rtol=2e-6, atol=1e-9)
+        half = x.size // 2
+        assert len(np.unique(t.cpu().numpy()[:half])) <= 256 and len(np.unique(t.cpu().numpy()[half:])) <= 256
+        # a whole outer step of one worker through Diloco.step, world size taken from the group
+        torch.manual_seed(3)
+        model = TinyLlama().to(dev)
+        d = Diloco(0.7, model)
+        before = d.outer_data_flat.clone()
+        for p in model.parameters():
+            p.data.add_(torch.randn_like(p) * 1e-3)
+        inner = torch.cat([p.detach().reshape(-1) for p in model.parameters()])
+        announce("one-rank process group: Diloco.step")
+        d.step(model)
+        torch.cuda.synchronize()
+        # first outer step of SGD with Nesterov momentum: p -= lr * (1 + mu) * g, with g the quantized (outer - inner)
+        g_exact = before - inner
+        moved = before - d.outer_data_flat
+        err = (moved - 0.7 * 1.9 * g_exact).abs() / (0.7 * 1.9)
+        bin_width = 6 * 1e-3 / 256                   # per bucket about this: 6 sigma over 256 bins
+        assert float((err > 1.2 * bin_width).float().mean()) < 0.01        # all but the clipped tails (beyond 3 sigma)
+        assert float(err.mean()) < 0.5 * bin_width
+        assert torch.equal(torch.cat([p.detach().reshape(-1) for p in model.parameters()]), d.outer_data_flat)
+    finally:
+        dist.destroy_process_group()
