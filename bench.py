@@ -253,7 +253,25 @@ def main() -> int:
     launches_per_bucket = sum(v["launches"] for v in prof.values()) / (args.steps * N_LAYERS)
     bracketed_us_per_bucket = sum(v["total_ms"] for v in prof.values()) * 1e3 / (args.steps * N_LAYERS)
     wall_us_per_bucket = sec * 1e6 / N_LAYERS
-    event_overhead_us = max(0.0, (bracketed_us_per_bucket - wall_us_per_bucket) / launches_per_bucket)
+    overhead_from_buckets_us = max(0.0, (bracketed_us_per_bucket - wall_us_per_bucket) / launches_per_bucket)
+    # The same difference on a kernel long enough (about 100 us) that the host can never fall behind, also
+    # under a profiler, where launching the 4 us second-stage kernels back to back leaves gaps: 20 copies
+    # of 256 MiB bracketed, against the same 20 back to back.
+    cal_src = torch.empty(1 << 26, dtype=torch.float32, device=dev).normal_()
+    cal_dst = torch.empty_like(cal_src)
+
+    def cal_copy():
+        _lib.check(lib.prime_copy_bytes(cal_dst.data_ptr(), cal_src.data_ptr(), cal_src.numel() * 4, st), "copy_bytes")
+
+    cal_wall = timed(cal_copy, 20, 3)
+    _lib.profile_begin()
+    for _ in range(20):
+        cal_copy()
+    cal_prof = _lib.profile_end()["copy_kernel"]
+    overhead_from_copies_us = max(0.0, cal_prof["total_ms"] / cal_prof["launches"] * 1e3 - cal_wall * 1e6)
+    del cal_src, cal_dst
+    event_overhead_us = min(overhead_from_buckets_us, overhead_from_copies_us) if overhead_from_buckets_us > 0 \
+        else overhead_from_copies_us
     dom = prof["quantize_kernel+hist"]
     dom_event_us = dom["total_ms"] / dom["launches"] * 1e3
     dom_us = dom_event_us - event_overhead_us
@@ -299,6 +317,8 @@ def main() -> int:
         "avg_launch_us": round(dom_us, 2),
         "avg_launch_us_event_bracket": round(dom_event_us, 2),
         "event_overhead_us": round(event_overhead_us, 2),
+        "event_overhead_us_from_bucket_sequence": round(overhead_from_buckets_us, 2),
+        "event_overhead_us_from_long_copies": round(overhead_from_copies_us, 2),
         "last_level_cache": {
             "note": "achieved is algorithmic bytes over the launch time as the job runs: the statistics pass has just "
                     "streamed the bucket through the 256 MB last-level cache, which serves part of this pass",
