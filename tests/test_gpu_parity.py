@@ -401,6 +401,34 @@ def test_literal_norm_against_the_compiled_reference_at_2p24(abi, oracle):
     assert -2e-3 < rel < -1e-4
 
 
+@pytest.mark.parametrize("name", ["normal:1048583", "student:4194304", "normal:16777216"])
+def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, name):
+    # fixtures that travel without the reference: scale bits, SHA-256 of the codes and code populations of
+    # the compiled reference at sizes up to the benchmark's first configuration (2^24 elements)
+    import hashlib
+    import json
+    from pathlib import Path
+
+    want = json.loads((Path(__file__).parent / "golden" / "uniform8_reference_large.json").read_text())[name]
+    x = case_input(name)
+    announce(f"large golden {name}")
+    codes, lut, qp = abi.uniform_literal(abi.to_dev(x))
+    torch.cuda.synchronize()
+    q = abi.qparams(qp)
+    assert int(np.array([q["scale"]], np.float32).view(np.uint32)[0]) == want["scale_bits"]
+    gc = codes.cpu().numpy()
+    assert hashlib.sha256(gc.tobytes()).hexdigest() == want["codes_sha256"]
+    assert np.bincount(gc, minlength=256).tolist() == want["counts"]
+    ref_lut = np.array(want["lut"], np.float32)
+    assert lut_rel_err(lut.cpu().numpy(), ref_lut.astype(np.float64), float(q["scale"])) < 2e-5
+    # the default path uses the exact norm: same codes for all but the elements the scale difference moves
+    codes_e, _, qp_e = abi.uniform(abi.to_dev(x))
+    rel = float(q["scale"]) / float(abi.qparams(qp_e)["scale"]) - 1
+    assert -2e-3 < rel <= 0
+    moved = (codes_e.cpu().numpy() != gc).mean()
+    assert moved <= 45 * abs(rel) + 1e-6          # a code moves when |x| / scale crosses a boundary: at most ~|code - 128| * |rel|
+
+
 def test_results_do_not_depend_on_scheduling(abi):
     announce("determinism")
     x = torch.randn(3_000_001, device=abi.dev) * 1e-3

@@ -354,3 +354,28 @@ def test_outer_sgd_nesterov_is_torch_sgd_bit_for_bit(oracle):
                 oracle.outer_sgd_nesterov(mine, buf, g, lr, mu, first_step=(step == 0))
                 assert np.array_equal(mine, p.detach().numpy()), (n, lr, mu, step)
                 assert np.array_equal(buf, opt.state[p]["momentum_buffer"].numpy()), (n, lr, mu, step)
+
+
+@pytest.mark.parametrize("name", ["normal:1048583", "student:4194304", "normal:16777216"])
+def test_oracle_reproduces_the_large_digests_of_the_compiled_reference(oracle, name):
+    # sizes where libtorch's norm visibly differs from the exact one: the literal restatement must give
+    # the reference's scale bits and codes (SHA-256 and populations written by tests/golden/make_fixtures.py)
+    import hashlib
+    import json
+    from pathlib import Path
+
+    from tests.golden.make_fixtures import case_input
+
+    want = json.loads((Path(__file__).parent / "golden" / "uniform8_reference_large.json").read_text())[name]
+    x = case_input(name)
+    assert hashlib.sha256(x.tobytes()).hexdigest() == want["input_sha256"]      # the generator still draws the same input
+    assert int(np.array([oracle.norm_literal(x)], np.float32).view(np.uint32)[0]) == want["norm_bits"]
+    codes, lut, scale = oracle.uniform_8bit_quantize(x, "literal")
+    assert int(np.array([scale], np.float32).view(np.uint32)[0]) == want["scale_bits"]
+    assert hashlib.sha256(codes.tobytes()).hexdigest() == want["codes_sha256"]
+    assert np.bincount(codes, minlength=256).tolist() == want["counts"]
+    ref_lut = np.array(want["lut"], np.float32)
+    assert np.abs(lut - ref_lut).max() <= 2e-5 * max(float(scale), np.abs(ref_lut).max())
+    # and the exact scale is larger, by libtorch's accumulation loss
+    rel = float(scale) / float(oracle.scale_exact(x)) - 1
+    assert -2e-3 < rel <= 0
