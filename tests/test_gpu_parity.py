@@ -429,6 +429,34 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
     assert moved <= 45 * abs(rel) + 1e-6          # a code moves when |x| / scale crosses a boundary: at most ~|code - 128| * |rel|
 
 
+@pytest.mark.parametrize("option,values", [("hist_replicas", (1, 2, 4, 8, 16)), ("blocks_per_cu", (1, 2, 3, 4)),
+                                           ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20))])
+def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle, option, values):
+    # the options change scheduling and cache hints only: codes, scale and lookup must not move,
+    # on ordinary data, on a tensor crowded into a few codes, and through a ring step
+    rng = np.random.default_rng(31)
+    n = 700_001
+    inputs = {"normal": (rng.standard_normal(n) * 1e-3).astype(np.float32),
+              "near one": (1 + rng.standard_normal(n) * 1e-2).astype(np.float32)}
+    old = _lib.get_option(option)
+    try:
+        for value in values:
+            _lib.set_option(option, value)
+            for label, x in inputs.items():
+                xt, codes, lut, q = check_uniform(abi, oracle, x, f"{option}={value} {label}")
+                acc = abi.to_dev(inputs["normal"][::-1].copy())
+                c2, l2, qp2 = abi.ring_step(acc, codes, lut)
+                want = inputs["normal"][::-1].copy()
+                oracle.index_add(want, lut.cpu().numpy(), codes.cpu().numpy())
+                assert np.array_equal(acc.cpu().numpy(), want)
+                q2 = abi.qparams(qp2)
+                assert q2["scale"] == oracle.scale_exact(want)
+                oc2, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q2["scale"]))
+                assert np.array_equal(c2.cpu().numpy(), oc2)
+    finally:
+        _lib.set_option(option, old)
+
+
 def test_results_do_not_depend_on_scheduling(abi):
     announce("determinism")
     x = torch.randn(3_000_001, device=abi.dev) * 1e-3
