@@ -138,3 +138,14 @@ def test_shim_registers_the_reference_import_paths():
         for k in [k for k in sys.modules if k == "zeroband" or k.startswith("zeroband.")]:
             del sys.modules[k]
         sys.modules.update({k: v for k, v in had.items() if v is not None})
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # one GPU per box: the benchmark says so instead of pretending to scale
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 2 and "one GPU" in res.stderr and res.stdout.strip() == ""
