@@ -115,6 +115,31 @@ def test_outer_step_kernels_on_element_aligned_views(dev, oracle, shift):
     assert np.array_equal(p.cpu().numpy(), wp) and np.array_equal(b.cpu().numpy(), wb) and torch.equal(inner, p)
 
 
+def test_division_kernels_keep_denormals_like_the_cpu(dev, oracle):
+    # pseudo-gradients of converged parameters can be denormal: (outer - inner) / W and chunk / W must round
+    # as the CPU does, not flush to zero
+    from prime_amd import ops
+
+    rng = np.random.default_rng(0)
+    n = 4099
+    a = (rng.standard_normal(n) * 1e-38).astype(np.float32)
+    b = (rng.standard_normal(n) * 1e-38).astype(np.float32)
+    a[:8] = [1e-38, 3e-39, 1e-45, 0, -0.0, 2e-38, 1.1754944e-38, -1e-44]
+    b[:8] = [0, 1e-39, 0, 0, 0, 1e-38, 1e-45, 1e-45]
+    announce("denormal division")
+    for W in (2.0, 3.0, 8.0, 14.0):
+        out = torch.empty(n, device=dev)
+        ops.pseudo_gradient_(out, torch.from_numpy(a).to(dev), torch.from_numpy(b).to(dev), W)
+        want = oracle.pseudo_gradient(a, b, W)
+        assert (np.abs(want) < 1.1754944e-38).sum() > n // 2 and np.count_nonzero(want) > n // 2
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        t = torch.from_numpy(a.copy()).to(dev)
+        ops.div_(t, W)
+        w2 = a.copy()
+        oracle.div_scalar(w2, W)
+        assert np.array_equal(t.cpu().numpy().view(np.uint32), w2.view(np.uint32))
+
+
 class TinyLlama(nn.Module):
     """Parameter names shaped like the reference model's (layers.<i>.*), so the layer bucketing of
     get_offloaded_param (diloco.py:165-167) has something to group."""
