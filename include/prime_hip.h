@@ -102,6 +102,17 @@ int prime_quantize_lookup_u8(const float* x, int64_t n, float scale, uint8_t* co
 int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float* lut,
                                 prime_qparams* qparams_out, void* ws, prime_stream_t stream);
 
+/* prime_uniform_8bit_quantize for callers that cannot allocate device memory or carry a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): no counterpart in the reference.  The per-workgroup partials live in a scratch
+ * array inside the library's own device image (8 MiB + 35 KiB per GPU, held until the process
+ * ends; its address is looked up once per device on the first call there).  Calls no hipMalloc,
+ * hipFree or other allocating routine.  Same results as prime_uniform_8bit_quantize, bit for
+ * bit.  n above 2^40 is rejected with PRIME_EINVAL.  All calls on one GPU share that GPU's
+ * array: calls that overlap on one GPU (two streams, two threads) race; order them. */
+int prime_uniform_8bit_quantize_noalloc(const float* x, int64_t n, uint8_t* codes, float* lut,
+                                        prime_qparams* qparams_out, prime_stream_t stream);
+
 /* The norm as the reference receives it from libtorch's CPU kernel at compression.cpp:113
  * (eight serial fp32 fused-multiply-add lanes, lanes added in order, scalar tail, sqrtf: the
  * order observed in libtorch 2.10 on x86-64 with 256-bit vectors), and the scale of :113-116

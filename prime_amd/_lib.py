@@ -59,6 +59,7 @@ SIGNATURES = {
     "prime_average_buckets": (ctypes.c_int, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp]),
     "prime_quantize_lookup_u8": (ctypes.c_int, [_vp, _i64, _f32, _vp, _vp, _vp, _vp]),
     "prime_uniform_8bit_quantize": (ctypes.c_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "prime_uniform_8bit_quantize_noalloc": (ctypes.c_int, [_vp, _i64, _vp, _vp, _vp, _vp]),
     "prime_uniform_8bit_quantize_buckets": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, ctypes.c_int]),
     "prime_uniform_8bit_quantize_batched": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp]),
     "prime_dequant_set": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp]),

@@ -68,6 +68,30 @@ def kernel_resources() -> dict:
     return out
 
 
+def device_data_symbols() -> dict:
+    """Data objects of the gfx950 code object as the production flags compile it:
+    {symbol name: {"size", "bind"}}.  A __device__ variable that host code looks up by symbol
+    (hipGetSymbolAddress) must be GLOBAL there: the runtime resolves it through the code object's
+    dynamic symbols and aborts the process when the name is missing."""
+    import tempfile
+
+    flags = [f for f in HIPCC_FLAGS if f not in ("-shared", "-fPIC")]
+    llvm = Path("/opt/rocm/llvm/bin")
+    with tempfile.TemporaryDirectory() as tmp:
+        obj, co = Path(tmp) / "device.o", Path(tmp) / "device.co"
+        subprocess.run(["hipcc", *flags, "--cuda-device-only", "-c", *map(str, SOURCES), "-o", str(obj)],
+                       check=True, capture_output=True)
+        subprocess.run([str(llvm / "clang-offload-bundler"), "--unbundle", "--type=o", f"--input={obj}",
+                        "--targets=hip-amdgcn-amd-amdhsa--gfx950", f"--output={co}"], check=True, capture_output=True)
+        res = subprocess.run([str(llvm / "llvm-readelf"), "--dyn-syms", str(co)], check=True, capture_output=True, text=True)
+    out = {}
+    for line in res.stdout.splitlines():
+        f = line.split()
+        if len(f) == 8 and f[3] == "OBJECT" and not f[7].endswith(".kd"):
+            out[f[7]] = {"size": int(f[2]), "bind": f[4]}
+    return out
+
+
 if __name__ == "__main__":
     build()
     sys.exit(0)

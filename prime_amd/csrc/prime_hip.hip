@@ -247,6 +247,39 @@ bool bad_n(int64_t n) { return n < 0 || n > kMaxElems; }
 
 }  // namespace
 
+// Scratch of the entry point that allocates nothing: one Workspace per GPU in the code object's
+// own device memory (8 MiB + 35 KiB, held by every device the library runs on until the process
+// ends).  In host code the array's name is only a stand-in for the symbol, not a device address:
+// the address is looked up once per device with hipGetSymbolAddress, kept, and every launch and
+// every other use of the memory gets that pointer.
+static __device__ __align__(256) unsigned char scratch[sizeof(Workspace)];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// *out = the current device's copy of `scratch`.  Returns 0, or the error code (text set).
+int scratch_workspace(Workspace** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(PRIME_EINVAL, "device index out of range for the built-in scratch");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        if (!ptr) return fail(PRIME_EWORKSPACE, "hipGetSymbolAddress(scratch) returned a null address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = static_cast<Workspace*>(g_scratch_ptr[dev]);
+    return 0;
+}
+
+}  // namespace
+
 extern "C" {
 
 int prime_hip_abi_version(void) { return PRIME_HIP_ABI_VERSION; }
@@ -397,6 +430,17 @@ int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float
     if (int rc = run_stats_partials(x, n, w, st, &parts)) return rc;
     if (int rc = run_quantize(x, n, 0.0f, parts, qparams_out, kZeroPoint, codes, w, true, st, &grid)) return rc;
     return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
+}
+
+int prime_uniform_8bit_quantize_noalloc(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out,
+                                        prime_stream_t stream) {
+    if (n > kMaxElems) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_noalloc: n exceeds the 2^40 elements the built-in scratch is laid out for");
+    if (n < 0 || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_noalloc: bad argument");
+    Workspace* w = nullptr;
+    if (int rc = scratch_workspace(&w)) return rc;
+    // Nothing in the workspace has to start at zero: every partial a kernel reads was stored by the
+    // kernel before it in this same call.
+    return prime_uniform_8bit_quantize(x, n, codes, lut, qparams_out, w, stream);
 }
 
 int prime_norm_literal_f32(const float* x, int64_t n, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {

@@ -84,3 +84,18 @@ def test_no_kernel_spills_and_streaming_kernels_keep_full_occupancy():
     for name, v in res.items():
         if any(s in name for s in streaming):
             assert v["occupancy"] == 8 and v["vgprs"] <= 64, (name, v)
+
+
+def test_built_in_scratch_is_a_dynamic_symbol_of_the_code_object():
+    # the entry point that allocates nothing finds its scratch with hipGetSymbolAddress, which
+    # resolves the name in the code object's dynamic symbols (and aborts when it is missing):
+    # the array has to be exported there, at the size of one workspace
+    from prime_amd import _lib
+    from prime_amd.build import device_data_symbols
+
+    syms = device_data_symbols()
+    scratch = {k: v for k, v in syms.items() if "scratch" in k}
+    assert len(scratch) == 1, syms
+    (info,) = scratch.values()
+    assert info["bind"] == "GLOBAL"
+    assert info["size"] == _lib.load().prime_workspace_bytes()
