@@ -105,6 +105,34 @@ template <bool NT> struct Mem<false, NT> {
     }
 };
 
+// Cache policy of a streamed store (the cache-policy bits of gfx950 memory instructions).
+// Write-through (agent scope: the line leaves the XCD's L2 at once instead of waiting there,
+// dirty, for an eviction that then competes with the read stream) is the fastest for the code
+// and fp32 outputs that sit beside a larger read stream; non-temporal is the fastest for a plain
+// copy far larger than the last-level cache; plain write-back is best when the next kernel reads
+// the data back at once.
+constexpr int kStorePlain = 0;
+constexpr int kStoreNt = 2;              // nt
+constexpr int kStoreWriteThrough = 16;   // sc1
+
+// A window of a buffer for buffer instructions: a wave-uniform base plus a 32-bit byte offset
+// per lane.  The hardware drops stores and returns zero for loads at or beyond `bytes`.
+struct Window {
+    __amdgpu_buffer_rsrc_t rsrc;
+    __device__ __forceinline__ Window(const void* base, int64_t bytes) {
+        const int64_t lim = bytes < 0 ? 0 : (bytes > 0x7fffffff ? 0x7fffffff : bytes);
+        rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(lim), 0x00020000);
+    }
+    template <int POLICY>
+    __device__ __forceinline__ void st32(uint32_t byte_off, uint32_t v) const {
+        __builtin_amdgcn_raw_buffer_store_b32(v, rsrc, static_cast<int>(byte_off), 0, POLICY);
+    }
+    template <int POLICY>
+    __device__ __forceinline__ void st128(uint32_t byte_off, f4a v) const {
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4a, v), rsrc, static_cast<int>(byte_off), 0, POLICY);
+    }
+};
+
 __device__ __forceinline__ double wave_sum(double v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
@@ -225,15 +253,27 @@ __device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int np
 // main part): unless it is set, each vector needs the check i < nvec.
 // U is the number of vectors body handles per call (kUnroll unless the kernel needs the registers:
 // the kernels that divide keep two operands per vector and a division sequence live).
-template <int U = kUnroll, typename Body>
-__device__ __forceinline__ void sweep(int64_t nvec, Body&& body) {
+// sweep_tiles hands body the workgroup-uniform first vector of the piece (the lane adds threadIdx.x),
+// which a buffer window needs as its base, and with REVERSE walks the tensor from its end: a pass that
+// re-reads what the pass before it has just streamed then starts with the part the last-level
+// cache still holds instead of the part that has already been displaced.
+template <int U = kUnroll, bool REVERSE = false, typename Body>
+__device__ __forceinline__ void sweep_tiles(int64_t nvec, Body&& body) {
     const int64_t G = gridDim.x;
     const int64_t rows = (nvec + kThreads - 1) / kThreads;
     const int64_t rounds = (nvec / kThreads) / (G * U);
-    for (int64_t k = 0; k < rounds; ++k)
-        body(((k * G + blockIdx.x) * U) * kThreads + threadIdx.x, static_cast<int64_t>(kThreads), std::true_type{});
     const int64_t r0 = rounds * G * U + blockIdx.x;
-    if (r0 < rows) body(r0 * kThreads + threadIdx.x, G * kThreads, std::false_type{});
+    if (REVERSE && r0 < rows) body(r0 * kThreads, G * kThreads, std::false_type{});
+    for (int64_t kk = 0; kk < rounds; ++kk) {
+        const int64_t k = REVERSE ? rounds - 1 - kk : kk;
+        body(((k * G + blockIdx.x) * U) * kThreads, static_cast<int64_t>(kThreads), std::true_type{});
+    }
+    if (!REVERSE && r0 < rows) body(r0 * kThreads, G * kThreads, std::false_type{});
+}
+
+template <int U = kUnroll, typename Body>
+__device__ __forceinline__ void sweep(int64_t nvec, Body&& body) {
+    sweep_tiles<U, false>(nvec, [&](int64_t base, int64_t stride, auto full_t) { body(base + threadIdx.x, stride, full_t); });
 }
 
 __device__ __forceinline__ void stats_add4(const f4a v, double& s, double& q) {
@@ -264,6 +304,123 @@ __device__ __forceinline__ void hist_add(LdsHist<R>& h, int code, float x) {
     const int slot = code * R + (threadIdx.x & (R - 1));
     __hip_atomic_fetch_add(&h.sum[slot], static_cast<double>(x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     __hip_atomic_fetch_add(&h.cnt[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// Histogram of the quantize pass in fixed point: one 64-bit LDS atomic per element.  An element with
+// code c lies d = x * inv - (c - 128) bins from the centre of its bin (|d| <= 1/2 unless c is 0 or
+// 255, where the clipped elements collect); the bin's sum of x is ((c - 128) * count + sum of d) / inv.
+// d comes from one fused multiply-add (a single rounding of the exact x * inv - k) and is added as the
+// integer round(d * 2^22) + 2^31 in bits [47:0] of the slot, with 1 in bits [63:48]: count and sum
+// in one atomic, integer sums that do not depend on the order of the additions.  Per element the
+// table carries an error below 2^-23 of a bin width.  Elements with |x * inv| > 628 (or not a number)
+// are beyond the range of the 32-bit residual: they count with residual 0 and their x goes to a pair of
+// fp64 accumulators (they all have code 0 or 255).  A slot holds 2^16 - 1 additions; the workgroup
+// moves the slots into 64-bit accumulators before any slot can have seen that many.
+constexpr float kResidualOne = 4194304.0f;      // 2^22
+constexpr float kFarBins = 628.0f;              // |d| <= 628 + 128 * 2^-24... minus the clipped centre: below 512
+constexpr int kFarCopies = 16;
+
+template <int R>
+struct ResidualHist {
+    unsigned long long slot[kBins * R];
+    long long wide_sum[kBins];
+    unsigned long long wide_cnt[kBins];
+    double far_sum[2][kFarCopies];
+    unsigned far_cnt[2][kFarCopies];
+    // main rounds between two flushes: kThreads / R lanes share a slot and add 4 * kUnroll elements each per round
+    static constexpr int kPerRound = (kThreads / R) * 4 * kUnroll;
+    static constexpr int kFlushRounds = 65535 / kPerRound - 2;
+    static_assert(kFlushRounds >= 1, "too few copies of a bin for this workgroup size");
+};
+
+template <int R>
+__device__ __forceinline__ void rhist_zero(ResidualHist<R>& h) {
+    for (int i = threadIdx.x; i < kBins * R; i += kThreads) h.slot[i] = 0ull;
+    for (int i = threadIdx.x; i < kBins; i += kThreads) { h.wide_sum[i] = 0; h.wide_cnt[i] = 0ull; }
+    if (threadIdx.x < 2 * kFarCopies) {
+        h.far_sum[threadIdx.x / kFarCopies][threadIdx.x % kFarCopies] = 0.0;
+        h.far_cnt[threadIdx.x / kFarCopies][threadIdx.x % kFarCopies] = 0u;
+    }
+}
+
+// round(d * 2^22) of the residual of x in the bin of `code`; meaningless (and replaced) for far elements
+__device__ __forceinline__ int residual_fixed(float x, float inv, int code) {
+    const float d = __builtin_fmaf(x, inv, -static_cast<float>(code - kZeroPoint));
+    return static_cast<int>(__builtin_rintf(d * kResidualOne));
+}
+
+template <int R>
+__device__ __forceinline__ void rhist_add(ResidualHist<R>& h, int code, int fixed) {
+    const unsigned long long v = (1ull << 48) | static_cast<unsigned long long>(static_cast<unsigned>(fixed) ^ 0x80000000u);
+    __hip_atomic_fetch_add(&h.slot[code * R + (threadIdx.x & (R - 1))], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+__device__ __forceinline__ bool is_far(float x, float inv) { return !(__builtin_fabsf(x * inv) <= kFarBins); }
+
+template <int R>
+__device__ __forceinline__ void rhist_add_far(ResidualHist<R>& h, int code, float x) {
+    const int side = code == kBins - 1, c = threadIdx.x & (kFarCopies - 1);
+    __hip_atomic_fetch_add(&h.far_sum[side][c], static_cast<double>(x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __hip_atomic_fetch_add(&h.far_cnt[side][c], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// The four elements of one vector.  Every lane of the workgroup must be able to reach this (no barrier inside).
+template <int R>
+__device__ __forceinline__ void rhist_add4(ResidualHist<R>& h, const f4a v, float inv, int a, int b, int c, int d) {
+    int fa = residual_fixed(v.x, inv, a), fb = residual_fixed(v.y, inv, b), fc = residual_fixed(v.z, inv, c),
+        fd = residual_fixed(v.w, inv, d);
+    const bool ra = is_far(v.x, inv), rb = is_far(v.y, inv), rc = is_far(v.z, inv), rd = is_far(v.w, inv);
+    if (ra | rb | rc | rd) {
+        if (ra) { fa = 0; rhist_add_far(h, a, v.x); }
+        if (rb) { fb = 0; rhist_add_far(h, b, v.y); }
+        if (rc) { fc = 0; rhist_add_far(h, c, v.z); }
+        if (rd) { fd = 0; rhist_add_far(h, d, v.w); }
+    }
+    rhist_add(h, a, fa);
+    rhist_add(h, b, fb);
+    rhist_add(h, c, fc);
+    rhist_add(h, d, fd);
+}
+
+// Move the slots into the 64-bit accumulators.  Called by all lanes of the workgroup (two barriers).
+template <int R>
+__device__ __forceinline__ void rhist_flush(ResidualHist<R>& h) {
+    __syncthreads();
+    for (int b = threadIdx.x; b < kBins; b += kThreads) {
+        unsigned long long cnt = 0, sum = 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const unsigned long long v = h.slot[b * R + r];
+            h.slot[b * R + r] = 0ull;
+            cnt += v >> 48;
+            sum += v & 0xffffffffffffull;
+        }
+        h.wide_sum[b] += static_cast<long long>(sum) - static_cast<long long>(cnt << 31);
+        h.wide_cnt[b] += cnt;
+    }
+    __syncthreads();
+}
+
+// The workgroup's partial (after a last flush): bin sums of x in fp64 and counts, 4 KiB contiguous.
+template <int R>
+__device__ __forceinline__ void rhist_store(ResidualHist<R>& h, float inv, Workspace* ws) {
+    rhist_flush(h);
+    for (int b = threadIdx.x; b < kBins; b += kThreads) {
+        const unsigned long long cnt = h.wide_cnt[b];
+        unsigned long long far_n = 0;
+        double far_s = 0.0;
+        if (b == 0 || b == kBins - 1) {
+            const int side = b != 0;
+#pragma unroll
+            for (int c = 0; c < kFarCopies; ++c) { far_n += h.far_cnt[side][c]; far_s += h.far_sum[side][c]; }
+        }
+        const double centre = static_cast<double>(static_cast<long long>(cnt - far_n) * (b - kZeroPoint));
+        const double bins = centre + static_cast<double>(h.wide_sum[b]) * (1.0 / kResidualOne);
+        BinAcc acc;
+        acc.sum = bins / static_cast<double>(inv) + far_s;
+        acc.cnt = cnt;
+        ws->hist[blockIdx.x][b] = acc;
+    }
 }
 
 // Register-side accumulators for a tensor whose values crowd into a few codes (a constant, or

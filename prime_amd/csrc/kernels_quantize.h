@@ -5,32 +5,40 @@
 // Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
 
 // K2 (+K3 when HIST): quantize to uint8, 4 codes packed per 32-bit store, and the 256-bin
-// sum / count histogram of the same elements.  5 bytes per element.
-template <bool ALIGNED, bool NT, bool HIST, int R>
+// sum / count histogram of the same elements.  5 bytes per element.  REVERSE walks the tensor from
+// its end (for the pass that follows a pass over the same tensor); POLICY is the cache policy of
+// the code stores.  The histogram is the fixed-point one (one LDS atomic per element) whenever
+// 1 / scale is a finite non-zero number; otherwise (scale 0, infinite or not a number: an all-zero
+// tensor, a single element) the fp64 one.
+template <bool ALIGNED, bool NT, bool HIST, int R, bool REVERSE, int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
                                                             int stats_parts, prime_qparams* qp_out, int zero_point,
                                                             uint8_t* __restrict__ codes, Workspace* ws) {
     using M = Mem<ALIGNED, NT>;
-    __shared__ LdsHist<HIST ? R : 1> hist;
-    if (HIST) hist_zero(hist);
+    union Hist {
+        ResidualHist<HIST ? R : 1> fixed;
+        LdsHist<HIST ? R : 1> fp;
+    };
+    __shared__ Hist hist;
     // the scale: given by value, or derived here from the statistics partials of the pass before
     // (stats_parts < 0: the record a preceding kernel left in the workspace)
-    int hot_base = INT_MIN;              // set when the statistics show a tensor crowded into a few codes
-    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &hot_base)
+    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out)
                       : stats_parts < 0 ? ws->qp.inv_scale
                                         : 1.0f / scale_val;
-    if (HIST) __syncthreads();
+    const bool fixed = HIST && inv != 0.0f && __builtin_fabsf(inv) < __builtin_inff();      // false for NaN
+    if (HIST) {
+        if (fixed) rhist_zero(hist.fixed);
+        else hist_zero(hist.fp);
+        __syncthreads();
+    }
     const int64_t nvec = n >> 2;
-    auto pass = [&](auto narrow_t) {
-        constexpr bool narrow = decltype(narrow_t)::value;
-        HotCodes hot;
-        hot.base = hot_base;
-        auto add = [&](int code, float xv) {
-            if (narrow) hist_add_hot(hist, hot, code, xv);
-            else hist_add(hist, code, xv);
-        };
-        sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    auto pass = [&](auto fixed_t) {
+        constexpr bool kFixed = decltype(fixed_t)::value;
+        int since_flush = 0;
+        sweep_tiles<kUnroll, REVERSE>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
             constexpr bool full = decltype(full_t)::value;
+            const int64_t i0 = base + threadIdx.x;
+            const Window out(codes + base * 4, (nvec - base) * 4);
             f4a v[kUnroll];
 #pragma unroll
             for (int j = 0; j < kUnroll; ++j) {
@@ -45,15 +53,25 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
                     const int b = quantize_code(v[j].y, inv, zero_point);
                     const int c = quantize_code(v[j].z, inv, zero_point);
                     const int d = quantize_code(v[j].w, inv, zero_point);
-                    M::stu32(codes, i, static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) |
-                                           (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24));
+                    const uint32_t word = static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) |
+                                          (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24);
+                    if (ALIGNED) out.template st32<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 4u, word);
+                    else M::stu32(codes, i, word);
                     if (HIST) {
-                        add(a, v[j].x);
-                        add(b, v[j].y);
-                        add(c, v[j].z);
-                        add(d, v[j].w);
+                        if (kFixed) {
+                            rhist_add4(hist.fixed, v[j], inv, a, b, c, d);
+                        } else {
+                            hist_add(hist.fp, a, v[j].x);
+                            hist_add(hist.fp, b, v[j].y);
+                            hist_add(hist.fp, c, v[j].z);
+                            hist_add(hist.fp, d, v[j].w);
+                        }
                     }
                 }
+            }
+            if (HIST && kFixed && full && ++since_flush == ResidualHist<HIST ? R : 1>::kFlushRounds) {
+                rhist_flush(hist.fixed);       // every lane of the workgroup runs the same rounds
+                since_flush = 0;
             }
         });
         if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
@@ -61,15 +79,26 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
             const float v = x[i];
             const int a = quantize_code(v, inv, zero_point);
             codes[i] = static_cast<uint8_t>(a);
-            if (HIST) add(a, v);
+            if (HIST) {
+                if (kFixed) {
+                    const bool far = is_far(v, inv);
+                    if (far) rhist_add_far(hist.fixed, a, v);
+                    rhist_add(hist.fixed, a, far ? 0 : residual_fixed(v, inv, a));
+                } else {
+                    hist_add(hist.fp, a, v);
+                }
+            }
         }
-        if (HIST && narrow) hist_flush_hot(hist, hot);
     };
-    if (HIST && hot_base != INT_MIN) pass(std::true_type{});
+    if (HIST && fixed) pass(std::true_type{});
     else pass(std::false_type{});
     if (HIST) {
-        __syncthreads();
-        hist_store(hist, ws);
+        if (fixed) {
+            rhist_store(hist.fixed, inv, ws);
+        } else {
+            __syncthreads();
+            hist_store(hist.fp, ws);
+        }
     }
 }
 

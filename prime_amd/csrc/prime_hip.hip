@@ -53,6 +53,8 @@ struct Options {
     int nt_load_min_mib = 512;      // tensors of at least this many MiB are loaded with the non-temporal hint
     int nt_second_min_mib = 0;      // the same for the quantize pass that re-reads a tensor: its last use, always hinted
     int hist_replicas = 8;          // 1, 2, 4, 8 or 16 copies of each LDS bin
+    int code_store_policy = kStoreWriteThrough;   // cache policy of the code stores (0 plain, 2 nt, 16 write-through)
+    int reverse_second_pass = 1;    // the pass that re-reads a tensor walks it from its end
 };
 Options g_opt;
 
@@ -159,36 +161,48 @@ int run_stats(const float* x, int64_t n, prime_qparams* out, Workspace* ws, hipS
     return run_stats_finalize(ws, parts, n, out, st);
 }
 
-template <bool HIST, int R>
-void launch_quantize_r(bool al, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
+template <bool HIST, int R, bool REVERSE, int POLICY>
+void launch_quantize_p(bool al, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
                        prime_qparams* qp_out, int zp, uint8_t* codes, Workspace* ws) {
     const int id = HIST ? kIdQuantizeHist : kIdQuantize;
     if (!al)
-        launch(id, 5.0 * n, quantize_kernel<false, false, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
-    else if (stats_parts > 0 ? (n >> 18) >= g_opt.nt_second_min_mib : use_nt(n))
-        launch(id, 5.0 * n, quantize_kernel<true, true, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+        launch(id, 5.0 * n, quantize_kernel<false, false, HIST, R, REVERSE, kStorePlain>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    else if (stats_parts != 0 ? (n >> 18) >= g_opt.nt_second_min_mib : use_nt(n))
+        launch(id, 5.0 * n, quantize_kernel<true, true, HIST, R, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     else
-        launch(id, 5.0 * n, quantize_kernel<true, false, HIST, R>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+        launch(id, 5.0 * n, quantize_kernel<true, false, HIST, R, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+}
+
+template <bool HIST, int R>
+void launch_quantize_r(bool al, bool reverse, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
+                       prime_qparams* qp_out, int zp, uint8_t* codes, Workspace* ws) {
+#define PRIME_Q(REV, POL) launch_quantize_p<HIST, R, REV, POL>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws)
+    const int pol = g_opt.code_store_policy;
+    if (reverse) {
+        if (pol == kStoreNt) PRIME_Q(true, kStoreNt);
+        else if (pol == kStorePlain) PRIME_Q(true, kStorePlain);
+        else PRIME_Q(true, kStoreWriteThrough);
+    } else {
+        if (pol == kStoreNt) PRIME_Q(false, kStoreNt);
+        else if (pol == kStorePlain) PRIME_Q(false, kStorePlain);
+        else PRIME_Q(false, kStoreWriteThrough);
+    }
+#undef PRIME_Q
 }
 
 // stats_parts > 0: take the scale from that many statistics partials in the workspace (and
 // publish it to qp_out); otherwise use `scale`.  Returns the grid size through *grid_out: the
-// number of histogram partials written.
+// number of histogram partials written.  second_pass: the tensor has just been streamed by the
+// kernel before this one, so walk it from its end (what the last-level cache still holds comes first).
 int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_qparams* qp_out, int zp, uint8_t* codes,
-                 Workspace* ws, bool hist, hipStream_t st, int* grid_out) {
+                 Workspace* ws, bool hist, hipStream_t st, int* grid_out, bool second_pass = false) {
     const int grid = grid_for(n);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
-    if (!hist) {
-        launch_quantize_r<false, 1>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
-    } else {
-        switch (g_opt.hist_replicas) {
-            case 1: launch_quantize_r<true, 1>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
-            case 2: launch_quantize_r<true, 2>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
-            default: launch_quantize_r<true, 8>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
-            case 16: launch_quantize_r<true, 16>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
-            case 4: launch_quantize_r<true, 4>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws); break;
-        }
-    }
+    const bool rev = second_pass && g_opt.reverse_second_pass;
+    if (!hist) launch_quantize_r<false, 1>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    else if (g_opt.hist_replicas <= 4) launch_quantize_r<true, 4>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    else if (g_opt.hist_replicas == 8) launch_quantize_r<true, 8>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    else launch_quantize_r<true, 16>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     if (grid_out) *grid_out = grid;
     return launch_check("quantize_kernel");
 }
@@ -295,6 +309,12 @@ int prime_hip_set_option(const char* name, int value) {
         if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
             return fail(PRIME_EINVAL, "hist_replicas must be 1, 2, 4, 8 or 16");
         g_opt.hist_replicas = value;
+    } else if (!strcmp(name, "code_store_policy")) {
+        if (value != kStorePlain && value != kStoreNt && value != kStoreWriteThrough)
+            return fail(PRIME_EINVAL, "code_store_policy must be 0 (plain), 2 (non-temporal) or 16 (write-through)");
+        g_opt.code_store_policy = value;
+    } else if (!strcmp(name, "reverse_second_pass")) {
+        g_opt.reverse_second_pass = value != 0;
     } else if (!strcmp(name, "nt_load_min_mib")) {
         if (value < 0) return fail(PRIME_EINVAL, "nt_load_min_mib must be >= 0");
         g_opt.nt_load_min_mib = value;
@@ -311,6 +331,8 @@ int prime_hip_get_option(const char* name, int* value) {
     if (!name || !value) return fail(PRIME_EINVAL, "null argument");
     if (!strcmp(name, "blocks_per_cu")) *value = g_opt.blocks_per_cu;
     else if (!strcmp(name, "hist_replicas")) *value = g_opt.hist_replicas;
+    else if (!strcmp(name, "code_store_policy")) *value = g_opt.code_store_policy;
+    else if (!strcmp(name, "reverse_second_pass")) *value = g_opt.reverse_second_pass;
     else if (!strcmp(name, "nt_load_min_mib")) *value = g_opt.nt_load_min_mib;
     else if (!strcmp(name, "nt_second_min_mib")) *value = g_opt.nt_second_min_mib;
     else if (!strcmp(name, "unroll")) *value = kUnroll;
@@ -428,7 +450,7 @@ int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float
     }
     int parts = 0, grid = 0;
     if (int rc = run_stats_partials(x, n, w, st, &parts)) return rc;
-    if (int rc = run_quantize(x, n, 0.0f, parts, qparams_out, kZeroPoint, codes, w, true, st, &grid)) return rc;
+    if (int rc = run_quantize(x, n, 0.0f, parts, qparams_out, kZeroPoint, codes, w, true, st, &grid, true)) return rc;
     return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
 }
 
@@ -542,7 +564,7 @@ int ring_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_
     } else {
         if (int rc = run_dequant<ADD, true>(chunk, lut_in, codes_in, n, w, st, &grid)) return rc;
     }
-    if (int rc = run_quantize(chunk, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid)) return rc;
+    if (int rc = run_quantize(chunk, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid, true)) return rc;
     return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
 }
 
@@ -626,7 +648,7 @@ int prime_ring_first_touch(const float* outer, const float* inner, int64_t n, fl
                    nullptr, nullptr, 1.0f, grad_out, w);
     }
     if (int rc = launch_check("first_touch_kernel")) return rc;
-    if (int rc = run_quantize(grad_out, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid)) return rc;
+    if (int rc = run_quantize(grad_out, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid, true)) return rc;
     return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
 }
 

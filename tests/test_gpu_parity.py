@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from prime_amd import _lib
-from tests.conftest import lut_rel_err
+from tests.conftest import lut_rel_err, tables_agree
 from tests.golden.make_fixtures import CASES, case_input
 from tests.gpu_util import Abi, announce
 
@@ -161,7 +161,7 @@ def test_cfg5_two_thousand_small_tensors_batched(abi, oracle):
         announce(f"cfg5 single tensor {t} n={sizes[t]}")
         c1, l1, _ = abi.uniform(ft[off[t]:off[t + 1]])
         assert np.array_equal(c1.cpu().numpy(), gc[off[t]:off[t + 1]])
-        assert np.allclose(l1.cpu().numpy(), gl[t], rtol=1e-6, atol=0)
+        assert tables_agree(l1.cpu().numpy(), gl[t], abi.qparams(gq[t])["scale"], 2 * LUT_TOL)
 
 
 def test_cfg5_edge_tensors(abi, oracle):
@@ -710,8 +710,9 @@ def test_requantize_codes_equals_quantizing_the_dequantized_chunk(abi, oracle, n
     _check_requantized(abi, oracle, codes_in, lut_in, codes, lut, qp)
     assert torch.equal(codes, codes2)
     assert abi.qparams(qp)["scale"] == abi.qparams(qp2)["scale"] or n == 1
-    a, b = lut.cpu().numpy(), lut2.cpu().numpy()
-    assert np.allclose(a, b, rtol=2e-6, atol=0, equal_nan=True)
+    # both tables are within the bar of the fp64 bin means, so within twice the bar of each other
+    # (one bin width as the floor: an entry near zero has no meaningful relative error)
+    assert tables_agree(lut.cpu().numpy(), lut2.cpu().numpy(), abi.qparams(qp)["scale"], 2 * LUT_TOL)
 
 
 def test_requantize_codes_misaligned_special_values_and_foreign_tables(abi, oracle):

@@ -7,6 +7,7 @@ import pytest
 import torch
 import torch.distributed as dist
 
+from tests.conftest import tables_agree
 from tests.gpu_util import announce
 
 pytestmark = pytest.mark.gpu
@@ -235,8 +236,11 @@ def test_reference_import_paths_reach_the_hip_kernels(dev):
         assert codes.dtype == torch.uint8 and codes.shape == a.shape and lut.shape == (256,)
         diff = (lut[codes.long()] - a).abs()
         assert float(diff.max()) <= 6 * float(a.norm() / math.sqrt(N - 1)) / 256 * 1.01 or float(diff.median()) < 0.2
+        # the table of the fused pass (fixed-point residual sums) and that of average_buckets (fp64 sums)
+        # are both within 1e-6 of the exact bin means
         new_lut = average_buckets(a, codes, 256)
-        assert torch.equal(new_lut, lut)
+        scale = 6 * float(a.norm() / math.sqrt(N - 1)) / 256
+        assert tables_agree(new_lut.cpu().numpy(), lut.cpu().numpy(), scale, 2e-6)
         q = quantize_per_tensor_uint8(torch.ones(N, device=dev) * 10, 0.01, 128)
         assert bool((q == 255).all())
     finally:
