@@ -42,7 +42,7 @@ int prime_hip_abi_version(void);
 const char* prime_hip_last_error(void);
 
 /* Tuning knobs: "blocks_per_cu" (resident workgroups per compute unit), "hist_replicas" (copies
- * of each LDS histogram bin: 1, 2, 4, 8, 16), "nt_load_min_mib" (tensors at least this large
+ * of each LDS histogram bin in the fused quantize pass: 1, 2, 4, 8), "nt_load_min_mib" (tensors at least this large
  * are read with non-temporal loads in their first pass), "nt_second_min_mib" (the same for the
  * quantize pass that reads a tensor for the last time).  Returns 0 if the name is known.  The
  * options are process-wide and read at launch time: set them before work is enqueued, not

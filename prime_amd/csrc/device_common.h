@@ -317,25 +317,27 @@ __device__ __forceinline__ void hist_add(LdsHist<R>& h, int code, float x) {
 // fp64 accumulators (they all have code 0 or 255).  A slot holds 2^16 - 1 additions; the workgroup
 // moves the slots into 64-bit accumulators before any slot can have seen that many.
 constexpr float kResidualOne = 4194304.0f;      // 2^22
-constexpr float kFarBins = 628.0f;              // |d| <= 628 + 128 * 2^-24... minus the clipped centre: below 512
+constexpr float kFarBins = 628.0f;              // the residual of a nearer element is below 512 bins
 constexpr int kFarCopies = 16;
+constexpr int kMaxCopies = 8;                   // LDS copies of a bin, chosen per launch: 1, 2, 4 or 8
 
-template <int R>
+// `shift` = log2 of the number of copies of each bin in use: lanes pick a copy by lane id, so that
+// lanes of a wavefront that meet in one bin spread over several addresses.  Few copies are fastest on
+// data that spreads over many bins; a tensor crowded into a few bins (a constant, weights near 1)
+// wants all eight.
 struct ResidualHist {
-    unsigned long long slot[kBins * R];
+    unsigned long long slot[kBins * kMaxCopies];
     long long wide_sum[kBins];
     unsigned long long wide_cnt[kBins];
     double far_sum[2][kFarCopies];
     unsigned far_cnt[2][kFarCopies];
-    // main rounds between two flushes: kThreads / R lanes share a slot and add 4 * kUnroll elements each per round
-    static constexpr int kPerRound = (kThreads / R) * 4 * kUnroll;
-    static constexpr int kFlushRounds = 65535 / kPerRound - 2;
-    static_assert(kFlushRounds >= 1, "too few copies of a bin for this workgroup size");
+    // main rounds between two flushes: kThreads >> shift lanes share a slot and add 4 * kUnroll elements each per round
+    static __device__ __forceinline__ int flush_rounds(int shift) { return 65535 / ((kThreads >> shift) * 4 * kUnroll) - 2; }
 };
+static_assert(65535 / (kThreads * 4 * kUnroll) - 2 >= 1, "a slot must hold more than three rounds of a whole workgroup");
 
-template <int R>
-__device__ __forceinline__ void rhist_zero(ResidualHist<R>& h) {
-    for (int i = threadIdx.x; i < kBins * R; i += kThreads) h.slot[i] = 0ull;
+__device__ __forceinline__ void rhist_zero(ResidualHist& h, int shift) {
+    for (int i = threadIdx.x; i < (kBins << shift); i += kThreads) h.slot[i] = 0ull;
     for (int i = threadIdx.x; i < kBins; i += kThreads) { h.wide_sum[i] = 0; h.wide_cnt[i] = 0ull; }
     if (threadIdx.x < 2 * kFarCopies) {
         h.far_sum[threadIdx.x / kFarCopies][threadIdx.x % kFarCopies] = 0.0;
@@ -349,24 +351,22 @@ __device__ __forceinline__ int residual_fixed(float x, float inv, int code) {
     return static_cast<int>(__builtin_rintf(d * kResidualOne));
 }
 
-template <int R>
-__device__ __forceinline__ void rhist_add(ResidualHist<R>& h, int code, int fixed) {
+// `copy` = the lane's copy index, threadIdx.x & ((1 << shift) - 1)
+__device__ __forceinline__ void rhist_add(ResidualHist& h, int shift, int copy, int code, int fixed) {
     const unsigned long long v = (1ull << 48) | static_cast<unsigned long long>(static_cast<unsigned>(fixed) ^ 0x80000000u);
-    __hip_atomic_fetch_add(&h.slot[code * R + (threadIdx.x & (R - 1))], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __hip_atomic_fetch_add(&h.slot[(code << shift) + copy], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
 __device__ __forceinline__ bool is_far(float x, float inv) { return !(__builtin_fabsf(x * inv) <= kFarBins); }
 
-template <int R>
-__device__ __forceinline__ void rhist_add_far(ResidualHist<R>& h, int code, float x) {
+__device__ __forceinline__ void rhist_add_far(ResidualHist& h, int code, float x) {
     const int side = code == kBins - 1, c = threadIdx.x & (kFarCopies - 1);
     __hip_atomic_fetch_add(&h.far_sum[side][c], static_cast<double>(x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     __hip_atomic_fetch_add(&h.far_cnt[side][c], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-// The four elements of one vector.  Every lane of the workgroup must be able to reach this (no barrier inside).
-template <int R>
-__device__ __forceinline__ void rhist_add4(ResidualHist<R>& h, const f4a v, float inv, int a, int b, int c, int d) {
+// The four elements of one vector (no barrier inside: lanes may skip it).
+__device__ __forceinline__ void rhist_add4(ResidualHist& h, int shift, int copy, const f4a v, float inv, int a, int b, int c, int d) {
     int fa = residual_fixed(v.x, inv, a), fb = residual_fixed(v.y, inv, b), fc = residual_fixed(v.z, inv, c),
         fd = residual_fixed(v.w, inv, d);
     const bool ra = is_far(v.x, inv), rb = is_far(v.y, inv), rc = is_far(v.z, inv), rd = is_far(v.w, inv);
@@ -376,22 +376,20 @@ __device__ __forceinline__ void rhist_add4(ResidualHist<R>& h, const f4a v, floa
         if (rc) { fc = 0; rhist_add_far(h, c, v.z); }
         if (rd) { fd = 0; rhist_add_far(h, d, v.w); }
     }
-    rhist_add(h, a, fa);
-    rhist_add(h, b, fb);
-    rhist_add(h, c, fc);
-    rhist_add(h, d, fd);
+    rhist_add(h, shift, copy, a, fa);
+    rhist_add(h, shift, copy, b, fb);
+    rhist_add(h, shift, copy, c, fc);
+    rhist_add(h, shift, copy, d, fd);
 }
 
 // Move the slots into the 64-bit accumulators.  Called by all lanes of the workgroup (two barriers).
-template <int R>
-__device__ __forceinline__ void rhist_flush(ResidualHist<R>& h) {
+__device__ __forceinline__ void rhist_flush(ResidualHist& h, int shift) {
     __syncthreads();
     for (int b = threadIdx.x; b < kBins; b += kThreads) {
         unsigned long long cnt = 0, sum = 0;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const unsigned long long v = h.slot[b * R + r];
-            h.slot[b * R + r] = 0ull;
+        for (int r = 0; r < (1 << shift); ++r) {
+            const unsigned long long v = h.slot[(b << shift) + r];
+            h.slot[(b << shift) + r] = 0ull;
             cnt += v >> 48;
             sum += v & 0xffffffffffffull;
         }
@@ -402,9 +400,8 @@ __device__ __forceinline__ void rhist_flush(ResidualHist<R>& h) {
 }
 
 // The workgroup's partial (after a last flush): bin sums of x in fp64 and counts, 4 KiB contiguous.
-template <int R>
-__device__ __forceinline__ void rhist_store(ResidualHist<R>& h, float inv, Workspace* ws) {
-    rhist_flush(h);
+__device__ __forceinline__ void rhist_store(ResidualHist& h, int shift, float inv, Workspace* ws) {
+    rhist_flush(h, shift);
     for (int b = threadIdx.x; b < kBins; b += kThreads) {
         const unsigned long long cnt = h.wide_cnt[b];
         unsigned long long far_n = 0;

@@ -222,7 +222,8 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_remap_kernel(con
 // values are taken in the same pass (the next quantization's scale).  With DIV the updated value
 // is divided by `divisor` before it is stored and counted: chunk.div_(world_size) of
 // ReduceOp::AVG (collectives.cpp:155-159) folded into the last accumulation of a chunk.
-template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV = false>
+// POLICY is the cache policy of the fp32 stores.
+template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut,
                                                            const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
                                                            float divisor) {
@@ -233,8 +234,10 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float*
     const int64_t nvec = n >> 2;
     constexpr int U = DIV ? kDivUnroll : kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep_tiles<U>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
+        const int64_t i0 = base + threadIdx.x;
+        const Window win(out + base * 4, (nvec - base) * 16);
         uint32_t c[U];
         f4a a[U];
 #pragma unroll
@@ -255,7 +258,8 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float*
             if (ADD) v += a[j];
             if (DIV) v = v / divisor;
             if (full || i < nvec) {
-                M::stf4(out, i, v, !STATS);   // with STATS the quantize pass reads it again: no streaming hint
+                if (ALIGNED) win.template st128<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 16u, v);
+                else M::stf4(out, i, v, false);
                 if (STATS) {
                     if (j & 1) stats_add4(v, s1, q1); else stats_add4(v, s0, q0);
                 }

@@ -10,13 +10,15 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
 }
 
 // chunk /= world_size for ReduceOp::AVG (collectives.cpp:155-159): an fp32 division in place.
-template <bool ALIGNED>
+template <bool ALIGNED, int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void div_kernel(float* __restrict__ x, int64_t n, float d) {
     using M = Mem<ALIGNED, false>;
     const int64_t nvec = n >> 2;
     constexpr int U = kDivUnroll;
-    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep_tiles<U>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
+        const int64_t i0 = base + threadIdx.x;
+        const Window win(x + base * 4, (nvec - base) * 16);
         f4a v[U];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
@@ -26,7 +28,10 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void div_kernel(float* __r
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
-            if (full || i < nvec) M::stf4(x, i, v[j] / d, false);
+            if (full || i < nvec) {
+                if (ALIGNED) win.template st128<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 16u, v[j] / d);
+                else M::stf4(x, i, v[j] / d, false);
+            }
         }
     });
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
@@ -39,15 +44,17 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void div_kernel(float* __r
 // (src/zeroband/diloco.py:93-101): grad = outer_param - inner_param, then the whole flat buffer
 // divided by the world size; an fp32 subtraction and an fp32 division per element.
 // 12 bytes per element.
-template <bool ALIGNED>
+template <bool ALIGNED, bool NT, int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer,
                                                                                    const float* __restrict__ inner, int64_t n,
                                                                                    float world_size, float* __restrict__ out) {
-    using M = Mem<ALIGNED, false>;
+    using M = Mem<ALIGNED, NT>;
     const int64_t nvec = n >> 2;
     constexpr int U = kDivUnroll;
-    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep_tiles<U>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
+        const int64_t i0 = base + threadIdx.x;
+        const Window win(out + base * 4, (nvec - base) * 16);
         f4a a[U], b[U];
 #pragma unroll
         for (int j = 0; j < U; ++j) {
@@ -59,7 +66,11 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void pseudo_gradient_kerne
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
-            if (full || i < nvec) M::stf4(out, i, (a[j] - b[j]) / world_size, false);
+            if (full || i < nvec) {
+                const f4a g = (a[j] - b[j]) / world_size;
+                if (ALIGNED) win.template st128<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 16u, g);
+                else M::stf4(out, i, g, false);
+            }
         }
     });
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
@@ -75,13 +86,13 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void pseudo_gradient_kerne
 // acc = grad + lut[codes] (collectives.cpp:128-133), and with a divisor other than 1 the sum is
 // divided (ReduceOp::AVG, :155-159).  The fp64 sum and sum of squares of what is stored are the
 // statistics of the quantization that follows.  12 bytes per element, 13 with codes.
-template <bool CODES, bool ALIGNED>
+template <bool CODES, bool ALIGNED, bool NT, int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(const float* __restrict__ outer,
                                                                                const float* __restrict__ inner, int64_t n,
                                                                                float world_size, const uint8_t* __restrict__ codes,
                                                                                const float* __restrict__ lut, float divisor,
                                                                                float* __restrict__ out, Workspace* ws) {
-    using M = Mem<ALIGNED, false>;
+    using M = Mem<ALIGNED, NT>;
     __shared__ float s_lut[kBins];
     if (CODES) {
         for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
@@ -91,8 +102,10 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
     const int64_t nvec = n >> 2;
     constexpr int U = kDivUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    sweep<U>(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep_tiles<U>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
+        const int64_t i0 = base + threadIdx.x;
+        const Window win(out + base * 4, (nvec - base) * 16);
         f4a a[U], b[U];
         uint32_t c[U];
 #pragma unroll
@@ -117,7 +130,8 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
                 if (div) v = v / divisor;
             }
             if (full || i < nvec) {
-                M::stf4(out, i, v, false);       // the quantize pass reads it again: no streaming hint
+                if (ALIGNED) win.template st128<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 16u, v);
+                else M::stf4(out, i, v, false);
                 if (j & 1) stats_add4(v, s1, q1); else stats_add4(v, s0, q0);
             }
         }
@@ -153,22 +167,25 @@ __device__ __forceinline__ void outer_sgd_one(float& p, float& buf, float g, flo
 // the inner model (sync_inner_model, :137-144) in the same pass.  The gradient is fp32
 // (24 bytes per element) or, with CODES, uint8 codes and their lookup table (21 bytes per
 // element, and the dequantize pass is saved).
-template <bool CODES, bool ALIGNED>
+template <bool CODES, bool ALIGNED, bool NT, int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom,
                                                                               const float* __restrict__ grad,
                                                                               const uint8_t* __restrict__ codes,
                                                                               const float* __restrict__ lut,
                                                                               float* __restrict__ inner, int64_t n, float neg_lr,
                                                                               float mu, int first) {
-    using M = Mem<ALIGNED, false>;
+    using M = Mem<ALIGNED, NT>;
     __shared__ float s_lut[kBins];
     if (CODES) {
         for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
         __syncthreads();
     }
     const int64_t nvec = n >> 2;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep_tiles(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
+        const int64_t i0 = base + threadIdx.x;
+        const Window wp(param + base * 4, (nvec - base) * 16), wm(mom + base * 4, (nvec - base) * 16),
+            wi(inner ? inner + base * 4 : nullptr, inner ? (nvec - base) * 16 : 0);
         f4a p[kUnroll], m[kUnroll], g[kUnroll];
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
@@ -194,9 +211,16 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void outer_step_kernel(flo
                     p[j][c] = pc;
                     m[j][c] = mc;
                 }
-                M::stf4(param, i, p[j], false);
-                M::stf4(mom, i, m[j], false);
-                if (inner) M::stf4(inner, i, p[j], true);
+                if (ALIGNED) {
+                    const uint32_t off = static_cast<uint32_t>(threadIdx.x + j * stride) * 16u;
+                    wp.template st128<POLICY>(off, p[j]);
+                    wm.template st128<POLICY>(off, m[j]);
+                    wi.template st128<POLICY>(off, p[j]);      // an empty window without an inner model: dropped
+                } else {
+                    M::stf4(param, i, p[j], false);
+                    M::stf4(mom, i, m[j], false);
+                    if (inner) M::stf4(inner, i, p[j], true);
+                }
             }
         }
     });
@@ -212,10 +236,13 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void outer_step_kernel(flo
     }
 }
 
+template <int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
-    using M = Mem<true, false>;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    using M = Mem<true, true>;
+    sweep_tiles(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
+        const int64_t i0 = base + threadIdx.x;
+        const Window win(dst + base, (nvec - base) * 16);
         f4a v[kUnroll];
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
@@ -225,7 +252,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void copy_kernel(f4a* __re
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
             const int64_t i = i0 + j * stride;
-            if (full || i < nvec) M::stf4(reinterpret_cast<float*>(dst), i, v[j], true);
+            if (full || i < nvec) win.template st128<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 16u, v[j]);
         }
     });
 }

@@ -4,37 +4,67 @@
 //
 // Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
 
+// One (sum, count) pair for bin 0 as the workgroup's whole histogram partial: every lane brings the
+// fp64 sum and the number of the elements it saw.
+__device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, Workspace* ws) {
+    __shared__ double sh_s[kWaves];
+    __shared__ unsigned long long sh_c[kWaves];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    s = wave_sum(s);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_down(c, off, 64);
+    if (lane == 0) { sh_s[wave] = s; sh_c[wave] = c; }
+    __syncthreads();
+    for (int b = threadIdx.x; b < kBins; b += kThreads) {
+        BinAcc acc{0.0, 0ull};
+        if (b == 0)
+            for (int w = 0; w < kWaves; ++w) { acc.sum += sh_s[w]; acc.cnt += sh_c[w]; }
+        ws->hist[blockIdx.x][b] = acc;
+    }
+}
+
 // K2 (+K3 when HIST): quantize to uint8, 4 codes packed per 32-bit store, and the 256-bin
 // sum / count histogram of the same elements.  5 bytes per element.  REVERSE walks the tensor from
 // its end (for the pass that follows a pass over the same tensor); POLICY is the cache policy of
-// the code stores.  The histogram is the fixed-point one (one LDS atomic per element) whenever
-// 1 / scale is a finite non-zero number; otherwise (scale 0, infinite or not a number: an all-zero
-// tensor, a single element) the fp64 one.
-template <bool ALIGNED, bool NT, bool HIST, int R, bool REVERSE, int POLICY>
+// the code stores.  The histogram is the fixed-point one (one LDS atomic per element, 2^copies_shift
+// copies of each bin, eight when the statistics show a tensor crowded into a few bins) whenever
+// 1 / scale is a finite non-zero number.  When 1 / scale is infinite or not a number (scale 0: an
+// all-zero tensor) every element has code 0 and the histogram is one sum; a zero 1 / scale (an
+// infinite scale: a single element) takes the fp64 histogram.
+template <bool ALIGNED, bool NT, bool HIST, bool REVERSE, int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
                                                             int stats_parts, prime_qparams* qp_out, int zero_point,
-                                                            uint8_t* __restrict__ codes, Workspace* ws) {
+                                                            uint8_t* __restrict__ codes, Workspace* ws, int copies_shift) {
     using M = Mem<ALIGNED, NT>;
+    constexpr int kFpCopies = 8;
     union Hist {
-        ResidualHist<HIST ? R : 1> fixed;
-        LdsHist<HIST ? R : 1> fp;
+        ResidualHist fixed;
+        LdsHist<kFpCopies> fp;
     };
-    __shared__ Hist hist;
+    __shared__ std::conditional_t<HIST, Hist, int> hist_mem;      // no histogram memory without HIST
+    Hist& hist = reinterpret_cast<Hist&>(hist_mem);
     // the scale: given by value, or derived here from the statistics partials of the pass before
     // (stats_parts < 0: the record a preceding kernel left in the workspace)
-    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out)
+    int narrow = INT_MIN;                // set when the statistics show a tensor crowded into a few codes
+    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &narrow)
                       : stats_parts < 0 ? ws->qp.inv_scale
                                         : 1.0f / scale_val;
-    const bool fixed = HIST && inv != 0.0f && __builtin_fabsf(inv) < __builtin_inff();      // false for NaN
+    enum { kPlain, kFixed, kFp, kBin0 };
+    const int mode = !HIST ? kPlain : !(__builtin_fabsf(inv) < __builtin_inff()) ? kBin0 : inv != 0.0f ? kFixed : kFp;
+    const int shift = narrow != INT_MIN ? 3 : copies_shift;        // 8 = kMaxCopies
+    const int copy = threadIdx.x & ((1 << shift) - 1);
     if (HIST) {
-        if (fixed) rhist_zero(hist.fixed);
-        else hist_zero(hist.fp);
+        if (mode == kFixed) rhist_zero(hist.fixed, shift);
+        else if (mode == kFp) hist_zero(hist.fp);
         __syncthreads();
     }
     const int64_t nvec = n >> 2;
-    auto pass = [&](auto fixed_t) {
-        constexpr bool kFixed = decltype(fixed_t)::value;
+    double lane_sum = 0.0;               // kBin0
+    unsigned long long lane_cnt = 0;
+    auto pass = [&](auto mode_t) {
+        constexpr int kMode = decltype(mode_t)::value;
         int since_flush = 0;
+        const int flush_rounds = kMode == kFixed ? ResidualHist::flush_rounds(shift) : 0;
         sweep_tiles<kUnroll, REVERSE>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
             constexpr bool full = decltype(full_t)::value;
             const int64_t i0 = base + threadIdx.x;
@@ -57,20 +87,24 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
                                           (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24);
                     if (ALIGNED) out.template st32<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 4u, word);
                     else M::stu32(codes, i, word);
-                    if (HIST) {
-                        if (kFixed) {
-                            rhist_add4(hist.fixed, v[j], inv, a, b, c, d);
-                        } else {
-                            hist_add(hist.fp, a, v[j].x);
-                            hist_add(hist.fp, b, v[j].y);
-                            hist_add(hist.fp, c, v[j].z);
-                            hist_add(hist.fp, d, v[j].w);
-                        }
+                    if (kMode == kFixed) {
+                        rhist_add4(hist.fixed, shift, copy, v[j], inv, a, b, c, d);
+                    } else if (kMode == kFp) {
+                        hist_add(hist.fp, a, v[j].x);
+                        hist_add(hist.fp, b, v[j].y);
+                        hist_add(hist.fp, c, v[j].z);
+                        hist_add(hist.fp, d, v[j].w);
+                    } else if (kMode == kBin0) {
+                        lane_sum += static_cast<double>(v[j].x);
+                        lane_sum += static_cast<double>(v[j].y);
+                        lane_sum += static_cast<double>(v[j].z);
+                        lane_sum += static_cast<double>(v[j].w);
+                        lane_cnt += 4;
                     }
                 }
             }
-            if (HIST && kFixed && full && ++since_flush == ResidualHist<HIST ? R : 1>::kFlushRounds) {
-                rhist_flush(hist.fixed);       // every lane of the workgroup runs the same rounds
+            if (kMode == kFixed && full && ++since_flush == flush_rounds) {
+                rhist_flush(hist.fixed, shift);       // every lane of the workgroup runs the same rounds
                 since_flush = 0;
             }
         });
@@ -79,25 +113,30 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
             const float v = x[i];
             const int a = quantize_code(v, inv, zero_point);
             codes[i] = static_cast<uint8_t>(a);
-            if (HIST) {
-                if (kFixed) {
-                    const bool far = is_far(v, inv);
-                    if (far) rhist_add_far(hist.fixed, a, v);
-                    rhist_add(hist.fixed, a, far ? 0 : residual_fixed(v, inv, a));
-                } else {
-                    hist_add(hist.fp, a, v);
-                }
+            if (kMode == kFixed) {
+                const bool far = is_far(v, inv);
+                if (far) rhist_add_far(hist.fixed, a, v);
+                rhist_add(hist.fixed, shift, copy, a, far ? 0 : residual_fixed(v, inv, a));
+            } else if (kMode == kFp) {
+                hist_add(hist.fp, a, v);
+            } else if (kMode == kBin0) {
+                lane_sum += static_cast<double>(v);
+                lane_cnt += 1;
             }
         }
     };
-    if (HIST && fixed) pass(std::true_type{});
-    else pass(std::false_type{});
+    if (mode == kFixed) pass(std::integral_constant<int, kFixed>{});
+    else if (mode == kFp) pass(std::integral_constant<int, kFp>{});
+    else if (mode == kBin0) pass(std::integral_constant<int, kBin0>{});
+    else pass(std::integral_constant<int, kPlain>{});
     if (HIST) {
-        if (fixed) {
-            rhist_store(hist.fixed, inv, ws);
-        } else {
+        if (mode == kFixed) {
+            rhist_store(hist.fixed, shift, inv, ws);
+        } else if (mode == kFp) {
             __syncthreads();
             hist_store(hist.fp, ws);
+        } else {
+            hist_store_bin0(lane_sum, lane_cnt, ws);
         }
     }
 }

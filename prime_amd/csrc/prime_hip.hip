@@ -52,9 +52,12 @@ struct Options {
     int blocks_per_cu = PRIME_BLOCKS_PER_CU;
     int nt_load_min_mib = 512;      // tensors of at least this many MiB are loaded with the non-temporal hint
     int nt_second_min_mib = 0;      // the same for the quantize pass that re-reads a tensor: its last use, always hinted
-    int hist_replicas = 8;          // 1, 2, 4, 8 or 16 copies of each LDS bin
+    int hist_replicas = 4;          // 1, 2, 4 or 8 copies of each LDS bin of the fused quantize pass
     int code_store_policy = kStoreWriteThrough;   // cache policy of the code stores (0 plain, 2 nt, 16 write-through)
     int reverse_second_pass = 1;    // the pass that re-reads a tensor walks it from its end
+    int f32_store_policy = kStoreWriteThrough;          // fp32 outputs nobody reads back soon (dequantize, outer step)
+    int f32_reread_store_policy = kStoreWriteThrough;   // fp32 outputs the next kernel reads back (ring step, first touch)
+    int copy_store_policy = kStoreNt;                   // the plain copy (the byte counters' yardstick)
 };
 Options g_opt;
 
@@ -137,6 +140,14 @@ void launch(int id, double algo_bytes, void (*kernel)(KArgs...), int grid, int t
     g_prof.launches.push_back(t);
 }
 
+// Calls f with the store policy as a compile-time constant.
+template <typename F>
+void with_policy(int policy, F&& f) {
+    if (policy == kStoreNt) f(std::integral_constant<int, kStoreNt>{});
+    else if (policy == kStoreWriteThrough) f(std::integral_constant<int, kStoreWriteThrough>{});
+    else f(std::integral_constant<int, kStorePlain>{});
+}
+
 int run_stats_finalize(Workspace* ws, int nparts, int64_t n, prime_qparams* out, hipStream_t st) {
     launch(kIdStatsFinalize, 16.0 * nparts, stats_finalize_kernel, 1, kFinalThreads, st, ws, nparts, n, out);
     return launch_check("stats_finalize_kernel");
@@ -161,22 +172,24 @@ int run_stats(const float* x, int64_t n, prime_qparams* out, Workspace* ws, hipS
     return run_stats_finalize(ws, parts, n, out, st);
 }
 
-template <bool HIST, int R, bool REVERSE, int POLICY>
+template <bool HIST, bool REVERSE, int POLICY>
 void launch_quantize_p(bool al, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
                        prime_qparams* qp_out, int zp, uint8_t* codes, Workspace* ws) {
     const int id = HIST ? kIdQuantizeHist : kIdQuantize;
+    int shift = 0;
+    while ((1 << (shift + 1)) <= g_opt.hist_replicas) ++shift;
     if (!al)
-        launch(id, 5.0 * n, quantize_kernel<false, false, HIST, R, REVERSE, kStorePlain>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+        launch(id, 5.0 * n, quantize_kernel<false, false, HIST, REVERSE, kStorePlain>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
     else if (stats_parts != 0 ? (n >> 18) >= g_opt.nt_second_min_mib : use_nt(n))
-        launch(id, 5.0 * n, quantize_kernel<true, true, HIST, R, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+        launch(id, 5.0 * n, quantize_kernel<true, true, HIST, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
     else
-        launch(id, 5.0 * n, quantize_kernel<true, false, HIST, R, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+        launch(id, 5.0 * n, quantize_kernel<true, false, HIST, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
 }
 
-template <bool HIST, int R>
+template <bool HIST>
 void launch_quantize_r(bool al, bool reverse, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
                        prime_qparams* qp_out, int zp, uint8_t* codes, Workspace* ws) {
-#define PRIME_Q(REV, POL) launch_quantize_p<HIST, R, REV, POL>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws)
+#define PRIME_Q(REV, POL) launch_quantize_p<HIST, REV, POL>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws)
     const int pol = g_opt.code_store_policy;
     if (reverse) {
         if (pol == kStoreNt) PRIME_Q(true, kStoreNt);
@@ -199,10 +212,8 @@ int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_
     const int grid = grid_for(n);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
     const bool rev = second_pass && g_opt.reverse_second_pass;
-    if (!hist) launch_quantize_r<false, 1>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
-    else if (g_opt.hist_replicas <= 4) launch_quantize_r<true, 4>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
-    else if (g_opt.hist_replicas == 8) launch_quantize_r<true, 8>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
-    else launch_quantize_r<true, 16>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    if (!hist) launch_quantize_r<false>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    else launch_quantize_r<true>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     if (grid_out) *grid_out = grid;
     return launch_check("quantize_kernel");
 }
@@ -217,18 +228,29 @@ int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins
     return launch_check("lut_finalize_kernel");
 }
 
+template <bool ADD, bool STATS, bool DIV, int POLICY>
+void launch_dequant(int id, double bytes, int grid, hipStream_t st, float* out, const float* lut, const uint8_t* codes, int64_t n,
+                    Workspace* ws, float divisor) {
+    if (!(aligned_to(out, 16) && aligned_to(codes, 4)))
+        launch(id, bytes, dequant_kernel<ADD, STATS, false, false, DIV, kStorePlain>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
+    else if (use_nt(n))
+        launch(id, bytes, dequant_kernel<ADD, STATS, true, true, DIV, POLICY>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
+    else
+        launch(id, bytes, dequant_kernel<ADD, STATS, true, false, DIV, POLICY>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
+}
+
+// The fp32 stores of a pass whose output the next kernel reads back at once (STATS: the quantize
+// pass follows) take f32_reread_store_policy, the others f32_store_policy.
 template <bool ADD, bool STATS, bool DIV = false>
 int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out,
                 float divisor = 1.0f) {
     const int grid = grid_for(n);
     const int id = STATS ? (ADD ? kIdDequantAddStats : kIdDequantSetStats) : (ADD ? kIdDequantAdd : kIdDequantSet);
     const double bytes = (ADD ? 9.0 : 5.0) * n;
-    if (!(aligned_to(out, 16) && aligned_to(codes, 4)))
-        launch(id, bytes, dequant_kernel<ADD, STATS, false, false, DIV>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
-    else if (use_nt(n))
-        launch(id, bytes, dequant_kernel<ADD, STATS, true, true, DIV>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
-    else
-        launch(id, bytes, dequant_kernel<ADD, STATS, true, false, DIV>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
+    const int pol = STATS ? g_opt.f32_reread_store_policy : g_opt.f32_store_policy;
+    if (pol == kStoreNt) launch_dequant<ADD, STATS, DIV, kStoreNt>(id, bytes, grid, st, out, lut, codes, n, ws, divisor);
+    else if (pol == kStoreWriteThrough) launch_dequant<ADD, STATS, DIV, kStoreWriteThrough>(id, bytes, grid, st, out, lut, codes, n, ws, divisor);
+    else launch_dequant<ADD, STATS, DIV, kStorePlain>(id, bytes, grid, st, out, lut, codes, n, ws, divisor);
     if (grid_out) *grid_out = grid;
     return launch_check("dequant_kernel");
 }
@@ -306,13 +328,17 @@ int prime_hip_set_option(const char* name, int value) {
         if (value < 1 || value > 16) return fail(PRIME_EINVAL, "blocks_per_cu must be 1..16");
         g_opt.blocks_per_cu = value;
     } else if (!strcmp(name, "hist_replicas")) {
-        if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
-            return fail(PRIME_EINVAL, "hist_replicas must be 1, 2, 4, 8 or 16");
+        if (value != 1 && value != 2 && value != 4 && value != 8)
+            return fail(PRIME_EINVAL, "hist_replicas must be 1, 2, 4 or 8");
         g_opt.hist_replicas = value;
     } else if (!strcmp(name, "code_store_policy")) {
         if (value != kStorePlain && value != kStoreNt && value != kStoreWriteThrough)
             return fail(PRIME_EINVAL, "code_store_policy must be 0 (plain), 2 (non-temporal) or 16 (write-through)");
         g_opt.code_store_policy = value;
+    } else if (!strcmp(name, "f32_store_policy") || !strcmp(name, "f32_reread_store_policy") || !strcmp(name, "copy_store_policy")) {
+        if (value != kStorePlain && value != kStoreNt && value != kStoreWriteThrough)
+            return fail(PRIME_EINVAL, "a store policy must be 0 (plain), 2 (non-temporal) or 16 (write-through)");
+        (name[0] == 'c' ? g_opt.copy_store_policy : name[4] == 's' ? g_opt.f32_store_policy : g_opt.f32_reread_store_policy) = value;
     } else if (!strcmp(name, "reverse_second_pass")) {
         g_opt.reverse_second_pass = value != 0;
     } else if (!strcmp(name, "nt_load_min_mib")) {
@@ -333,6 +359,9 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "hist_replicas")) *value = g_opt.hist_replicas;
     else if (!strcmp(name, "code_store_policy")) *value = g_opt.code_store_policy;
     else if (!strcmp(name, "reverse_second_pass")) *value = g_opt.reverse_second_pass;
+    else if (!strcmp(name, "f32_store_policy")) *value = g_opt.f32_store_policy;
+    else if (!strcmp(name, "f32_reread_store_policy")) *value = g_opt.f32_reread_store_policy;
+    else if (!strcmp(name, "copy_store_policy")) *value = g_opt.copy_store_policy;
     else if (!strcmp(name, "nt_load_min_mib")) *value = g_opt.nt_load_min_mib;
     else if (!strcmp(name, "nt_second_min_mib")) *value = g_opt.nt_second_min_mib;
     else if (!strcmp(name, "unroll")) *value = kUnroll;
@@ -596,9 +625,11 @@ int prime_div_f32(float* x, int64_t n, float divisor, prime_stream_t stream) {
     if (n == 0) return 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (aligned_to(x, 16))
-        launch(kIdDiv, 8.0 * n, div_kernel<true>, grid_for(n), kThreads, st, x, n, divisor);
+        with_policy(g_opt.f32_store_policy, [&](auto P) {
+            launch(kIdDiv, 8.0 * n, div_kernel<true, decltype(P)::value>, grid_for(n), kThreads, st, x, n, divisor);
+        });
     else
-        launch(kIdDiv, 8.0 * n, div_kernel<false>, grid_for(n), kThreads, st, x, n, divisor);
+        launch(kIdDiv, 8.0 * n, div_kernel<false, kStorePlain>, grid_for(n), kThreads, st, x, n, divisor);
     return launch_check("div_kernel");
 }
 
@@ -609,9 +640,14 @@ int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n,
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int grid = grid_for(n);
     if (aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(out, 16))
-        launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<true>, grid, kThreads, st, outer, inner, n, world_size, out);
+        with_policy(g_opt.f32_store_policy, [&](auto P) {
+            if (use_nt(n))
+                launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<true, true, decltype(P)::value>, grid, kThreads, st, outer, inner, n, world_size, out);
+            else
+                launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<true, false, decltype(P)::value>, grid, kThreads, st, outer, inner, n, world_size, out);
+        });
     else
-        launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<false>, grid, kThreads, st, outer, inner, n, world_size, out);
+        launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<false, false, kStorePlain>, grid, kThreads, st, outer, inner, n, world_size, out);
     return launch_check("pseudo_gradient_kernel");
 }
 
@@ -632,20 +668,34 @@ int prime_ring_first_touch(const float* outer, const float* inner, int64_t n, fl
     }
     int grid = grid_for(n);
     const bool al = aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(grad_out, 16) && (!codes_in || aligned_to(codes_in, 4));
+    const uint8_t* no_codes = nullptr;
+    const float* no_lut = nullptr;
     if (codes_in) {
         if (al)
-            launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, true>, grid, kThreads, st, outer, inner, n, world_size,
-                   codes_in, lut_in, divisor, grad_out, w);
+            with_policy(g_opt.f32_reread_store_policy, [&](auto P) {
+                if (use_nt(n))
+                    launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, true, true, decltype(P)::value>, grid, kThreads, st, outer,
+                           inner, n, world_size, codes_in, lut_in, divisor, grad_out, w);
+                else
+                    launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, true, false, decltype(P)::value>, grid, kThreads, st, outer,
+                           inner, n, world_size, codes_in, lut_in, divisor, grad_out, w);
+            });
         else
-            launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, false>, grid, kThreads, st, outer, inner, n, world_size,
+            launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, false, false, kStorePlain>, grid, kThreads, st, outer, inner, n, world_size,
                    codes_in, lut_in, divisor, grad_out, w);
     } else {
         if (al)
-            launch(kIdFirstTouch, 12.0 * n, first_touch_kernel<false, true>, grid, kThreads, st, outer, inner, n, world_size,
-                   nullptr, nullptr, 1.0f, grad_out, w);
+            with_policy(g_opt.f32_reread_store_policy, [&](auto P) {
+                if (use_nt(n))
+                    launch(kIdFirstTouch, 12.0 * n, first_touch_kernel<false, true, true, decltype(P)::value>, grid, kThreads, st, outer, inner,
+                           n, world_size, no_codes, no_lut, 1.0f, grad_out, w);
+                else
+                    launch(kIdFirstTouch, 12.0 * n, first_touch_kernel<false, true, false, decltype(P)::value>, grid, kThreads, st, outer, inner,
+                           n, world_size, no_codes, no_lut, 1.0f, grad_out, w);
+            });
         else
-            launch(kIdFirstTouch, 12.0 * n, first_touch_kernel<false, false>, grid, kThreads, st, outer, inner, n, world_size,
-                   nullptr, nullptr, 1.0f, grad_out, w);
+            launch(kIdFirstTouch, 12.0 * n, first_touch_kernel<false, false, false, kStorePlain>, grid, kThreads, st, outer, inner, n, world_size,
+                   no_codes, no_lut, 1.0f, grad_out, w);
     }
     if (int rc = launch_check("first_touch_kernel")) return rc;
     if (int rc = run_quantize(grad_out, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid, true)) return rc;
@@ -661,12 +711,20 @@ int prime_outer_sgd_nesterov_f32(float* param, float* momentum_buf, const float*
     const int grid = grid_for(n);
     const bool al = aligned_to(param, 16) && aligned_to(momentum_buf, 16) && aligned_to(grad, 16) && aligned_to(inner_out, 16);
     const double bytes = (inner_out ? 24.0 : 20.0) * n;
+    const uint8_t* no_codes = nullptr;
+    const float* no_lut = nullptr;
     if (al)
-        launch(kIdOuterStep, bytes, outer_step_kernel<false, true>, grid, kThreads, st, param, momentum_buf, grad, nullptr, nullptr,
-               inner_out, n, -lr, momentum, first_step);
+        with_policy(g_opt.f32_store_policy, [&](auto P) {
+            if (use_nt(n))
+                launch(kIdOuterStep, bytes, outer_step_kernel<false, true, true, decltype(P)::value>, grid, kThreads, st, param, momentum_buf,
+                       grad, no_codes, no_lut, inner_out, n, -lr, momentum, first_step);
+            else
+                launch(kIdOuterStep, bytes, outer_step_kernel<false, true, false, decltype(P)::value>, grid, kThreads, st, param, momentum_buf,
+                       grad, no_codes, no_lut, inner_out, n, -lr, momentum, first_step);
+        });
     else
-        launch(kIdOuterStep, bytes, outer_step_kernel<false, false>, grid, kThreads, st, param, momentum_buf, grad, nullptr, nullptr,
-               inner_out, n, -lr, momentum, first_step);
+        launch(kIdOuterStep, bytes, outer_step_kernel<false, false, false, kStorePlain>, grid, kThreads, st, param, momentum_buf, grad, no_codes,
+               no_lut, inner_out, n, -lr, momentum, first_step);
     return launch_check("outer_step_kernel");
 }
 
@@ -679,12 +737,19 @@ int prime_outer_sgd_nesterov_u8(float* param, float* momentum_buf, const uint8_t
     const int grid = grid_for(n);
     const bool al = aligned_to(param, 16) && aligned_to(momentum_buf, 16) && aligned_to(codes, 4) && aligned_to(inner_out, 16);
     const double bytes = (inner_out ? 21.0 : 17.0) * n;
+    const float* no_grad = nullptr;
     if (al)
-        launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, true>, grid, kThreads, st, param, momentum_buf, nullptr, codes, lut,
-               inner_out, n, -lr, momentum, first_step);
+        with_policy(g_opt.f32_store_policy, [&](auto P) {
+            if (use_nt(n))
+                launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, true, true, decltype(P)::value>, grid, kThreads, st, param,
+                       momentum_buf, no_grad, codes, lut, inner_out, n, -lr, momentum, first_step);
+            else
+                launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, true, false, decltype(P)::value>, grid, kThreads, st, param,
+                       momentum_buf, no_grad, codes, lut, inner_out, n, -lr, momentum, first_step);
+        });
     else
-        launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, false>, grid, kThreads, st, param, momentum_buf, nullptr, codes, lut,
-               inner_out, n, -lr, momentum, first_step);
+        launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, false, false, kStorePlain>, grid, kThreads, st, param, momentum_buf, no_grad, codes,
+               lut, inner_out, n, -lr, momentum, first_step);
     return launch_check("outer_step_kernel");
 }
 
@@ -695,8 +760,10 @@ int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t
     if (n_bytes == 0) return 0;
     const int64_t nvec = n_bytes >> 4;
     const int grid = grid_for(nvec * 4);
-    launch(kIdCopy, 2.0 * n_bytes, copy_kernel, grid, kThreads, static_cast<hipStream_t>(stream), static_cast<f4a*>(dst),
-           static_cast<const f4a*>(src), nvec);
+    with_policy(g_opt.copy_store_policy, [&](auto P) {
+        launch(kIdCopy, 2.0 * n_bytes, copy_kernel<decltype(P)::value>, grid, kThreads, static_cast<hipStream_t>(stream),
+               static_cast<f4a*>(dst), static_cast<const f4a*>(src), nvec);
+    });
     return launch_check("copy_kernel");
 }
 

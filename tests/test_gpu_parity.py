@@ -429,8 +429,10 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
     assert moved <= 45 * abs(rel) + 1e-6          # a code moves when |x| / scale crosses a boundary: at most ~|code - 128| * |rel|
 
 
-@pytest.mark.parametrize("option,values", [("hist_replicas", (1, 2, 4, 8, 16)), ("blocks_per_cu", (1, 2, 3, 4)),
-                                           ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20))])
+@pytest.mark.parametrize("option,values", [("hist_replicas", (1, 2, 4, 8)), ("blocks_per_cu", (1, 2, 3, 4)),
+                                           ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20)),
+                                           ("code_store_policy", (0, 2, 16)), ("f32_reread_store_policy", (0, 2, 16)),
+                                           ("reverse_second_pass", (0, 1))])
 def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle, option, values):
     # the options change scheduling and cache hints only: codes, scale and lookup must not move,
     # on ordinary data, on a tensor crowded into a few codes, and through a ring step
