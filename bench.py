@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 pseudo-gradient compression path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--legs a,b,...]
 
 One "step" is one pass of the hot path over the workload of benchmark configuration 2: the 22
 per-layer pseudo-gradient buckets of a 1B Llama-style model (51,380,224 fp32 elements each,
@@ -14,17 +14,26 @@ The single JSON line printed at the end carries
                  written once) over the whole step, wall clock between two synchronisations, with
                  the buckets dealt over three HIP streams (--streams); one_stream is the same work
                  strictly bucket after bucket
-  roofline       the dominant kernel (quantize + histogram, 5 bytes per element) priced against
-                 the 8 TB/s HBM peak from per-launch HIP-event times taken in a second pass over
-                 the same workload
+  roofline       the dominant kernel (quantize + histogram, 5 bytes per element) on a 2^28-element
+                 tensor (1 GiB, four times the last-level cache, so what it reads comes from HBM),
+                 priced against the 8 TB/s HBM peak from per-launch HIP-event times inside
+                 uniform_8bit_quantize calls that rotate over three such tensors; the same kernel on
+                 the 205 MB buckets of the step (partly served by the last-level cache) is listed
+                 beside it, as run and with its input cold
+  tensor_2p28    every operation of the path on 2^28-element tensors, one row each: statistics,
+                 quantize (a2), average_buckets (a3), dequantize add / set (a4 / a5), the fused
+                 quantize + lookup, uniform_8bit_quantize and the ring reduce step
   ring_step      benchmark configuration 3: W = 8 chunks of 2^26 elements; quantize chunk 0, then 7 hops of
                  dequantize-add + requantize (14 bytes per element per hop)
-  tensor_2p28    uniform_8bit_quantize on one 2^28-element tensor, the size the target is quoted on
   other_configs  benchmark configurations 1, 4 and 5 (round trip on 2^24 elements; 42 buckets of a 10B model's
                  shard with outliers, quantize + dequantize; 2,000 small tensors in one launch and the
                  edge tensors), each as algorithmic GB/s
   cpu_baseline   the reference's own compression.cpp (compiled into oracle/_ref) on this box's
-                 host cores, on a bounded sample (one bucket, a few repetitions)
+                 host cores, on a bounded sample (one bucket, a few repetitions), with the same
+                 operations one by one
+
+--legs runs a subset (buckets, t28, ring, outer, diloco, configs, staging): what a profiler run
+of one workload uses, so that every kernel name in its trace belongs to one element count.
 """
 from __future__ import annotations
 
@@ -44,11 +53,12 @@ BUCKET_ELEMS = 4 * 2048 * 2048 + 3 * 2048 * 5632    # 51,380,224
 N_LAYERS = 22
 RING_W = 8
 RING_CHUNK = 1 << 26
-# HBM bytes one launch of the dominant kernel moves on a 51,380,224-element bucket, from rocprofv3
-# FETCH_SIZE / WRITE_SIZE scaled by the same counters' readings for the 1 GiB copy below
-# (profiles/cfg2_buckets_hbm_traffic.txt): 205.7 MB read + 53.5 MB written (codes + 2 MB of
-# per-workgroup histogram partials) against 256.9 MB algorithmic.
-TRAFFIC_BYTES_PER_LAUNCH = 259.18e6
+N28 = 1 << 28
+# HBM bytes one launch of the dominant kernel moves on a 2^28-element tensor, from rocprofv3
+# FETCH_SIZE / WRITE_SIZE scaled by the same counters' readings for the 1 GiB copy that this
+# program runs first (profiles/uniform_2p28_hbm_traffic.txt); None until that file is made.
+TRAFFIC_BYTES_PER_LAUNCH_2P28 = None
+TRAFFIC_BYTES_PER_LAUNCH_BUCKET = None
 
 
 def student_t3(n, device, seed, scale):
@@ -148,6 +158,19 @@ def cpu_baseline(sample_elems: int, ring_elems: int, reps: int) -> dict:
         "elements_per_s": round(sample_elems / t, 1),
         "ms_per_bucket": round(t * 1e3, 3),
         "breakdown_ms": {k: round(v, 3) for k, v in parts.items()},
+        # the same operations one by one, as GB/s of their algorithmic bytes (beside tensor_2p28.operations)
+        "operations": {
+            "stats (norm)": {"GBps": round(4.0 * sample_elems / parts["norm_ms"] / 1e6, 3), "threads": 1, "elements": sample_elems},
+            "quantize_per_tensor_uint8 (a2)": {"GBps": round(5.0 * sample_elems / parts["quantize_ms"] / 1e6, 3), "threads": threads,
+                                               "elements": sample_elems},
+            "average_buckets (a3)": {"GBps": round(5.0 * sample_elems / parts["average_buckets_ms"] / 1e6, 3), "threads": threads,
+                                     "elements": sample_elems},
+            "index_add (a4)": {"GBps": round(9.0 * ring_elems / t_add / 1e9, 3), "threads": 1, "elements": ring_elems,
+                               "note": "as shipped: the OpenMP pragma is inert without -fopenmp (src/zeroband/C/collectives.py:17)"},
+            "index_set (a5)": {"GBps": round(5.0 * ring_elems / t_set / 1e9, 3), "threads": 1, "elements": ring_elems},
+            "uniform_8bit_quantize (a1)": {"GBps": round(9.0 * sample_elems / t / 1e9, 3), "threads": threads, "elements": sample_elems},
+            "ring reduce step (a4 + a1)": {"GBps": round(14.0 * ring_elems / hop / 1e9, 3), "threads": threads, "elements": ring_elems},
+        },
         "ring_step": {
             "value": round(14.0 * ring_elems / hop / 1e9, 3),
             "unit": "GB/s",
@@ -162,6 +185,11 @@ def cpu_baseline(sample_elems: int, ring_elems: int, reps: int) -> dict:
     }
 
 
+def _per_launch(prof: dict, overhead_us: float) -> dict:
+    """{kernel: (avg launch us net of the bracket overhead, algorithmic bytes per launch)}"""
+    return {k: (max(v["total_ms"] / v["launches"] * 1e3 - overhead_us, 1e-3), v["algo_bytes"] / v["launches"]) for k, v in prof.items()}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -170,9 +198,12 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--streams", type=int, default=3,
                     help="HIP streams the buckets are spread over in the timed region (1 = strictly one after another)")
-    ap.add_argument("--legs", default="buckets,ring,t28,outer,diloco,configs,staging",
-                    help="comma list of buckets (always run: it carries value and roofline), ring, t28, outer, diloco, configs, "
-                         "staging")
+    ap.add_argument("--legs", default="buckets,t28,ring,outer,diloco,configs,staging",
+                    help="comma list of buckets (carries value), t28 (carries roofline and the per-operation rows), ring, "
+                         "outer, diloco, configs, staging")
+    ap.add_argument("--t28-ops", default="",
+                    help="comma list of substrings: the t28 leg runs only the operations whose name contains one of them "
+                         "(uniform_8bit_quantize always runs: it carries the roofline)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -185,6 +216,7 @@ def main() -> int:
     for opt in filter(None, os.environ.get("PRIME_HIP_OPTIONS", "").split(",")):   # tuning sweeps: name=value,...
         name, val = opt.split("=")
         _lib.set_option(name, int(val))
+    legs = set(args.legs.split(","))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     st = torch.cuda.current_stream(dev).cuda_stream
@@ -209,8 +241,9 @@ def main() -> int:
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
 
-    # A plain copy of known size (1 GiB read + 1 GiB written), untimed: the dispatch a profiler's
-    # FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled against.
+    # A plain copy of known size (1 GiB read + 1 GiB written), untimed, and the FIRST launch of
+    # copy_kernel in the process: the dispatch a profiler's FETCH_SIZE / WRITE_SIZE readings of the
+    # other kernels are scaled against (prime_amd.rocprof_summary takes the first one).
     yard_src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
     yard_dst = torch.empty_like(yard_src)
     _lib.check(lib.prime_copy_bytes(yard_dst.data_ptr(), yard_src.data_ptr(), yard_src.numel() * 4, st), "copy_bytes")
@@ -218,45 +251,9 @@ def main() -> int:
     del yard_src, yard_dst
     torch.cuda.empty_cache()
 
-    # ---- config 2: 22 layer buckets, quantize + lookup per bucket -------------------------------
-    buckets = [student_t3(BUCKET_ELEMS, dev, layer, 1e-4) for layer in range(N_LAYERS)]
-    codes = [torch.empty(BUCKET_ELEMS, dtype=torch.uint8, device=dev) for _ in range(N_LAYERS)]
-    luts = torch.empty((N_LAYERS, 256), dtype=torch.float32, device=dev)
-    qps = torch.empty((N_LAYERS, 4), dtype=torch.float64, device=dev)
-
-    def step_buckets():
-        for i in range(N_LAYERS):
-            uniform(buckets[i], codes[i], luts[i], qps[i])
-
-    # The measured path: the buckets dealt over --streams HIP streams (prime_amd.ops.BucketPlan ->
-    # prime_uniform_8bit_quantize_buckets), so one bucket's statistics pass overlaps its neighbours'
-    # quantize pass and the launch ramps; results are those of the one-by-one loop.
-    plan = ops.BucketPlan(buckets, codes, luts, qps, n_streams=args.streams)
-    sec_pipelined = timed(plan.run, args.steps, args.warmup)
-    elems = BUCKET_ELEMS * N_LAYERS
-    value = 9.0 * elems / sec_pipelined / 1e9
-    # The same buckets strictly one after another on one stream: the reference's order, and the
-    # gapless sequence the per-kernel figures below are calibrated against.
-    sec = timed(step_buckets, args.steps, args.warmup)
-    value_one_stream = 9.0 * elems / sec / 1e9
-
-    # Third pass over the same workload, one stream, with a start and a stop HIP event on every
-    # launch (on the launch stream): the roofline figures.  An event-bracketed launch cannot overlap its dispatch
-    # with the kernel before it, so each bracket reads a few microseconds long.  That overhead is
-    # measured here, not assumed: the one-stream region above runs the same launches back to back
-    # (a kernel trace shows no gaps between them), so (sum of bracketed durations per bucket -
-    # wall time per bucket) / launches per bucket is the overhead of one bracket.
-    _lib.profile_begin()
-    for _ in range(args.steps):
-        step_buckets()
-    prof = _lib.profile_end()
-    launches_per_bucket = sum(v["launches"] for v in prof.values()) / (args.steps * N_LAYERS)
-    bracketed_us_per_bucket = sum(v["total_ms"] for v in prof.values()) * 1e3 / (args.steps * N_LAYERS)
-    wall_us_per_bucket = sec * 1e6 / N_LAYERS
-    overhead_from_buckets_us = max(0.0, (bracketed_us_per_bucket - wall_us_per_bucket) / launches_per_bucket)
-    # The same difference on a kernel long enough (about 100 us) that the host can never fall behind, also
-    # under a profiler, where launching the 4 us second-stage kernels back to back leaves gaps: 20 copies
-    # of 256 MiB bracketed, against the same 20 back to back.
+    # An event-bracketed launch cannot overlap its dispatch with the kernel before it, so a bracket can
+    # read a few microseconds long.  Measured here, not assumed: twenty 256 MiB copies (long enough that
+    # the host never falls behind, also under a profiler) bracketed, against the same twenty back to back.
     cal_src = torch.empty(1 << 26, dtype=torch.float32, device=dev).normal_()
     cal_dst = torch.empty_like(cal_src)
 
@@ -268,77 +265,20 @@ def main() -> int:
     for _ in range(20):
         cal_copy()
     cal_prof = _lib.profile_end()["copy_kernel"]
-    overhead_from_copies_us = max(0.0, cal_prof["total_ms"] / cal_prof["launches"] * 1e3 - cal_wall * 1e6)
-    del cal_src, cal_dst
-    event_overhead_us = min(overhead_from_buckets_us, overhead_from_copies_us) if overhead_from_buckets_us > 0 \
-        else overhead_from_copies_us
-    dom = prof["quantize_kernel+hist"]
-    dom_event_us = dom["total_ms"] / dom["launches"] * 1e3
-    dom_us = dom_event_us - event_overhead_us
-    achieved = dom["algo_bytes"] / dom["launches"] / (dom_us * 1e-6) / 1e9
-    kernels = {k: {"avg_us": round(v["total_ms"] / v["launches"] * 1e3 - event_overhead_us, 2),
-                   "avg_us_event_bracket": round(v["total_ms"] / v["launches"] * 1e3, 2),
-                   "launches": v["launches"]} for k, v in prof.items()}
-    for k, v in prof.items():
-        kernels[k]["algo_GBps"] = round(v["algo_bytes"] / v["launches"] / (kernels[k]["avg_us"] * 1e-6) / 1e9, 1)
-    # The statistics pass leaves much of a 205 MB bucket in the 256 MB last-level cache, and the
-    # quantize pass that follows is partly served from there.  How much that is worth: the same kernel
-    # on the same buckets with 1 GiB of cached reads of other data between the two passes.
-    flush_src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
-    nt_keep = _lib.get_option("nt_load_min_mib")
-    flushed_us = []
-    for i in range(min(6, N_LAYERS)):
-        _lib.check(lib.prime_uniform_8bit_quantize(buckets[i].data_ptr(), BUCKET_ELEMS, codes[i].data_ptr(), luts[i].data_ptr(),
-                                                   qps[i].data_ptr(), ws.data_ptr(), st), "uniform")        # sets the scale
-        scale_i = float(ops.unpack_qparams(qps[i])["scale"])
-        _lib.set_option("nt_load_min_mib", 10 ** 6)           # plain loads: the flush must displace the bucket
-        _lib.check(lib.prime_stats_f32(flush_src.data_ptr(), flush_src.numel(), qps[i].data_ptr(), ws.data_ptr(), st), "flush")
-        _lib.set_option("nt_load_min_mib", 0)                 # the quantize pass loads non-temporally, as in the fused call
-        torch.cuda.synchronize()
-        _lib.profile_begin()
-        _lib.check(lib.prime_quantize_lookup_u8(buckets[i].data_ptr(), BUCKET_ELEMS, scale_i, codes[i].data_ptr(), luts[i].data_ptr(),
-                                                ws.data_ptr(), st), "quantize_lookup")
-        torch.cuda.synchronize()
-        fp = _lib.profile_end()
-        _lib.set_option("nt_load_min_mib", nt_keep)
-        if i:                                                 # the first is a warm-up
-            flushed_us.append(fp["quantize_kernel+hist"]["total_ms"] * 1e3 - event_overhead_us)
-    del flush_src
-    flushed = statistics.mean(flushed_us)
-    roofline = {
-        "bound": "hbm",
-        "kernel": "quantize_kernel<aligned, hist, R=8> (quantize + 256-bin sum/count histogram)",
-        "achieved": round(achieved, 1),
-        "peak": HBM_PEAK_GBS,
-        "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-        "algo_bytes_per_launch": 5 * BUCKET_ELEMS,
-        "avg_launch_us": round(dom_us, 2),
-        "avg_launch_us_event_bracket": round(dom_event_us, 2),
-        "event_overhead_us": round(event_overhead_us, 2),
-        "event_overhead_us_from_bucket_sequence": round(overhead_from_buckets_us, 2),
-        "event_overhead_us_from_long_copies": round(overhead_from_copies_us, 2),
-        "last_level_cache": {
-            "note": "achieved is algorithmic bytes over the launch time as the job runs: the statistics pass has just "
-                    "streamed the bucket through the 256 MB last-level cache, which serves part of this pass",
-            "avg_launch_us_after_1GiB_of_other_reads": round(flushed, 2),
-            "achieved_after_1GiB_of_other_reads": round(5 * BUCKET_ELEMS / (flushed * 1e-6) / 1e9, 1),
-            "frac_after_1GiB_of_other_reads": round(5 * BUCKET_ELEMS / (flushed * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-        },
-        "kernels": kernels,
-    }
-    del buckets, codes, plan
-    torch.cuda.empty_cache()
+    overhead_from_copies_us = cal_prof["total_ms"] / cal_prof["launches"] * 1e3 - cal_wall * 1e6      # not clamped: a negative
+    del cal_src, cal_dst                                                                             # reading must show
+    event_overhead_us = max(0.0, overhead_from_copies_us)
+    overhead_note = {"event_overhead_us_applied": round(event_overhead_us, 2),
+                     "event_overhead_us_from_long_copies": round(overhead_from_copies_us, 2)}
 
     out = {
         "metric": "quantize+lookup & ring-reduce-step GB/s on 1 GPU; % of HBM peak; vs CPU ops",
-        "value": round(value, 1),
+        "value": None,
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(sec_pipelined * 1e3, 4),
+        "ms_per_step": None,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -347,19 +287,176 @@ def main() -> int:
         "config": {
             "workload": "benchmark configuration 2: 22 per-layer pseudo-gradient buckets x 51,380,224 fp32 elements, "
                         "Student-t(3)*1e-4 (torch cuda generator, seed = layer), uniform_8bit_quantize bucket by bucket",
-            "elements_per_step": elems,
+            "elements_per_step": BUCKET_ELEMS * N_LAYERS,
             "streams": args.streams,
             "algorithmic_bytes_per_element": 9,
             "n_bins": 256,
         },
-        "elements_per_s": round(elems / sec_pipelined, 1),
-        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-        "one_stream": {"value": round(value_one_stream, 1), "unit": "GB/s", "ms_per_step": round(sec * 1e3, 4),
-                       "frac_of_hbm_peak": round(value_one_stream / HBM_PEAK_GBS, 4)},
-        "roofline": roofline,
     }
+    bucket_kernel = None
 
-    legs = set(args.legs.split(","))
+    if "buckets" in legs:
+        # ---- config 2: 22 layer buckets, quantize + lookup per bucket ---------------------------
+        buckets = [student_t3(BUCKET_ELEMS, dev, layer, 1e-4) for layer in range(N_LAYERS)]
+        codes = [torch.empty(BUCKET_ELEMS, dtype=torch.uint8, device=dev) for _ in range(N_LAYERS)]
+        luts = torch.empty((N_LAYERS, 256), dtype=torch.float32, device=dev)
+        qps = torch.empty((N_LAYERS, 4), dtype=torch.float64, device=dev)
+
+        def step_buckets():
+            for i in range(N_LAYERS):
+                uniform(buckets[i], codes[i], luts[i], qps[i])
+
+        # The measured path: the buckets dealt over --streams HIP streams (prime_amd.ops.BucketPlan ->
+        # prime_uniform_8bit_quantize_buckets), so one bucket's statistics pass overlaps its neighbours'
+        # quantize pass and the launch ramps; results are those of the one-by-one loop.
+        plan = ops.BucketPlan(buckets, codes, luts, qps, n_streams=args.streams)
+        sec_pipelined = timed(plan.run, args.steps, args.warmup)
+        elems = BUCKET_ELEMS * N_LAYERS
+        value = 9.0 * elems / sec_pipelined / 1e9
+        # The same buckets strictly one after another on one stream: the reference's order.
+        sec = timed(step_buckets, args.steps, args.warmup)
+        value_one_stream = 9.0 * elems / sec / 1e9
+        # Third pass, one stream, with a start and a stop HIP event on every launch.
+        _lib.profile_begin()
+        for _ in range(args.steps):
+            step_buckets()
+        prof = _lib.profile_end()
+        launches_per_bucket = sum(v["launches"] for v in prof.values()) / (args.steps * N_LAYERS)
+        bracketed_us_per_bucket = sum(v["total_ms"] for v in prof.values()) * 1e3 / (args.steps * N_LAYERS)
+        overhead_note["event_overhead_us_from_bucket_sequence"] = round(
+            (bracketed_us_per_bucket - sec * 1e6 / N_LAYERS) / launches_per_bucket, 2)
+        per = _per_launch(prof, event_overhead_us)
+        # The same kernel with its input cold: the scales are known now, so quantize + lookup runs over
+        # the 22 buckets in turn with nothing in between; each bucket was last touched 4.3 GB of traffic ago.
+        scales = [float(ops.unpack_qparams(qps[i])["scale"]) for i in range(N_LAYERS)]
+
+        def cold_pass():
+            for i in range(N_LAYERS):
+                _lib.check(lib.prime_quantize_lookup_u8(buckets[i].data_ptr(), BUCKET_ELEMS, scales[i], codes[i].data_ptr(),
+                                                        luts[i].data_ptr(), ws.data_ptr(), st), "quantize_lookup")
+
+        cold_pass()
+        torch.cuda.synchronize()
+        _lib.profile_begin()
+        for _ in range(max(2, args.steps // 3)):
+            cold_pass()
+        cold = _per_launch(_lib.profile_end(), event_overhead_us)["quantize_kernel+hist"][0]
+        dom_us, dom_bytes = per["quantize_kernel+hist"]
+        bucket_kernel = {
+            "workload": "one 51,380,224-element bucket (205 MB) of the step; the statistics pass has just streamed it, and "
+                        "the 256 MB last-level cache serves part of this pass",
+            "avg_launch_us": round(dom_us, 2), "achieved": round(dom_bytes / dom_us / 1e3, 1),
+            "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBS, 4),
+            "input_cold": {"what": "quantize + lookup with the scale given, over the 22 buckets in turn: every bucket comes from HBM",
+                           "avg_launch_us": round(cold, 2), "achieved": round(dom_bytes / cold / 1e3, 1),
+                           "frac": round(dom_bytes / cold / 1e3 / HBM_PEAK_GBS, 4)},
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH_BUCKET,
+            "kernels": {k: {"avg_us": round(us, 2), "algo_GBps": round(b / us / 1e3, 1), "launches": prof[k]["launches"]}
+                        for k, (us, b) in per.items()},
+        }
+        out.update({
+            "value": round(value, 1),
+            "ms_per_step": round(sec_pipelined * 1e3, 4),
+            "elements_per_s": round(elems / sec_pipelined, 1),
+            "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+            "one_stream": {"value": round(value_one_stream, 1), "unit": "GB/s", "ms_per_step": round(sec * 1e3, 4),
+                           "frac_of_hbm_peak": round(value_one_stream / HBM_PEAK_GBS, 4)},
+        })
+        del buckets, codes, plan
+        torch.cuda.empty_cache()
+
+    if "t28" in legs:
+        # ---- 2^28-element tensors: the size the target is quoted on; every operation of the path ----
+        n28 = N28
+        xs28 = []
+        for seed in range(3):          # three tensors in rotation: 3 GiB between two visits of the same data
+            g = torch.Generator(device=dev).manual_seed(seed)
+            xs28.append(torch.randn(n28, device=dev, generator=g) * 1e-3)
+        c28 = torch.empty(n28, dtype=torch.uint8, device=dev)
+        cin28 = torch.empty(n28, dtype=torch.uint8, device=dev)
+        l28 = torch.empty(256, dtype=torch.float32, device=dev)
+        lin28 = torch.empty(256, dtype=torch.float32, device=dev)
+        qp28 = torch.empty(4, dtype=torch.float64, device=dev)
+        o28 = torch.empty(n28, device=dev)
+        uniform(xs28[0], cin28, lin28, qp28)
+        torch.cuda.synchronize()
+        scale28 = float(ops.unpack_qparams(qp28)["scale"])
+        import ctypes
+
+        calls = {
+            "stats (norm)": (4, lambda r: lib.prime_stats_f32(xs28[r % 3].data_ptr(), n28, qp28.data_ptr(), ws.data_ptr(), st)),
+            "quantize_per_tensor_uint8 (a2)": (5, lambda r: lib.prime_quantize_u8(xs28[r % 3].data_ptr(), n28, ctypes.c_float(scale28), 128,
+                                                                               c28.data_ptr(), st)),
+            "average_buckets (a3)": (5, lambda r: lib.prime_average_buckets(xs28[r % 3].data_ptr(), cin28.data_ptr(), n28, 256, l28.data_ptr(),
+                                                                            None, ws.data_ptr(), st)),
+            "index_add (a4)": (9, lambda r: lib.prime_dequant_add(o28.data_ptr(), lin28.data_ptr(), cin28.data_ptr(), n28, st)),
+            "index_set (a5)": (5, lambda r: lib.prime_dequant_set(o28.data_ptr(), lin28.data_ptr(), cin28.data_ptr(), n28, st)),
+            "quantize + lookup, scale given (K2+K3)": (5, lambda r: lib.prime_quantize_lookup_u8(xs28[r % 3].data_ptr(), n28, ctypes.c_float(scale28),
+                                                                                                c28.data_ptr(), l28.data_ptr(), ws.data_ptr(), st)),
+            "uniform_8bit_quantize (a1)": (9, lambda r: lib.prime_uniform_8bit_quantize(xs28[r % 3].data_ptr(), n28, c28.data_ptr(), l28.data_ptr(),
+                                                                                        qp28.data_ptr(), ws.data_ptr(), st)),
+            "ring reduce step (a4 + a1)": (14, lambda r: lib.prime_ring_reduce_step(xs28[1 + r % 2].data_ptr(), cin28.data_ptr(), lin28.data_ptr(), n28,
+                                                                                   c28.data_ptr(), l28.data_ptr(), None, ws.data_ptr(), st)),
+        }
+        rows, uni_prof = {}, None
+        only = [w for w in args.t28_ops.split(",") if w]
+        for name, (bpe, fn) in calls.items():
+            if only and not name.startswith("uniform") and not any(w in name for w in only):
+                continue
+            for r in range(args.warmup):
+                _lib.check(fn(r), name)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for r in range(args.steps):
+                _lib.check(fn(r), name)
+            torch.cuda.synchronize()
+            wall = (time.perf_counter() - t0) / args.steps
+            _lib.profile_begin()
+            for r in range(args.steps):
+                _lib.check(fn(r), name)
+            prof28 = _lib.profile_end()
+            per28 = _per_launch(prof28, event_overhead_us)
+            kern_us = sum(us for us, _ in per28.values())
+            rows[name] = {"bytes_per_element": bpe, "us": round(kern_us, 2), "GBps": round(bpe * n28 / kern_us / 1e3, 1),
+                          "elements_per_s": round(n28 / (kern_us * 1e-6), 1), "frac_of_hbm_peak": round(bpe * n28 / kern_us / 1e3 / HBM_PEAK_GBS, 4),
+                          "us_wall_back_to_back": round(wall * 1e6, 2),
+                          "kernels": {k: {"avg_us": round(us, 2), "algo_GBps": round(b / us / 1e3, 1)} for k, (us, b) in per28.items()}}
+            if name.startswith("uniform"):
+                uni_prof = per28
+        dom_us, dom_bytes = uni_prof["quantize_kernel+hist"]
+        uni, ring28 = rows["uniform_8bit_quantize (a1)"], rows.get("ring reduce step (a4 + a1)", {})
+        out["tensor_2p28"] = {
+            "workload": "2^28-element fp32 tensors N(0,1e-3), three in rotation; per operation: sum of its kernels' launch times "
+                        "(HIP events per launch), and wall time of back-to-back calls",
+            "value": uni["GBps"], "unit": "GB/s", "ms": round(uni["us"] / 1e3, 4), "elements_per_s": uni["elements_per_s"],
+            "frac_of_hbm_peak": uni["frac_of_hbm_peak"],
+            "ring_reduce_step": {"value": ring28["GBps"], "unit": "GB/s", "ms": round(ring28["us"] / 1e3, 4),
+                                 "frac_of_hbm_peak": ring28["frac_of_hbm_peak"]} if ring28 else None,
+            "operations": rows,
+        }
+        out["roofline"] = {
+            "bound": "hbm",
+            "kernel": "quantize_kernel<aligned, nt loads, hist, write-through stores> (quantize + 256-bin sum/count histogram)",
+            "workload": "inside uniform_8bit_quantize on 2^28-element tensors (1 GiB each, three in rotation: nothing of the tensor "
+                        "is left in the 256 MB last-level cache when the call starts)",
+            "achieved": round(dom_bytes / dom_us / 1e3, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBS, 4),
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH_2P28,
+            "algo_bytes_per_launch": 5 * n28,
+            "avg_launch_us": round(dom_us, 2),
+            **overhead_note,
+            "on_the_buckets_of_the_step": bucket_kernel,
+        }
+        del xs28, c28, cin28, o28
+        torch.cuda.empty_cache()
+    elif bucket_kernel is not None:
+        out["roofline"] = {"bound": "hbm", "kernel": "quantize_kernel+hist", "workload": bucket_kernel["workload"],
+                           "achieved": bucket_kernel["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bucket_kernel["frac"],
+                           "traffic": TRAFFIC_BYTES_PER_LAUNCH_BUCKET, "algo_bytes_per_launch": 5 * BUCKET_ELEMS,
+                           "avg_launch_us": bucket_kernel["avg_launch_us"], **overhead_note, "on_the_buckets_of_the_step": bucket_kernel}
+
     if "ring" in legs:
         # ---- config 3: ring reduce-scatter hops for W = 8 ranks' chunks ---------------------------
         chunks = []
@@ -408,49 +505,6 @@ def main() -> int:
             "kernels": kernel_table(rprof, event_overhead_us),
         }
         del chunks, pristine, cbuf
-        torch.cuda.empty_cache()
-
-    if "t28" in legs:
-        # ---- one 2^28-element tensor ---------------------------------------------------------------
-        n28 = 1 << 28
-        g = torch.Generator(device=dev).manual_seed(0)
-        x28 = torch.randn(n28, device=dev, generator=g) * 1e-3
-        c28 = torch.empty(n28, dtype=torch.uint8, device=dev)
-        l28 = torch.empty(256, dtype=torch.float32, device=dev)
-        qp28 = torch.empty(4, dtype=torch.float64, device=dev)
-        s28 = timed(lambda: uniform(x28, c28, l28, qp28), args.steps, args.warmup)
-        gbs28 = 9.0 * n28 / s28 / 1e9
-        _lib.profile_begin()
-        for _ in range(args.steps):
-            uniform(x28, c28, l28, qp28)
-        tprof = _lib.profile_end()
-        # the ring's reduce step at the same size: acc += lut[codes]; (codes, lut) = uniform_8bit_quantize(acc)
-        acc28 = torch.randn(n28, device=dev, generator=g) * 1e-3
-        keep28 = acc28.clone()
-        co28 = torch.empty(n28, dtype=torch.uint8, device=dev)
-        lo28 = torch.empty(256, dtype=torch.float32, device=dev)
-        r28 = []
-        for it in range(args.warmup + args.steps):
-            acc28.copy_(keep28)                 # every step accumulates onto the rank's own data
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            ring_step(acc28, c28, l28, co28, lo28)
-            torch.cuda.synchronize()
-            if it >= args.warmup:
-                r28.append(time.perf_counter() - t0)
-        rs28 = statistics.mean(r28)
-        rg28 = 14.0 * n28 / rs28 / 1e9
-        out["tensor_2p28"] = {
-            "workload": "uniform_8bit_quantize on one 2^28-element fp32 tensor N(0,1e-3)",
-            "value": round(gbs28, 1), "unit": "GB/s", "ms": round(s28 * 1e3, 4),
-            "elements_per_s": round(n28 / s28, 1), "frac_of_hbm_peak": round(gbs28 / HBM_PEAK_GBS, 4),
-            "kernels": kernel_table(tprof, event_overhead_us),
-            "ring_reduce_step": {"workload": "one ring reduce step on a 2^28-element accumulator (14 bytes per element), "
-                                             "timed call by call with a host synchronisation either side",
-                                 "value": round(rg28, 1), "unit": "GB/s", "ms": round(rs28 * 1e3, 4),
-                                 "frac_of_hbm_peak": round(rg28 / HBM_PEAK_GBS, 4)},
-        }
-        del x28, c28, acc28, keep28, co28
         torch.cuda.empty_cache()
 
     if "outer" in legs:
@@ -738,7 +792,7 @@ def main() -> int:
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(BUCKET_ELEMS, RING_CHUNK, reps=5)
-        out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1) if out["cpu_baseline"]["value"] else None
+        out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1) if out["value"] and out["cpu_baseline"]["value"] else None
 
     print(json.dumps(out))
     return 0

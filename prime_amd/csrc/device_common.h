@@ -365,21 +365,49 @@ __device__ __forceinline__ void rhist_add_far(ResidualHist& h, int code, float x
     __hip_atomic_fetch_add(&h.far_cnt[side][c], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-// The four elements of one vector (no barrier inside: lanes may skip it).
-__device__ __forceinline__ void rhist_add4(ResidualHist& h, int shift, int copy, const f4a v, float inv, int a, int b, int c, int d) {
-    int fa = residual_fixed(v.x, inv, a), fb = residual_fixed(v.y, inv, b), fc = residual_fixed(v.z, inv, c),
-        fd = residual_fixed(v.w, inv, d);
-    const bool ra = is_far(v.x, inv), rb = is_far(v.y, inv), rc = is_far(v.z, inv), rd = is_far(v.w, inv);
-    if (ra | rb | rc | rd) {
-        if (ra) { fa = 0; rhist_add_far(h, a, v.x); }
-        if (rb) { fb = 0; rhist_add_far(h, b, v.y); }
-        if (rc) { fc = 0; rhist_add_far(h, c, v.z); }
-        if (rd) { fd = 0; rhist_add_far(h, d, v.w); }
+// round_half_away(clamp(q, -128, 127)) as a float, for |q| <= kFarBins: the centre of the bin of a
+// product q = x * inv when the zero point is 128, i.e. code - 128.  trunc(c + copysign(0.49999997, c))
+// equals roundf(c) for every float in that range (0.49999997 is the float below 1/2: adding 1/2 itself
+// would round 0.49999997 up to 1; checked exhaustively on the host, tests/test_host.py).
+__device__ __forceinline__ float round_centre(float q) {
+    const float c = __builtin_amdgcn_fmed3f(q, -128.0f, 127.0f);
+    return __builtin_truncf(c + __builtin_copysignf(0.49999997f, c));
+}
+
+// The four elements of one vector in the fused pass: their packed codes (returned) and their
+// histogram entries (no barrier inside: lanes may skip it).  Products within kFarBins take the short
+// instruction sequence; a vector with a product beyond it, or not a number, takes the general one.
+__device__ __forceinline__ uint32_t rhist_quantize4(ResidualHist& h, int shift, int copy, const f4a v, float inv) {
+    const float qa = v.x * inv, qb = v.y * inv, qc = v.z * inv, qd = v.w * inv;
+    const bool ra = !(__builtin_fabsf(qa) <= kFarBins), rb = !(__builtin_fabsf(qb) <= kFarBins),
+               rc = !(__builtin_fabsf(qc) <= kFarBins), rd = !(__builtin_fabsf(qd) <= kFarBins);
+    int a, b, c, d, fa, fb, fc, fd;
+    if (!(ra | rb | rc | rd)) {
+        const float ka = round_centre(qa), kb = round_centre(qb), kc = round_centre(qc), kd = round_centre(qd);
+        a = static_cast<int>(ka) + kZeroPoint;
+        b = static_cast<int>(kb) + kZeroPoint;
+        c = static_cast<int>(kc) + kZeroPoint;
+        d = static_cast<int>(kd) + kZeroPoint;
+        fa = static_cast<int>(__builtin_rintf(__builtin_fmaf(v.x, inv, -ka) * kResidualOne));
+        fb = static_cast<int>(__builtin_rintf(__builtin_fmaf(v.y, inv, -kb) * kResidualOne));
+        fc = static_cast<int>(__builtin_rintf(__builtin_fmaf(v.z, inv, -kc) * kResidualOne));
+        fd = static_cast<int>(__builtin_rintf(__builtin_fmaf(v.w, inv, -kd) * kResidualOne));
+    } else {
+        a = quantize_code(v.x, inv, kZeroPoint);
+        b = quantize_code(v.y, inv, kZeroPoint);
+        c = quantize_code(v.z, inv, kZeroPoint);
+        d = quantize_code(v.w, inv, kZeroPoint);
+        fa = fb = fc = fd = 0;
+        if (ra) rhist_add_far(h, a, v.x); else fa = residual_fixed(v.x, inv, a);
+        if (rb) rhist_add_far(h, b, v.y); else fb = residual_fixed(v.y, inv, b);
+        if (rc) rhist_add_far(h, c, v.z); else fc = residual_fixed(v.z, inv, c);
+        if (rd) rhist_add_far(h, d, v.w); else fd = residual_fixed(v.w, inv, d);
     }
     rhist_add(h, shift, copy, a, fa);
     rhist_add(h, shift, copy, b, fb);
     rhist_add(h, shift, copy, c, fc);
     rhist_add(h, shift, copy, d, fd);
+    return static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) | (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24);
 }
 
 // Move the slots into the 64-bit accumulators.  Called by all lanes of the workgroup (two barriers).

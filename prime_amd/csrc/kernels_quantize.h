@@ -79,17 +79,21 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
             for (int j = 0; j < kUnroll; ++j) {
                 const int64_t i = i0 + j * stride;
                 if (full || i < nvec) {
-                    const int a = quantize_code(v[j].x, inv, zero_point);
-                    const int b = quantize_code(v[j].y, inv, zero_point);
-                    const int c = quantize_code(v[j].z, inv, zero_point);
-                    const int d = quantize_code(v[j].w, inv, zero_point);
-                    const uint32_t word = static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) |
-                                          (static_cast<uint32_t>(c) << 16) | (static_cast<uint32_t>(d) << 24);
+                    uint32_t word;
+                    int a = 0, b = 0, c = 0, d = 0;
+                    if (kMode == kFixed) {          // the histogram always has zero point 128 (compression.cpp:107)
+                        word = rhist_quantize4(hist.fixed, shift, copy, v[j], inv);
+                    } else {
+                        a = quantize_code(v[j].x, inv, zero_point);
+                        b = quantize_code(v[j].y, inv, zero_point);
+                        c = quantize_code(v[j].z, inv, zero_point);
+                        d = quantize_code(v[j].w, inv, zero_point);
+                        word = static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) | (static_cast<uint32_t>(c) << 16) |
+                               (static_cast<uint32_t>(d) << 24);
+                    }
                     if (ALIGNED) out.template st32<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 4u, word);
                     else M::stu32(codes, i, word);
-                    if (kMode == kFixed) {
-                        rhist_add4(hist.fixed, shift, copy, v[j], inv, a, b, c, d);
-                    } else if (kMode == kFp) {
+                    if (kMode == kFp) {
                         hist_add(hist.fp, a, v[j].x);
                         hist_add(hist.fp, b, v[j].y);
                         hist_add(hist.fp, c, v[j].z);

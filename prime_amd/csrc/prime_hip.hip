@@ -209,6 +209,7 @@ void launch_quantize_r(bool al, bool reverse, int grid, hipStream_t st, const fl
 // kernel before this one, so walk it from its end (what the last-level cache still holds comes first).
 int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_qparams* qp_out, int zp, uint8_t* codes,
                  Workspace* ws, bool hist, hipStream_t st, int* grid_out, bool second_pass = false) {
+    if (hist && zp != kZeroPoint) return fail(PRIME_EINVAL, "the fused quantize + lookup pass has zero point 128");
     const int grid = grid_for(n);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
     const bool rev = second_pass && g_opt.reverse_second_pass;

@@ -880,3 +880,29 @@ def test_pipelined_buckets_equal_one_by_one(abi, oracle, n_streams):
     for i in range(len(xs)):
         c1, l1, q1 = abi.uniform(xs[i])
         assert torch.equal(codes[i], c1) and torch.equal(luts[i], l1)
+
+
+def test_fused_pass_codes_for_every_float_within_and_around_the_fixed_point_range(abi, oracle):
+    # scale 1 makes x * inv = x: every float bit pattern with |x| < 1024 (the fused pass's short
+    # rounding sequence serves |x| <= 628, the general one the rest), both signs, through
+    # prime_quantize_lookup_u8, against the oracle's quantize_per_tensor
+    import ctypes
+
+    top = int(np.float32(1024.0).view(np.uint32))
+    step = 1 << 27
+    for sign in (0, 1):
+        for lo in range(0, top, step):
+            hi = min(lo + step, top)
+            announce(f"bit patterns sign={sign} [{lo:#x}, {hi:#x})")
+            bits = torch.arange(lo, hi, dtype=torch.int64, device=abi.dev)
+            if sign:
+                bits += 1 << 31
+            x = (bits - ((bits >> 31) << 32)).to(torch.int32).view(torch.float32)      # the bit pattern as an fp32 tensor
+            del bits
+            codes, _ = abi.quantize_lookup(x, 1.0)
+            got = codes.cpu().numpy()
+            hx = (np.arange(lo, hi, dtype=np.uint32) | np.uint32(sign << 31)).view(np.float32)
+            assert np.array_equal(x.cpu().numpy().view(np.uint32), hx.view(np.uint32))
+            want = oracle.quantize_per_tensor_uint8(hx, 1.0, 128)
+            bad = np.flatnonzero(got != want)
+            assert bad.size == 0, (sign, hx[bad[:5]], got[bad[:5]], want[bad[:5]])

@@ -1,5 +1,6 @@
 """Host-side mirror of the reference interface: names, signatures, error behaviour (CPU only)."""
 import inspect
+from pathlib import Path
 
 import pytest
 import torch
@@ -149,3 +150,16 @@ def test_bench_refuses_more_than_one_gpu():
     root = Path(__file__).resolve().parents[1]
     res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert res.returncode == 2 and "one GPU" in res.stderr and res.stdout.strip() == ""
+
+
+def test_short_rounding_sequence_equals_roundf_on_every_float_in_its_range(tmp_path):
+    # the fused quantize pass rounds products within its fixed-point range with
+    # trunc(c + copysign(0.49999997, c)); every one of the 2.3e9 floats of that range, on the host
+    import subprocess
+
+    src = Path(__file__).resolve().parent / "native" / "round_centre_check.c"
+    exe = tmp_path / "round_centre_check"
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", str(src), "-o", str(exe), "-lm"], check=True)
+    res = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert res.returncode == 0, res.stdout
+    assert "checked 2285502466 mismatches 0" in res.stdout
