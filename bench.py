@@ -56,9 +56,11 @@ RING_CHUNK = 1 << 26
 N28 = 1 << 28
 # HBM bytes one launch of the dominant kernel moves on a 2^28-element tensor, from rocprofv3
 # FETCH_SIZE / WRITE_SIZE scaled by the same counters' readings for the 1 GiB copy that this
-# program runs first (profiles/uniform_2p28_hbm_traffic.txt); None until that file is made.
-TRAFFIC_BYTES_PER_LAUNCH_2P28 = None
-TRAFFIC_BYTES_PER_LAUNCH_BUCKET = None
+# program runs first: 1074.0 MB read + 270.5 MB written (codes + 2 MB of per-workgroup histogram partials)
+# against 1342.2 MB algorithmic (profiles/uniform_2p28_hbm_traffic.txt), and 205.9 + 53.5 MB against 256.9 MB
+# on a 51,380,224-element bucket (profiles/cfg2_buckets_hbm_traffic.txt).
+TRAFFIC_BYTES_PER_LAUNCH_2P28 = 1344.52e6
+TRAFFIC_BYTES_PER_LAUNCH_BUCKET = 259.35e6
 
 
 def student_t3(n, device, seed, scale):

@@ -41,7 +41,13 @@ typedef struct prime_qparams {
 int prime_hip_abi_version(void);
 const char* prime_hip_last_error(void);
 
-/* Tuning knobs: "blocks_per_cu" (resident workgroups per compute unit), "hist_replicas" (copies
+/* Tuning knobs: "blocks_per_cu" (workgroups per compute unit of a streaming kernel),
+ * "large_read_grid_eighths" / "large_read_min_mi_elems" (kernels that read at least as much as they
+ * write use this many eighths of the compute units on tensors of at least that many Mi elements),
+ * "code_store_policy", "f32_store_policy", "f32_reread_store_policy", "copy_store_policy" (cache
+ * policy of the stores of codes, of fp32 outputs, of fp32 outputs the next kernel reads back, of
+ * the plain copy: 0 write-back, 2 non-temporal, 16 write-through), "reverse_second_pass" (the pass
+ * that re-reads a tensor walks it from its end), "hist_replicas" (copies
  * of each LDS histogram bin in the fused quantize pass: 1, 2, 4, 8), "nt_load_min_mib" (tensors at least this large
  * are read with non-temporal loads in their first pass), "nt_second_min_mib" (the same for the
  * quantize pass that reads a tensor for the last time).  Returns 0 if the name is known.  The

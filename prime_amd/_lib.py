@@ -95,6 +95,11 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: the HIP library is not built (run `python -m prime_amd.build`). "
             "There is no CPU fallback for these ops."
         )
+    # The library needs libamdhip64.so.7, and so does torch, which ships a copy of its own: the first
+    # one loaded serves the whole process.  torch's other ROCm libraries only work with torch's copy, so
+    # torch goes first (loading this library first, then torch, crashes at the first GPU call).
+    import torch  # noqa: F401
+
     lib = ctypes.CDLL(str(LIB_PATH))
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)   # AttributeError if the library lacks a declared symbol

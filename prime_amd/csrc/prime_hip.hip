@@ -49,12 +49,15 @@ int hip_fail(hipError_t e, const char* where) {
 }
 
 struct Options {
-    int blocks_per_cu = PRIME_BLOCKS_PER_CU;
+    int blocks_per_cu = 1;          // workgroups per compute unit a streaming kernel is launched with
+    int large_read_grid_eighths = 7;   // read-heavy kernels on large tensors: workgroups = this many eighths of the compute units
+    int64_t large_read_min_elems = int64_t(1) << 27;
     int nt_load_min_mib = 512;      // tensors of at least this many MiB are loaded with the non-temporal hint
     int nt_second_min_mib = 0;      // the same for the quantize pass that re-reads a tensor: its last use, always hinted
     int hist_replicas = 4;          // 1, 2, 4 or 8 copies of each LDS bin of the fused quantize pass
-    int code_store_policy = kStoreWriteThrough;   // cache policy of the code stores (0 plain, 2 nt, 16 write-through)
+    int code_store_policy = kStoreNt;   // cache policy of the code stores (0 plain, 2 nt, 16 write-through)
     int reverse_second_pass = 1;    // the pass that re-reads a tensor walks it from its end
+    int grid_cap = 0;               // experiment: upper bound on the workgroups of a streaming kernel (0: none)
     int f32_store_policy = kStoreWriteThrough;          // fp32 outputs nobody reads back soon (dequantize, outer step)
     int f32_reread_store_policy = kStoreWriteThrough;   // fp32 outputs the next kernel reads back (ring step, first touch)
     int copy_store_policy = kStoreNt;                   // the plain copy (the byte counters' yardstick)
@@ -75,13 +78,23 @@ int cu_count() {
 
 constexpr int64_t kRowElems = static_cast<int64_t>(kThreads) * 4;
 
-// Workgroups for a streaming kernel: one per row of kThreads 16-byte vectors until the
-// device is full (blocks_per_cu per compute unit), then each takes a longer span.
-int grid_for(int64_t n) {
+// Workgroups for a streaming kernel: one per row of kThreads 16-byte vectors until the device is
+// full (blocks_per_cu per compute unit), then each takes a longer span.  One 1024-thread workgroup
+// per compute unit is at least as fast as two from 4 Mi elements up (fewer concurrent streams into
+// HBM), and with `reads` (a kernel that reads at least as much as it writes) tensors of 2^27 elements
+// or more do best on seven eighths of the compute units: at 2^28 elements the statistics pass goes
+// from 158 to 152 us and the quantize pass from 241 to 218 us.  A kernel that mostly writes
+// (dequantize set) wants every compute unit.
+int grid_for(int64_t n, bool reads = false) {
     int64_t tiles = (n + kRowElems - 1) / kRowElems;
     if (tiles < 1) tiles = 1;
     int64_t cap = static_cast<int64_t>(cu_count()) * g_opt.blocks_per_cu;
+    if (reads && n >= g_opt.large_read_min_elems && g_opt.large_read_grid_eighths > 0) {
+        const int64_t c = static_cast<int64_t>(cu_count()) / 8 * g_opt.large_read_grid_eighths;
+        if (c >= 8 && c < cap) cap = c;
+    }
     if (cap > kMaxGrid) cap = kMaxGrid;
+    if (g_opt.grid_cap > 0 && cap > g_opt.grid_cap) cap = g_opt.grid_cap;
     return static_cast<int>(tiles < cap ? tiles : cap);
 }
 
@@ -155,7 +168,7 @@ int run_stats_finalize(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
 
 // First stage only: returns the number of partials through *parts.
 int run_stats_partials(const float* x, int64_t n, Workspace* ws, hipStream_t st, int* parts) {
-    const int grid = grid_for(n);
+    const int grid = grid_for(n, true);
     if (!aligned_to(x, 16))
         launch(kIdStats, 4.0 * n, stats_kernel<false, false>, grid, kThreads, st, x, n, ws);
     else if (use_nt(n))
@@ -180,7 +193,7 @@ void launch_quantize_p(bool al, int grid, hipStream_t st, const float* x, int64_
     while ((1 << (shift + 1)) <= g_opt.hist_replicas) ++shift;
     if (!al)
         launch(id, 5.0 * n, quantize_kernel<false, false, HIST, REVERSE, kStorePlain>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
-    else if (stats_parts != 0 ? (n >> 18) >= g_opt.nt_second_min_mib : use_nt(n))
+    else if ((n >> 18) >= g_opt.nt_second_min_mib)      // the quantize pass is always the last reader of the tensor
         launch(id, 5.0 * n, quantize_kernel<true, true, HIST, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
     else
         launch(id, 5.0 * n, quantize_kernel<true, false, HIST, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
@@ -210,7 +223,7 @@ void launch_quantize_r(bool al, bool reverse, int grid, hipStream_t st, const fl
 int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_qparams* qp_out, int zp, uint8_t* codes,
                  Workspace* ws, bool hist, hipStream_t st, int* grid_out, bool second_pass = false) {
     if (hist && zp != kZeroPoint) return fail(PRIME_EINVAL, "the fused quantize + lookup pass has zero point 128");
-    const int grid = grid_for(n);
+    const int grid = grid_for(n, true);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
     const bool rev = second_pass && g_opt.reverse_second_pass;
     if (!hist) launch_quantize_r<false>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
@@ -245,7 +258,7 @@ void launch_dequant(int id, double bytes, int grid, hipStream_t st, float* out, 
 template <bool ADD, bool STATS, bool DIV = false>
 int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, Workspace* ws, hipStream_t st, int* grid_out,
                 float divisor = 1.0f) {
-    const int grid = grid_for(n);
+    const int grid = grid_for(n, ADD);        // accumulate reads 5 bytes per element and writes 4; set reads 1 and writes 4
     const int id = STATS ? (ADD ? kIdDequantAddStats : kIdDequantSetStats) : (ADD ? kIdDequantAdd : kIdDequantSet);
     const double bytes = (ADD ? 9.0 : 5.0) * n;
     const int pol = STATS ? g_opt.f32_reread_store_policy : g_opt.f32_store_policy;
@@ -340,6 +353,14 @@ int prime_hip_set_option(const char* name, int value) {
         if (value != kStorePlain && value != kStoreNt && value != kStoreWriteThrough)
             return fail(PRIME_EINVAL, "a store policy must be 0 (plain), 2 (non-temporal) or 16 (write-through)");
         (name[0] == 'c' ? g_opt.copy_store_policy : name[4] == 's' ? g_opt.f32_store_policy : g_opt.f32_reread_store_policy) = value;
+    } else if (!strcmp(name, "large_read_grid_eighths")) {
+        if (value < 0 || value > 16) return fail(PRIME_EINVAL, "large_read_grid_eighths must be 0 (off) .. 16");
+        g_opt.large_read_grid_eighths = value;
+    } else if (!strcmp(name, "large_read_min_mi_elems")) {
+        if (value < 0) return fail(PRIME_EINVAL, "large_read_min_mi_elems must be >= 0");
+        g_opt.large_read_min_elems = static_cast<int64_t>(value) << 20;
+    } else if (!strcmp(name, "grid_cap")) {
+        g_opt.grid_cap = value;
     } else if (!strcmp(name, "reverse_second_pass")) {
         g_opt.reverse_second_pass = value != 0;
     } else if (!strcmp(name, "nt_load_min_mib")) {
@@ -360,6 +381,9 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "hist_replicas")) *value = g_opt.hist_replicas;
     else if (!strcmp(name, "code_store_policy")) *value = g_opt.code_store_policy;
     else if (!strcmp(name, "reverse_second_pass")) *value = g_opt.reverse_second_pass;
+    else if (!strcmp(name, "large_read_grid_eighths")) *value = g_opt.large_read_grid_eighths;
+    else if (!strcmp(name, "large_read_min_mi_elems")) *value = static_cast<int>(g_opt.large_read_min_elems >> 20);
+    else if (!strcmp(name, "grid_cap")) *value = g_opt.grid_cap;
     else if (!strcmp(name, "f32_store_policy")) *value = g_opt.f32_store_policy;
     else if (!strcmp(name, "f32_reread_store_policy")) *value = g_opt.f32_reread_store_policy;
     else if (!strcmp(name, "copy_store_policy")) *value = g_opt.copy_store_policy;
@@ -445,7 +469,7 @@ int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64
     Workspace* w = static_cast<Workspace*>(ws);
     int grid = 0;
     if (n > 0) {
-        grid = grid_for(n);
+        grid = grid_for(n, true);
         const int nb = static_cast<int>(n_bins < kBins ? n_bins : kBins);
         if (aligned_to(x, 16) && aligned_to(codes, 4))
             launch(kIdHist, 5.0 * n, hist_kernel<true, 8>, grid, kThreads, st, x, codes, n, nb, w);
@@ -667,7 +691,7 @@ int prime_ring_first_touch(const float* outer, const float* inner, int64_t n, fl
         if (int rc = run_stats(outer, 0, qparams_out, w, st)) return rc;
         return run_lut_finalize(w, 0, lut_out, kBins, nullptr, st);
     }
-    int grid = grid_for(n);
+    int grid = grid_for(n, true);
     const bool al = aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(grad_out, 16) && (!codes_in || aligned_to(codes_in, 4));
     const uint8_t* no_codes = nullptr;
     const float* no_lut = nullptr;

@@ -3,6 +3,7 @@
     python -m prime_amd.rocprof_summary trace    <dir> [--title T] [--command C]
     python -m prime_amd.rocprof_summary traffic  <fetch_dir> <write_dir> [--title T] [--command C]
     python -m prime_amd.rocprof_summary counters <dir> [<dir> ...] [--title T] [--command C]
+    (all three: [--bench-json FILE] appends the figures bench.py printed in that run, [--note TEXT])
 
 <dir> is what ``rocprofv3 ... --output-format csv -d <dir> -o bench`` wrote (it may put the files
 one level down, in a directory named after the host).  ``trace`` reads bench_kernel_trace.csv of a
@@ -126,12 +127,49 @@ def counters(directories) -> str:
     return "\n".join(lines)
 
 
+def bench_excerpt(path: str) -> str:
+    """What bench.py itself printed in the profiled run (its single JSON line): the figures it took
+    from HIP events, to set beside the profiler's."""
+    import json
+
+    text = [ln for ln in open(path).read().splitlines() if ln.startswith("{")]
+    if not text:
+        return "(no JSON line in " + path + ")"
+    d = json.loads(text[-1])
+    out = ["", "bench.py's own figures from the same run (HIP events around each launch):"]
+    if d.get("value") is not None:
+        out.append(f"  value={d['value']} GB/s ms_per_step={d['ms_per_step']} frac_of_hbm_peak={d.get('frac_of_hbm_peak')}")
+    r = d.get("roofline")
+    if r:
+        out.append("  roofline: " + json.dumps({k: v for k, v in r.items() if k not in ("on_the_buckets_of_the_step", "workload", "kernel")}))
+        b = r.get("on_the_buckets_of_the_step")
+        if b:
+            out.append("  bucket kernel: " + json.dumps({k: v for k, v in b.items() if k not in ("workload", "kernels")}))
+            for k, v in b["kernels"].items():
+                out.append(f"    {k:30s} avg_us={v['avg_us']:9.2f} algo_GBps={v['algo_GBps']}")
+    t = d.get("tensor_2p28")
+    if t:
+        for name, v in t["operations"].items():
+            out.append(f"  2^28 {name:42s} us={v['us']:9.2f} GBps={v['GBps']:8.1f} frac={v['frac_of_hbm_peak']:.4f}  " +
+                       " ".join(f"{k}={kv['avg_us']}" for k, kv in v["kernels"].items()))
+    for key in ("ring_step",):
+        if key in d:
+            out.append(f"  {key}: value={d[key]['value']} GB/s frac_of_hbm_peak={d[key]['frac_of_hbm_peak']} ms_per_hop={d[key]['ms_per_hop']}")
+            for k, v in d[key]["kernels"].items():
+                out.append(f"    {k:30s} avg_us={v['avg_us']:9.2f} algo_GBps={v['algo_GBps']}")
+    if "diloco_outer_step" in d:
+        out.append("  diloco_outer_step: " + json.dumps({k: v for k, v in d["diloco_outer_step"].items() if k != "workload"}))
+    return "\n".join(out)
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("kind", choices=("trace", "traffic", "counters"))
     ap.add_argument("dirs", nargs="+")
     ap.add_argument("--title", default="")
     ap.add_argument("--command", action="append", default=[])
+    ap.add_argument("--note", action="append", default=[])
+    ap.add_argument("--bench-json", default="", help="stdout of the profiled bench.py run: its own figures are appended")
     args = ap.parse_args(argv)
     head = []
     if args.title:
@@ -148,7 +186,9 @@ def main(argv=None) -> int:
         body = traffic(args.dirs[0], args.dirs[1])
     else:
         body = counters(args.dirs)
-    print("\n".join(head) + body)
+    tail = bench_excerpt(args.bench_json) if args.bench_json else ""
+    notes = "".join("\nnote: " + n for n in args.note)
+    print("\n".join(head) + body + ("\n" + tail if tail else "") + notes)
     return 0
 
 
