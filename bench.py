@@ -56,11 +56,11 @@ RING_CHUNK = 1 << 26
 N28 = 1 << 28
 # HBM bytes one launch of the dominant kernel moves on a 2^28-element tensor, from rocprofv3
 # FETCH_SIZE / WRITE_SIZE scaled by the same counters' readings for the 1 GiB copy that this
-# program runs first: 1074.0 MB read + 270.5 MB written (codes + 2 MB of per-workgroup histogram partials)
-# against 1342.2 MB algorithmic (profiles/uniform_2p28_hbm_traffic.txt), and 205.9 + 53.5 MB against 256.9 MB
+# program runs first: 1074.0 MB read + 269.3 MB written (codes + 0.9 MB of per-workgroup histogram partials)
+# against 1342.2 MB algorithmic (profiles/uniform_2p28_hbm_traffic.txt), and 205.8 + 52.4 MB against 256.9 MB
 # on a 51,380,224-element bucket (profiles/cfg2_buckets_hbm_traffic.txt).
-TRAFFIC_BYTES_PER_LAUNCH_2P28 = 1344.52e6
-TRAFFIC_BYTES_PER_LAUNCH_BUCKET = 259.35e6
+TRAFFIC_BYTES_PER_LAUNCH_2P28 = 1343.36e6
+TRAFFIC_BYTES_PER_LAUNCH_BUCKET = 258.27e6
 
 
 def student_t3(n, device, seed, scale):
@@ -374,12 +374,14 @@ def main() -> int:
         for seed in range(3):          # three tensors in rotation: 3 GiB between two visits of the same data
             g = torch.Generator(device=dev).manual_seed(seed)
             xs28.append(torch.randn(n28, device=dev, generator=g) * 1e-3)
-        c28 = torch.empty(n28, dtype=torch.uint8, device=dev)
+        # outputs rotate too: a single reused 256 MiB code buffer would live in the last-level cache and its
+        # writes would never reach HBM
+        c28s = [torch.empty(n28, dtype=torch.uint8, device=dev) for _ in range(3)]
+        o28s = [torch.empty(n28, device=dev) for _ in range(3)]
         cin28 = torch.empty(n28, dtype=torch.uint8, device=dev)
         l28 = torch.empty(256, dtype=torch.float32, device=dev)
         lin28 = torch.empty(256, dtype=torch.float32, device=dev)
         qp28 = torch.empty(4, dtype=torch.float64, device=dev)
-        o28 = torch.empty(n28, device=dev)
         uniform(xs28[0], cin28, lin28, qp28)
         torch.cuda.synchronize()
         scale28 = float(ops.unpack_qparams(qp28)["scale"])
@@ -388,22 +390,22 @@ def main() -> int:
         calls = {
             "stats (norm)": (4, lambda r: lib.prime_stats_f32(xs28[r % 3].data_ptr(), n28, qp28.data_ptr(), ws.data_ptr(), st)),
             "quantize_per_tensor_uint8 (a2)": (5, lambda r: lib.prime_quantize_u8(xs28[r % 3].data_ptr(), n28, ctypes.c_float(scale28), 128,
-                                                                               c28.data_ptr(), st)),
+                                                                               c28s[r % 3].data_ptr(), st)),
             "average_buckets (a3)": (5, lambda r: lib.prime_average_buckets(xs28[r % 3].data_ptr(), cin28.data_ptr(), n28, 256, l28.data_ptr(),
                                                                             None, ws.data_ptr(), st)),
-            "index_add (a4)": (9, lambda r: lib.prime_dequant_add(o28.data_ptr(), lin28.data_ptr(), cin28.data_ptr(), n28, st)),
-            "index_set (a5)": (5, lambda r: lib.prime_dequant_set(o28.data_ptr(), lin28.data_ptr(), cin28.data_ptr(), n28, st)),
+            "index_add (a4)": (9, lambda r: lib.prime_dequant_add(o28s[r % 3].data_ptr(), lin28.data_ptr(), cin28.data_ptr(), n28, st)),
+            "index_set (a5)": (5, lambda r: lib.prime_dequant_set(o28s[r % 3].data_ptr(), lin28.data_ptr(), cin28.data_ptr(), n28, st)),
             "quantize + lookup, scale given (K2+K3)": (5, lambda r: lib.prime_quantize_lookup_u8(xs28[r % 3].data_ptr(), n28, ctypes.c_float(scale28),
-                                                                                                c28.data_ptr(), l28.data_ptr(), ws.data_ptr(), st)),
-            "uniform_8bit_quantize (a1)": (9, lambda r: lib.prime_uniform_8bit_quantize(xs28[r % 3].data_ptr(), n28, c28.data_ptr(), l28.data_ptr(),
+                                                                                                c28s[r % 3].data_ptr(), l28.data_ptr(), ws.data_ptr(), st)),
+            "uniform_8bit_quantize (a1)": (9, lambda r: lib.prime_uniform_8bit_quantize(xs28[r % 3].data_ptr(), n28, c28s[r % 3].data_ptr(), l28.data_ptr(),
                                                                                         qp28.data_ptr(), ws.data_ptr(), st)),
-            "ring reduce step (a4 + a1)": (14, lambda r: lib.prime_ring_reduce_step(xs28[1 + r % 2].data_ptr(), cin28.data_ptr(), lin28.data_ptr(), n28,
-                                                                                   c28.data_ptr(), l28.data_ptr(), None, ws.data_ptr(), st)),
+            "ring reduce step (a4 + a1)": (14, lambda r: lib.prime_ring_reduce_step(o28s[r % 3].data_ptr(), cin28.data_ptr(), lin28.data_ptr(), n28,
+                                                                                   c28s[r % 3].data_ptr(), l28.data_ptr(), None, ws.data_ptr(), st)),
         }
         rows, uni_prof = {}, None
         only = [w for w in args.t28_ops.split(",") if w]
         for name, (bpe, fn) in calls.items():
-            if only and not name.startswith("uniform") and not any(w in name for w in only):
+            if only and name != "uniform_8bit_quantize (a1)" and not any(w in name for w in only):
                 continue
             for r in range(args.warmup):
                 _lib.check(fn(r), name)
@@ -423,13 +425,14 @@ def main() -> int:
                           "elements_per_s": round(n28 / (kern_us * 1e-6), 1), "frac_of_hbm_peak": round(bpe * n28 / kern_us / 1e3 / HBM_PEAK_GBS, 4),
                           "us_wall_back_to_back": round(wall * 1e6, 2),
                           "kernels": {k: {"avg_us": round(us, 2), "algo_GBps": round(b / us / 1e3, 1)} for k, (us, b) in per28.items()}}
-            if name.startswith("uniform"):
+            if name == "uniform_8bit_quantize (a1)":
                 uni_prof = per28
         dom_us, dom_bytes = uni_prof["quantize_kernel+hist"]
         uni, ring28 = rows["uniform_8bit_quantize (a1)"], rows.get("ring reduce step (a4 + a1)", {})
         out["tensor_2p28"] = {
-            "workload": "2^28-element fp32 tensors N(0,1e-3), three in rotation; per operation: sum of its kernels' launch times "
-                        "(HIP events per launch), and wall time of back-to-back calls",
+            "workload": "2^28-element fp32 tensors N(0,1e-3), inputs and outputs three in rotation (3 GiB between two visits of the same "
+                        "buffer); per operation: sum of its kernels' launch times (HIP events per launch), and wall time of "
+                        "back-to-back calls",
             "value": uni["GBps"], "unit": "GB/s", "ms": round(uni["us"] / 1e3, 4), "elements_per_s": uni["elements_per_s"],
             "frac_of_hbm_peak": uni["frac_of_hbm_peak"],
             "ring_reduce_step": {"value": ring28["GBps"], "unit": "GB/s", "ms": round(ring28["us"] / 1e3, 4),
@@ -439,8 +442,8 @@ def main() -> int:
         out["roofline"] = {
             "bound": "hbm",
             "kernel": "quantize_kernel<aligned, nt loads, hist, write-through stores> (quantize + 256-bin sum/count histogram)",
-            "workload": "inside uniform_8bit_quantize on 2^28-element tensors (1 GiB each, three in rotation: nothing of the tensor "
-                        "is left in the 256 MB last-level cache when the call starts)",
+            "workload": "inside uniform_8bit_quantize on 2^28-element tensors (1 GiB each; inputs and code buffers three in rotation: "
+                        "nothing of either is left in the 256 MB last-level cache when the call starts)",
             "achieved": round(dom_bytes / dom_us / 1e3, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -451,7 +454,7 @@ def main() -> int:
             **overhead_note,
             "on_the_buckets_of_the_step": bucket_kernel,
         }
-        del xs28, c28, cin28, o28
+        del xs28, c28s, cin28, o28s
         torch.cuda.empty_cache()
     elif bucket_kernel is not None:
         out["roofline"] = {"bound": "hbm", "kernel": "quantize_kernel+hist", "workload": bucket_kernel["workload"],
