@@ -151,7 +151,8 @@ int prime_uniform_8bit_quantize_buckets(const float* const* xs, const int64_t* n
 /* Many tensors in one launch: tensor t is x[offsets[t] .. offsets[t+1]) of a flat buffer, the
  * layout of the per-layer views of Diloco's flat pseudo-gradient buffer
  * (src/zeroband/diloco.py:147-201), each handled as uniform_8bit_quantize handles one tensor.
- * offsets: count+1 int64 on the device.  codes uses the same offsets; luts is count x 256;
+ * offsets: count+1 non-decreasing int64 on the device (not checked: they are read by the kernel).
+ * x and codes may be NULL only when count is 0.  codes uses the same offsets; luts is count x 256;
  * qparams_out (optional) is count entries.  Meant for small tensors: one workgroup each. */
 int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, int64_t count,
                                         uint8_t* codes, float* luts, prime_qparams* qparams_out,

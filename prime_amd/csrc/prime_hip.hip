@@ -557,7 +557,8 @@ int prime_uniform_8bit_quantize_buckets(const float* const* xs, const int64_t* n
 
 int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, int64_t count, uint8_t* codes, float* luts,
                                         prime_qparams* qparams_out, prime_stream_t stream) {
-    if (count < 0 || (count > 0 && (!offsets || !luts))) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: bad argument");
+    if (count < 0 || (count > 0 && (!offsets || !luts || !x || !codes)))
+        return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: bad argument");
     if (count > 0x7fffffff) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_batched: too many tensors");
     if (count == 0) return 0;
     if (aligned_to(x, 16) && aligned_to(codes, 4))

@@ -160,5 +160,19 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
 
 def ring_allreduce_single(tensor: torch.Tensor, avg: bool = False) -> None:
     """``ring_allreduce`` on a group of one rank: no message is sent, but both of the rank's
-    chunks still take the lossy quantize / dequantize round trip (collectives.cpp:161-173)."""
-    ring_allreduce_simulated([tensor.view(-1)], avg=avg)
+    chunks still take the lossy quantize / dequantize round trip (collectives.cpp:161-173).
+    The two chunks are those of ``flat.chunk(2)`` (:90): ceil(n / 2) elements and the rest, so an
+    odd number of elements is fine here, as it is in the reference's C++ (its Python twin's
+    divisibility check, src/zeroband/collectives.py:83, only matters for more than one rank)."""
+    flat = tensor.view(-1)
+    n = flat.numel()
+    if n % BUFFER_COUNT == 0:
+        ring_allreduce_simulated([flat], avg=avg)
+        return
+    if n < BUFFER_COUNT:
+        raise ValueError("a tensor of one element has no second chunk (collectives.cpp:161 indexes chunks[1])")
+    _check_ring_inputs([flat[:n - 1]])          # dtype, contiguity
+    first = (n + BUFFER_COUNT - 1) // BUFFER_COUNT
+    for ch in (flat[:first], flat[first:]):
+        codes, lut = ops.uniform_8bit_quantize(ch, True)                     # :162 (dividing by 1 changes nothing)
+        ops.dequantize_(ch, codes, lut, False)                               # :167-172

@@ -31,8 +31,9 @@ OUT_LARGE = Path(__file__).resolve().parent / "uniform8_reference_large.json"
 
 # Large cases are stored as digests: the scale bits, the SHA-256 of the codes and the code
 # populations.  At these sizes libtorch's norm differs visibly from the exact one (config 1 of the
-# benchmark is "normal:16777216"), so they pin the literal path where it matters.
-LARGE_CASES = ["normal:1048583", "student:4194304", "normal:16777216"]
+# benchmark is "normal:16777216"; 2^26 is the ring chunk of config 3 and 2^28 the size the throughput target is quoted on,
+# where the norm is 5e-3 and 3.7e-2 low), so they pin the literal path where it matters.
+LARGE_CASES = ["normal:1048583", "student:4194304", "normal:16777216", "normal:67108864", "normal:268435456"]
 
 
 def case_input(name: str) -> np.ndarray:

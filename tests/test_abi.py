@@ -51,6 +51,11 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.prime_copy_bytes(ctypes.c_void_p(4096), ctypes.c_void_p(8192), 7, None) == -1
     assert lib.prime_average_buckets(ctypes.c_void_p(4096), ctypes.c_void_p(4096), 4, 0, ctypes.c_void_p(4096),
                                      None, ctypes.c_void_p(4096), None) == -1    # n_bins < 1
+    p = ctypes.c_void_p(4096)
+    assert lib.prime_uniform_8bit_quantize_batched(None, p, 3, p, p, None, None) == -1       # null x with tensors to do
+    assert lib.prime_uniform_8bit_quantize_batched(p, p, 3, None, p, None, None) == -1       # null codes
+    assert lib.prime_uniform_8bit_quantize_batched(p, None, 3, p, p, None, None) == -1       # null offsets
+    assert lib.prime_uniform_8bit_quantize_batched(None, None, 0, None, None, None, None) == 0   # nothing to do
     assert lib.prime_ring_reduce_step(ctypes.c_void_p(4096), ctypes.c_void_p(4096), ctypes.c_void_p(4096), 4,
                                       ctypes.c_void_p(4096), ctypes.c_void_p(4096), None, None, None) == -2
 

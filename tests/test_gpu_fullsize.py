@@ -56,14 +56,15 @@ def test_uniform_8bit_quantize_2p28_properties(abi):
 
 
 def test_ring_reduce_step_2p26_chunks(abi):
-    # benchmark configuration 3 shape: 2^26-element chunks; three ranks' worth to bound memory and time
+    # benchmark configuration 3 in full: W = 8 ranks' 2^26-element chunks N(0, 1e-3), seed = rank; chunk 0 is
+    # quantized, then all 7 hops of dequantize-add + requantize, each checked through properties
     n = 1 << 26
-    g = torch.Generator(device=abi.dev).manual_seed(1)
-    x0 = torch.randn(n, device=abi.dev, generator=g) * 1e-3
+    x0 = torch.randn(n, device=abi.dev, generator=torch.Generator(device=abi.dev).manual_seed(0)) * 1e-3
     announce("2^26 ring: quantize rank 0")
     codes, lut, _ = abi.uniform(x0)
-    for r in (1, 2):
-        acc = torch.randn(n, device=abi.dev, generator=g) * 1e-3
+    del x0
+    for r in range(1, 8):
+        acc = torch.randn(n, device=abi.dev, generator=torch.Generator(device=abi.dev).manual_seed(r)) * 1e-3
         want = acc + lut[codes.long()]
         announce(f"2^26 ring hop {r}")
         codes, lut, qp = abi.ring_step(acc, codes, lut)
@@ -72,10 +73,17 @@ def test_ring_reduce_step_2p26_chunks(abi):
         q = abi.qparams(qp)
         sumsq = float((want.double() ** 2).sum())
         assert abs(q["sumsq"] - sumsq) <= 1e-12 * sumsq
+        exact = np.float32(6.0 * (float(np.float32(np.sqrt(sumsq))) / np.sqrt(n - 1)) / 256.0)
+        assert abs(float(q["scale"]) - float(exact)) <= 1e-6 * float(exact)
         cnt = torch.bincount(codes.int(), minlength=256)
         assert int(cnt.sum()) == n
         inside = (codes > 0) & (codes < 255)
         assert float((lut[codes.long()] - want)[inside].abs().max()) <= float(q["scale"])
+        sums = torch.bincount(codes.int(), weights=want.double(), minlength=256)
+        mean = torch.where(cnt > 0, sums / cnt.clamp(min=1).double(), torch.zeros_like(sums))
+        floor = torch.tensor(float(q["scale"]), device=abi.dev, dtype=torch.float64)
+        assert float(((lut.double() - mean).abs() / torch.maximum(mean.abs(), floor)).max()) <= 1e-6
+        del want, acc
 
 
 def test_config4_shard_all_42_buckets(abi):

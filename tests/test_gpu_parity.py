@@ -43,9 +43,14 @@ def check_uniform(abi, oracle, x: np.ndarray, label: str):
     assert np.array_equal(np.array([q["scale"]]), np.array([want_scale]), equal_nan=True), (label, q["scale"], want_scale)
     oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
     assert np.array_equal(gc, oc), (label, int((gc != oc).sum()))
-    mean, _ = oracle.average_buckets_f64(x, gc)
+    mean, cnt = oracle.average_buckets_f64(x, gc)
     floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1.0
     assert lut_rel_err(gl, mean, floor) <= LUT_TOL, label
+    assert not gl[cnt == 0].any(), label                       # an empty bin is 0.0f (compression.cpp:100)
+    # the bin populations behind the table: the histogram under the same codes, counts exact
+    lut2, cnt2 = abi.average_buckets(xt, codes)
+    assert np.array_equal(cnt2.cpu().numpy(), cnt), label
+    assert tables_agree(lut2.cpu().numpy(), gl, floor, 2 * LUT_TOL), label
     return xt, codes, lut, q
 
 
@@ -348,8 +353,9 @@ def test_golden_fixtures_of_the_compiled_reference(abi, oracle, golden, name):
         if float(q["scale"]) == ref_scale:
             assert not diff.any()
         else:
-            # a scale one ulp away may move elements that sit on a bin boundary, by one code
-            assert diff.mean() <= 1e-4
+            # a scale within 1e-6 may move elements that sit on a bin boundary, by one code: an element
+            # moves only if |x| / scale is within 1e-6 * 128 bins of a boundary, about n * 128 * 1e-6 * 2 of them
+            assert int(diff.sum()) <= math.ceil(x.size * 34 * 2.0 ** -24) + 1
             d = codes.cpu().numpy().astype(int)[diff] - golden[f"{key}/codes"].astype(int)[diff]
             assert (np.abs(d) == 1).all()
     else:
@@ -401,7 +407,7 @@ def test_literal_norm_against_the_compiled_reference_at_2p24(abi, oracle):
     assert -2e-3 < rel < -1e-4
 
 
-@pytest.mark.parametrize("name", ["normal:1048583", "student:4194304", "normal:16777216"])
+@pytest.mark.parametrize("name", ["normal:1048583", "student:4194304", "normal:16777216", "normal:67108864", "normal:268435456"])
 def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, name):
     # fixtures that travel without the reference: scale bits, SHA-256 of the codes and code populations of
     # the compiled reference at sizes up to the benchmark's first configuration (2^24 elements)
@@ -420,13 +426,28 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
     assert hashlib.sha256(gc.tobytes()).hexdigest() == want["codes_sha256"]
     assert np.bincount(gc, minlength=256).tolist() == want["counts"]
     ref_lut = np.array(want["lut"], np.float32)
-    assert lut_rel_err(lut.cpu().numpy(), ref_lut.astype(np.float64), float(q["scale"])) < 2e-5
+    # the reference's table is a sequential fp32 sum per thread: its own error grows with the bin populations
+    # (2e-5 up to 2^24 elements, 4e-4 at 2^28); the GPU's table is held to the fp64 means
+    assert lut_rel_err(lut.cpu().numpy(), ref_lut.astype(np.float64), float(q["scale"])) < 2e-5 * max(1.0, 2.0 * x.size / (1 << 24))
+    cnt = np.bincount(gc, minlength=256)
+    mean = np.bincount(gc, weights=x.astype(np.float64), minlength=256) / np.maximum(cnt, 1)
+    assert lut_rel_err(lut.cpu().numpy(), mean, float(q["scale"])) <= LUT_TOL
     # the default path uses the exact norm: same codes for all but the elements the scale difference moves
-    codes_e, _, qp_e = abi.uniform(abi.to_dev(x))
+    codes_e, lut_e, qp_e = abi.uniform(abi.to_dev(x))
     rel = float(q["scale"]) / float(abi.qparams(qp_e)["scale"]) - 1
-    assert -2e-3 < rel <= 0
-    moved = (codes_e.cpu().numpy() != gc).mean()
+    assert -5e-2 < rel <= 0
+    ce = codes_e.cpu().numpy()
+    moved = (ce != gc).mean()
     assert moved <= 45 * abs(rel) + 1e-6          # a code moves when |x| / scale crosses a boundary: at most ~|code - 128| * |rel|
+    # the default (exact-norm) output against the reference's own: a code moves by |code - 128| * |rel| bins at
+    # most, towards the centre, and the table's entries by the same relative amount
+    step = np.abs(ce.astype(np.int16) - gc.astype(np.int16))
+    assert int(step.max()) <= math.ceil(128 * abs(rel) + 0.5)
+    if abs(rel) < 3e-3:
+        assert int(step.max()) <= 1
+    le = lut_e.cpu().numpy().astype(np.float64)
+    both = (np.bincount(ce, minlength=256) > 0) & (np.array(want["counts"]) > 0)
+    assert np.all(np.abs(le - ref_lut)[both] <= (3 * abs(rel) + 2e-5) * np.maximum(np.abs(ref_lut[both]), float(q["scale"])))
 
 
 @pytest.mark.parametrize("option,values", [("hist_replicas", (1, 2, 4, 8)), ("blocks_per_cu", (1, 2, 3, 4)),

@@ -247,3 +247,57 @@ def test_reference_import_paths_reach_the_hip_kernels(dev):
         shim.uninstall()
         for k in [k for k in sys.modules if k == "zeroband" or k.startswith("zeroband.")]:
             del sys.modules[k]
+
+
+@pytest.mark.parametrize("W", [1, 2, 3, 4, 8])
+@pytest.mark.parametrize("avg", [False, True])
+@pytest.mark.parametrize("code_domain", [False, True])
+def test_ring_closed_form_on_chunkwise_constant_inputs(dev, W, avg, code_domain):
+    # rank r's chunk c is a constant; constant chunks quantize without loss and every partial sum is a
+    # small integer, so the ring must return exactly sum_r v[r, c] (divided by W for AVG) in every
+    # element of chunk c on every rank: pins the chunk-index algebra (collectives.cpp:116, 192), the
+    # forwarding condition (:136, :212), the division (:155-159) and the own-chunk round trip
+    # (:161-173) bit for bit, with the same inputs as the oracle's own closed-form test
+    from prime_amd import ops, ring
+    from tests.test_oracle_pins import closed_form_ring_inputs
+
+    csz = 4096
+    v, tensors = closed_form_ring_inputs(W, csz)
+    announce(f"closed-form ring W={W} avg={avg} code_domain={code_domain}")
+    gpu = [torch.from_numpy(t).to(dev) for t in tensors]
+    final = ring.ring_allreduce_simulated(gpu, avg=avg, keep_codes=code_domain)
+    torch.cuda.synchronize()
+    total = v.sum(axis=0, dtype=np.float64).astype(np.float32)
+    want = total / np.float32(W) if avg else total
+    for rk in range(W):
+        if code_domain:
+            got = np.stack([ops.dequantize(*final[rk][c]).cpu().numpy() for c in range(2 * W)])
+        else:
+            got = gpu[rk].cpu().numpy().reshape(2 * W, csz)
+        for c in range(2 * W):
+            assert np.all(got[c] == want[c]), (W, avg, rk, c, got[c][:3], want[c])
+
+
+@pytest.mark.parametrize("n", [3, 7, 1001, 65537])
+def test_single_rank_group_takes_an_odd_number_of_elements(dev, oracle, n):
+    # flat.chunk(2) of the reference's C++ (collectives.cpp:90): ceil(n / 2) elements and the rest, each
+    # through the quantize / dequantize round trip (:161-173)
+    from prime_amd import ring
+
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    t = torch.from_numpy(x.copy()).to(dev)
+    announce(f"single rank odd n={n}")
+    ring.ring_allreduce_single(t)
+    torch.cuda.synchronize()
+    (lo0, hi0), (lo1, hi1) = oracle.torch_chunk_bounds(n, 2)
+    want = x.copy()
+    for lo, hi in ((lo0, hi0), (lo1, hi1)):
+        codes, _, scale = oracle.uniform_8bit_quantize(x[lo:hi], "exact")
+        mean, _ = oracle.average_buckets_f64(x[lo:hi], codes)
+        want[lo:hi] = mean.astype(np.float32)[codes]
+    got = t.cpu().numpy()
+    floor = 6 * 1e-3 / 256
+    assert np.all(np.abs(got - want) <= 1e-6 * np.maximum(np.abs(want), floor))
+    with pytest.raises(ValueError):
+        ring.ring_allreduce_single(torch.zeros(1, device=dev))

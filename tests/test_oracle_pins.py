@@ -356,7 +356,7 @@ def test_outer_sgd_nesterov_is_torch_sgd_bit_for_bit(oracle):
                 assert np.array_equal(buf, opt.state[p]["momentum_buffer"].numpy()), (n, lr, mu, step)
 
 
-@pytest.mark.parametrize("name", ["normal:1048583", "student:4194304", "normal:16777216"])
+@pytest.mark.parametrize("name", ["normal:1048583", "student:4194304", "normal:16777216", "normal:67108864", "normal:268435456"])
 def test_oracle_reproduces_the_large_digests_of_the_compiled_reference(oracle, name):
     # sizes where libtorch's norm visibly differs from the exact one: the literal restatement must give
     # the reference's scale bits and codes (SHA-256 and populations written by tests/golden/make_fixtures.py)
@@ -375,7 +375,45 @@ def test_oracle_reproduces_the_large_digests_of_the_compiled_reference(oracle, n
     assert hashlib.sha256(codes.tobytes()).hexdigest() == want["codes_sha256"]
     assert np.bincount(codes, minlength=256).tolist() == want["counts"]
     ref_lut = np.array(want["lut"], np.float32)
-    assert np.abs(lut - ref_lut).max() <= 2e-5 * max(float(scale), np.abs(ref_lut).max())
-    # and the exact scale is larger, by libtorch's accumulation loss
+    assert np.abs(lut - ref_lut).max() <= 2e-5 * max(1.0, 2.0 * x.size / (1 << 24)) * max(float(scale), np.abs(ref_lut).max())
+    # and the exact scale is larger, by libtorch's accumulation loss (-7e-4 at 2^24, -5e-3 at 2^26, -3.7e-2 at 2^28)
     rel = float(scale) / float(oracle.scale_exact(x)) - 1
-    assert -2e-3 < rel <= 0
+    assert -5e-2 < rel <= 0
+    if x.size >= 1 << 26:
+        assert rel < -2e-3
+
+
+def closed_form_ring_inputs(W: int, csz: int):
+    """Rank r's chunk c is the constant 100 (r + 1) + c, except that chunk 1 sums to zero over the
+    ranks and chunk 0 is negative.  A constant chunk quantizes without loss (every element in one
+    bin whose mean is the constant; an all-zero chunk in code 0 with mean 0), and every partial sum
+    is a small integer, so ring_allreduce must return exactly sum_r v[r, c] in every element of
+    chunk c on every rank: one misrouted, dropped or repeated message changes that."""
+    import numpy as np
+
+    nb = 2 * W
+    v = np.zeros((W, nb), np.float32)
+    for r in range(W):
+        for c in range(nb):
+            v[r, c] = 100 * (r + 1) + c
+    v[:, 0] *= -1
+    if W > 1:
+        v[:, 1] = np.arange(W) - (W - 1) / 2.0 if W % 2 else np.arange(W) * 2 - (W - 1)      # sums to zero, integers
+    tensors = [np.repeat(v[r], csz).astype(np.float32) for r in range(W)]
+    return v, tensors
+
+
+@pytest.mark.parametrize("W", [1, 2, 3, 4, 8])
+@pytest.mark.parametrize("avg", [False, True])
+def test_ring_sim_closed_form_on_chunkwise_constant_inputs(oracle, W, avg):
+    # pins the chunk-index algebra (collectives.cpp:116, 192), the forwarding condition (:136, :212),
+    # the division for AVG (:155-159) and the own-chunk round trip (:161-173) exactly
+    csz = 512
+    v, tensors = closed_form_ring_inputs(W, csz)
+    oracle.ring_allreduce_sim(tensors, avg=avg)
+    total = v.sum(axis=0, dtype=np.float64).astype(np.float32)
+    want = total / np.float32(W) if avg else total
+    for r in range(W):
+        got = tensors[r].reshape(2 * W, csz)
+        for c in range(2 * W):
+            assert np.all(got[c] == want[c]), (W, avg, r, c, got[c][:3], want[c])
