@@ -1,15 +1,18 @@
 """Drop-in for ``zeroband.C.collectives`` (src/zeroband/C/collectives.py:23-35):
 ``ring_allreduce(tensor, op, group)`` with the per-hop compute on the GPU.
 
-This build runs on one GPU and contains no transport.  Groups it accepts:
+Groups it accepts:
 
+* a real c10d process group with a host (Gloo) backend, as the reference uses
+  (``ProcessGroupGloo``, C/collectives.py:30-35): one process per rank, messages through pinned host
+  memory and ``dist.isend`` / ``dist.irecv`` (``prime_amd.wire.ring_allreduce_group``); the ranks may
+  share one GPU.  A group of size 1 is the single rank's quantize / dequantize round trip;
 * a ``SimulatedRing`` holding the tensors of W ranks on one device: the full schedule runs
-  locally (``prime_amd.ring.ring_allreduce_simulated``);
-* ``FakeProcessGroup``: returns at once, as the reference does (C/collectives.py:32-33);
-* a real process group of size 1 (or the default group when it has one rank): the single
-  rank's quantize / dequantize round trip.
+  in one process (``prime_amd.ring.ring_allreduce_simulated``);
+* ``FakeProcessGroup``: returns at once, as the reference does (C/collectives.py:32-33).
 
-A real group with more than one rank raises NotImplementedError.
+A group whose backend cannot move host tensors (NCCL / RCCL only) raises NotImplementedError: a
+device-to-device transport needs a second GPU and is not part of this build.
 """
 from __future__ import annotations
 
@@ -65,6 +68,11 @@ def ring_allreduce(
     if group.size() == 1:
         ring.ring_allreduce_single(tensor, avg=avg)
         return
-    raise NotImplementedError(
-        "ring_allreduce over a real process group of more than one rank needs a transport, "
-        "which this single-GPU build does not contain; use SimulatedRing")
+    backend = str(dist.get_backend(group)).lower()
+    if "gloo" not in backend:
+        raise NotImplementedError(
+            f"ring_allreduce moves its messages through host memory and needs a Gloo group (got backend {backend!r}); "
+            "a device-to-device transport is not part of this single-GPU build")
+    from .. import wire
+
+    wire.ring_allreduce_group(tensor, avg, group)

@@ -15,8 +15,11 @@ def gloo_all_reduce(
     op: dist.ReduceOp = dist.ReduceOp.SUM,
     group: Optional[dist.ProcessGroup] = None,
 ) -> None:
-    """Uncompressed path: pre-divide for AVG, then a SUM all-reduce (collectives.py:12-28).
-    A ``SimulatedRing`` group is reduced in place, rank 0's tensor first."""
+    """Uncompressed path, as the reference spells it (collectives.py:12-28): divide by the group size
+    for AVG, then ``dist.all_reduce(tensor, op)`` with the caller's op.  (With AVG the reference thus
+    divides and then asks the backend for AVG as well; Gloo rejects AVG, so in practice only SUM reaches
+    it.  Kept as is: this path is the reference's, not a kernel of this build.)
+    A ``SimulatedRing`` group is reduced in place: pre-division for AVG, then the sum."""
     from .C.collectives import SimulatedRing
 
     if isinstance(group, SimulatedRing):
@@ -37,7 +40,7 @@ def gloo_all_reduce(
         raise ValueError(f"Unsupported reduce operation {op}. Only SUM and AVG are supported.")
     if op == dist.ReduceOp.AVG:
         tensor.div_(group.size())
-    dist.all_reduce(tensor, dist.ReduceOp.SUM, group=group)
+    dist.all_reduce(tensor, op, group=group)
 
 
 def all_reduce(

@@ -19,15 +19,19 @@ HIP stream of default priority and are ordered against the compute stream with e
 copy of step s overlaps the kernels of step s + 1, as the reference overlaps its sends with
 the next quantization.
 
-No transport is built here (one GPU, no process group): ``Loopback`` stands in for the pair of
-``send`` / ``recv`` calls between neighbours by copying host slot to host slot, which is enough
-to run the whole schedule through the staging path and to time the PCIe side.
+Two transports sit behind the stage.  ``ring_allreduce_group`` is the reference's own: one process
+per rank, ``dist.isend`` / ``dist.irecv`` of the pinned host slots over a c10d group with a host
+(Gloo) backend, the reference's tags and its two slots in flight; the ranks may share one GPU.
+``Loopback`` stands in for the neighbour's ``send`` / ``recv`` pair inside one process (W simulated
+ranks) by copying host slot to host slot, which runs the same schedule through the staging path
+and times the PCIe side without a second process.
 """
 from __future__ import annotations
 
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
+import torch.distributed as dist
 
 from . import ops
 from .ring import BUFFER_COUNT, _check_ring_inputs
@@ -195,3 +199,72 @@ def ring_allreduce_staged(tensors: Sequence[torch.Tensor], avg: bool = False, tr
                 ops.dequantize_(ch, codes, lut, False)
     assert not own
     return transport
+
+
+_stages: Dict[Tuple[int, int], HostStage] = {}
+
+
+def _stage_for(device: torch.device, chunk_numel: int) -> HostStage:
+    """One HostStage per (device, chunk size), kept: pinned allocations are slow and the per-layer
+    buckets of a model repeat a handful of sizes."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    key = (idx, int(chunk_numel))
+    st = _stages.get(key)
+    if st is None:
+        st = _stages[key] = HostStage(torch.device("cuda", idx), chunk_numel)
+    return st
+
+
+def ring_allreduce_group(tensor: torch.Tensor, avg: bool, group) -> None:
+    """``ring_allreduce`` (collectives.cpp:76-230) for THIS rank of a real process group whose backend
+    moves host memory (Gloo).  Schedule, tags and buffering are the reference's: at step s the rank
+    waits for the four transfers posted at step s - 2 (:118-122), folds the received message into
+    chunk c(s) on the GPU, and if s <= 2 (W - 1) quantizes that chunk and posts
+    ``isend(lookup, tag s + 1000)``, ``irecv(lookup)``, ``isend(codes, tag s)``, ``irecv(codes)`` with
+    the next and previous rank (:140-150, :217-227).  Messages live in the two pinned host slots of a
+    ``HostStage``; only codes and lookup cross PCIe.  In place; every rank must call it."""
+    W = group.size()
+    rank = dist.get_rank(group)
+    flat = tensor.view(-1)
+    n = _check_ring_inputs([flat] * W)
+    nb = BUFFER_COUNT * W
+    csz = n // nb
+    stage = _stage_for(flat.device, csz)
+    dst = dist.get_global_rank(group, (rank + 1) % W)                    # :111
+    src = dist.get_global_rank(group, (rank - 1 + W) % W)               # :112
+
+    def chunk(c: int) -> torch.Tensor:
+        return flat[c * csz:(c + 1) * csz]
+
+    own: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
+    for phase in (1, 2):
+        works: Dict[int, list] = {}
+        for step in range(1, nb + 1):
+            c = ((rank * BUFFER_COUNT - step) if phase == 1 else (rank * BUFFER_COUNT + BUFFER_COUNT - step)) % nb   # :116 / :192
+            ch = chunk(c)
+            sending = step <= (W - 1) * BUFFER_COUNT                                                              # :136 / :212
+            out = None
+            if (step - BUFFER_COUNT) in works:
+                for w in works.pop(step - BUFFER_COUNT):                 # :118-122
+                    w.wait()
+                codes_in, lut_in = stage.to_device(step - BUFFER_COUNT)
+                if sending:
+                    out = (ops.ring_reduce_step if phase == 1 else ops.ring_gather_step)(ch, codes_in, lut_in)
+                elif phase == 1:
+                    own[c] = ops.ring_reduce_div_step(ch, codes_in, lut_in, float(W) if avg else 1.0)
+                else:
+                    ops.dequantize_(ch, codes_in, lut_in, False)
+                stage.release(step - BUFFER_COUNT)
+            elif sending and c in own:
+                out = ops.ring_gather_step(ch, *own.pop(c))
+            elif sending:
+                out = ops.uniform_8bit_quantize(ch, False)
+            if out is not None:
+                stage.post_send(step, out[0], out[1])
+                lut_h, codes_h = stage.take_send(step)                   # the message is in pinned host memory
+                rl, rc = stage.recv_buffers(step)
+                lut_tag, codes_tag = message_tags(step)
+                works[step] = [dist.isend(lut_h, dst, group=group, tag=lut_tag), dist.irecv(rl, src, group=group, tag=lut_tag),
+                               dist.isend(codes_h, dst, group=group, tag=codes_tag), dist.irecv(rc, src, group=group, tag=codes_tag)]
+        assert not works
+    assert not own

@@ -81,3 +81,62 @@ def test_staged_ring_reuses_its_stages_across_calls(dev):
         assert all(torch.equal(a, b) for a, b in zip(direct, staged))
     with pytest.raises(ValueError, match="HostStage"):
         wire.ring_allreduce_staged(staged, stages=stages[:1])
+
+
+def _free_port() -> int:
+    import socket
+
+    with socket.socket() as sock:
+        sock.bind(("127.0.0.1", 0))
+        return sock.getsockname()[1]
+
+
+@pytest.mark.parametrize("W,op,pg", [(2, "sum", "default"), (4, "sum", "default"), (2, "avg", "newgroup"), (4, "avg", "default")])
+def test_ring_over_a_real_gloo_group_one_process_per_rank(dev, oracle, tmp_path, W, op, pg):
+    # the reference's own acceptance test (tests/test_c/test_collectives.py:14-68): W processes on
+    # localhost, a Gloo group, each rank randn(N) * 10; here every rank's kernels run on the one GPU and
+    # only codes + lookup travel (pinned host memory, dist.isend / irecv with the reference's tags).
+    # Each rank's result must equal the simulated ring's bit for bit (same kernels, same schedule), which
+    # tracks the oracle ring; and the reference's inequality against the exact all-reduce holds.
+    import math
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from prime_amd import ring
+
+    n = 1_000_000 - 1_000_000 % (2 * W)          # N of the reference test, made divisible (collectives.py:83)
+    seed = 4000 + W
+    root = Path(__file__).resolve().parents[1]
+    port = _free_port()
+    env = dict(os.environ, PYTHONPATH=str(root))
+    announce(f"gloo ring W={W} op={op} group={pg} port={port}")
+    procs = [subprocess.Popen([sys.executable, "-u", "-m", "tests.ring_worker", str(r), str(W), str(port), str(n), str(seed), op,
+                               str(tmp_path)] + (["newgroup"] if pg == "newgroup" else []),
+                              cwd=str(root), env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True) for r in range(W)]
+    outs = []
+    try:
+        for pr in procs:
+            out, _ = pr.communicate(timeout=150)
+            outs.append(out)
+    finally:
+        for pr in procs:
+            if pr.poll() is None:
+                pr.kill()
+    for r, pr in enumerate(procs):
+        assert pr.returncode == 0, f"rank {r} failed:\n{outs[r][-3000:]}"
+    xs = [(np.random.default_rng(seed + r).standard_normal(n) * 10).astype(np.float32) for r in range(W)]
+    sim = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    ring.ring_allreduce_simulated(sim, avg=(op == "avg"))
+    cpu = [x.copy() for x in xs]
+    oracle.ring_allreduce_sim(cpu, avg=(op == "avg"))
+    torch.cuda.synchronize()
+    exact = np.sum(np.stack(xs).astype(np.float64), axis=0) / (W if op == "avg" else 1)
+    for r in range(W):
+        got = np.load(tmp_path / f"rank{r}.npy")
+        assert np.array_equal(got, sim[r].cpu().numpy()), f"rank {r} differs from the simulated ring"
+        err_new = np.linalg.norm(got - exact)
+        err_old = np.linalg.norm(cpu[r] - exact)
+        assert abs(err_new - err_old) / math.sqrt(n) < 0.5            # tests/test_c/test_collectives.py:57
+        assert abs(err_new - err_old) / math.sqrt(n) < 0.02
