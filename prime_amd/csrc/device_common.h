@@ -171,7 +171,7 @@ __device__ __forceinline__ void finalize_from_norm(float norm, double sum, doubl
 
 // Workgroup reduction of (sum, sumsq) in a fixed order; the workgroup's partial goes to the
 // workspace for stats_finalize_kernel.
-__device__ __forceinline__ void block_stats_store(double s, double q, Workspace* ws) {
+__device__ __forceinline__ void block_stats_store(double s, double q, Workspace* ws, int slot) {
     __shared__ double sh_s[kWaves];
     __shared__ double sh_q[kWaves];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -183,8 +183,8 @@ __device__ __forceinline__ void block_stats_store(double s, double q, Workspace*
         double S = sh_s[0], Q = sh_q[0];
 #pragma unroll
         for (int w = 1; w < kWaves; ++w) { S += sh_s[w]; Q += sh_q[w]; }
-        ws->part_sum[blockIdx.x] = S;
-        ws->part_sq[blockIdx.x] = Q;
+        ws->part_sum[slot] = S;
+        ws->part_sq[slot] = Q;
     }
 }
 
@@ -201,24 +201,14 @@ __device__ __forceinline__ bool narrow_distribution(double sum, double sumsq, in
 // workgroup adds the same partials in the same order, so all of them derive the same scale
 // bit for bit and no separate launch is needed.  Returns 1 / scale; workgroup 0 publishes
 // the record.
+// The reduction itself: lane i brings the partial sums of workgroup i (and of i + THREADS, ...)
+// already added up as a (sum) and b (sum of squares).
 template <int THREADS>
-__device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
-                                                           int* hot_base = nullptr) {
+__device__ __forceinline__ float block_scale_reduce(double a, double b, Workspace* ws, int64_t n, prime_qparams* out, int* hot_base) {
     __shared__ double sh_s[THREADS / 64];
     __shared__ double sh_q[THREADS / 64];
     __shared__ float sh_inv;
     __shared__ int sh_hot;
-    constexpr int kIters = (kMaxGrid + THREADS - 1) / THREADS;
-    double ps[kIters], pq[kIters];
-#pragma unroll
-    for (int k = 0; k < kIters; ++k) {       // all loads in flight at once
-        const int i = threadIdx.x + k * THREADS;
-        ps[k] = i < nparts ? ws->part_sum[i] : 0.0;
-        pq[k] = i < nparts ? ws->part_sq[i] : 0.0;
-    }
-    double a = 0.0, b = 0.0;
-#pragma unroll
-    for (int k = 0; k < kIters; ++k) { a += ps[k]; b += pq[k]; }
     a = wave_sum(a);
     b = wave_sum(b);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -243,6 +233,23 @@ __device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int np
     return sh_inv;
 }
 
+template <int THREADS>
+__device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
+                                                           int* hot_base = nullptr) {
+    constexpr int kIters = (kMaxGrid + THREADS - 1) / THREADS;
+    double ps[kIters], pq[kIters];
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) {       // all loads in flight at once
+        const int i = threadIdx.x + k * THREADS;
+        ps[k] = i < nparts ? ws->part_sum[i] : 0.0;
+        pq[k] = i < nparts ? ws->part_sq[i] : 0.0;
+    }
+    double a = 0.0, b = 0.0;
+#pragma unroll
+    for (int k = 0; k < kIters; ++k) { a += ps[k]; b += pq[k]; }
+    return block_scale_reduce<THREADS>(a, b, ws, n, out, hot_base);
+}
+
 // Work distribution of the streaming kernels.  The tensor is cut into rows of kThreads
 // 16-byte vectors (16 KiB of floats per row at 1024 threads).  Main part: tiles of kUnroll
 // consecutive rows dealt round-robin to the G workgroups, so the whole grid sweeps the tensor
@@ -257,18 +264,23 @@ __device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int np
 // which a buffer window needs as its base, and with REVERSE walks the tensor from its end: a pass that
 // re-reads what the pass before it has just streamed then starts with the part the last-level
 // cache still holds instead of the part that has already been displaced.
+// sweep_tiles_of walks the share of workgroup `slot` of `G`; sweep_tiles and sweep walk the calling workgroup's own.
 template <int U = kUnroll, bool REVERSE = false, typename Body>
-__device__ __forceinline__ void sweep_tiles(int64_t nvec, Body&& body) {
-    const int64_t G = gridDim.x;
+__device__ __forceinline__ void sweep_tiles_of(int64_t nvec, int64_t slot, int64_t G, Body&& body) {
     const int64_t rows = (nvec + kThreads - 1) / kThreads;
     const int64_t rounds = (nvec / kThreads) / (G * U);
-    const int64_t r0 = rounds * G * U + blockIdx.x;
+    const int64_t r0 = rounds * G * U + slot;
     if (REVERSE && r0 < rows) body(r0 * kThreads, G * kThreads, std::false_type{});
     for (int64_t kk = 0; kk < rounds; ++kk) {
         const int64_t k = REVERSE ? rounds - 1 - kk : kk;
-        body(((k * G + blockIdx.x) * U) * kThreads, static_cast<int64_t>(kThreads), std::true_type{});
+        body(((k * G + slot) * U) * kThreads, static_cast<int64_t>(kThreads), std::true_type{});
     }
     if (!REVERSE && r0 < rows) body(r0 * kThreads, G * kThreads, std::false_type{});
+}
+
+template <int U = kUnroll, bool REVERSE = false, typename Body>
+__device__ __forceinline__ void sweep_tiles(int64_t nvec, Body&& body) {
+    sweep_tiles_of<U, REVERSE>(nvec, blockIdx.x, gridDim.x, body);
 }
 
 template <int U = kUnroll, typename Body>
@@ -427,25 +439,28 @@ __device__ __forceinline__ void rhist_flush(ResidualHist& h, int shift) {
     __syncthreads();
 }
 
-// The workgroup's partial (after a last flush): bin sums of x in fp64 and counts, 4 KiB contiguous.
-__device__ __forceinline__ void rhist_store(ResidualHist& h, int shift, float inv, Workspace* ws) {
-    rhist_flush(h, shift);
-    for (int b = threadIdx.x; b < kBins; b += kThreads) {
-        const unsigned long long cnt = h.wide_cnt[b];
-        unsigned long long far_n = 0;
-        double far_s = 0.0;
-        if (b == 0 || b == kBins - 1) {
-            const int side = b != 0;
+// Bin b of the workgroup's partial, after a last flush: the bin's sum of x in fp64 and its count.
+__device__ __forceinline__ BinAcc rhist_bin(const ResidualHist& h, float inv, int b) {
+    const unsigned long long cnt = h.wide_cnt[b];
+    unsigned long long far_n = 0;
+    double far_s = 0.0;
+    if (b == 0 || b == kBins - 1) {
+        const int side = b != 0;
 #pragma unroll
-            for (int c = 0; c < kFarCopies; ++c) { far_n += h.far_cnt[side][c]; far_s += h.far_sum[side][c]; }
-        }
-        const double centre = static_cast<double>(static_cast<long long>(cnt - far_n) * (b - kZeroPoint));
-        const double bins = centre + static_cast<double>(h.wide_sum[b]) * (1.0 / kResidualOne);
-        BinAcc acc;
-        acc.sum = bins / static_cast<double>(inv) + far_s;
-        acc.cnt = cnt;
-        ws->hist[blockIdx.x][b] = acc;
+        for (int c = 0; c < kFarCopies; ++c) { far_n += h.far_cnt[side][c]; far_s += h.far_sum[side][c]; }
     }
+    const double centre = static_cast<double>(static_cast<long long>(cnt - far_n) * (b - kZeroPoint));
+    const double bins = centre + static_cast<double>(h.wide_sum[b]) * (1.0 / kResidualOne);
+    BinAcc acc;
+    acc.sum = bins / static_cast<double>(inv) + far_s;
+    acc.cnt = cnt;
+    return acc;
+}
+
+// The workgroup's partial as workgroup `slot`, 4 KiB contiguous.
+__device__ __forceinline__ void rhist_store(ResidualHist& h, int shift, float inv, Workspace* ws, int slot) {
+    rhist_flush(h, shift);
+    for (int b = threadIdx.x; b < kBins; b += kThreads) ws->hist[slot][b] = rhist_bin(h, inv, b);
 }
 
 // Register-side accumulators for a tensor whose values crowd into a few codes (a constant, or
@@ -496,14 +511,18 @@ __device__ __forceinline__ void hist_flush_hot(LdsHist<R>& h, const HotCodes& ho
     }
 }
 
-// Store the workgroup's histogram (copies added in a fixed order) as its partial: one
-// 16-byte store per lane, 4 KiB contiguous per workgroup.
+// Bin b of the workgroup's histogram: its copies added in a fixed order.
 template <int R>
-__device__ __forceinline__ void hist_store(LdsHist<R>& h, Workspace* ws) {
-    for (int b = threadIdx.x; b < kBins; b += kThreads) {
-        BinAcc acc{0.0, 0ull};
+__device__ __forceinline__ BinAcc hist_bin(const LdsHist<R>& h, int b) {
+    BinAcc acc{0.0, 0ull};
 #pragma unroll
-        for (int r = 0; r < R; ++r) { acc.sum += h.sum[b * R + r]; acc.cnt += h.cnt[b * R + r]; }
-        ws->hist[blockIdx.x][b] = acc;
-    }
+    for (int r = 0; r < R; ++r) { acc.sum += h.sum[b * R + r]; acc.cnt += h.cnt[b * R + r]; }
+    return acc;
+}
+
+// Store the workgroup's histogram as the partial of workgroup `slot`: one 16-byte store per lane,
+// 4 KiB contiguous per workgroup.
+template <int R>
+__device__ __forceinline__ void hist_store(LdsHist<R>& h, Workspace* ws, int slot) {
+    for (int b = threadIdx.x; b < kBins; b += kThreads) ws->hist[slot][b] = hist_bin(h, b);
 }

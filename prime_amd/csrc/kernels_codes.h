@@ -278,5 +278,5 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float*
             q0 = fma(d, d, q0);
         }
     }
-    if (STATS) block_stats_store(s0 + s1, q0 + q1, ws);
+    if (STATS) block_stats_store(s0 + s1, q0 + q1, ws, blockIdx.x);
 }

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
         s0 += d;
         q0 = fma(d, d, q0);
     }
-    block_stats_store(s0 + s1, q0 + q1, ws);
+    block_stats_store(s0 + s1, q0 + q1, ws, blockIdx.x);
 }
 
 // One element of the outer optimizer, torch.optim.SGD(lr, momentum, nesterov=True) as the

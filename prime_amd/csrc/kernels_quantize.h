@@ -4,9 +4,9 @@
 //
 // Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
 
-// One (sum, count) pair for bin 0 as the workgroup's whole histogram partial: every lane brings the
-// fp64 sum and the number of the elements it saw.
-__device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, Workspace* ws) {
+// The workgroup's total of a per-lane fp64 sum and element count, in lane 0: lanes of a wavefront by
+// shuffles, then the wavefronts in order.  Two barriers; every lane calls it.
+__device__ __forceinline__ BinAcc block_sum_bin0(double s, unsigned long long c) {
     __shared__ double sh_s[kWaves];
     __shared__ unsigned long long sh_c[kWaves];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -15,12 +15,18 @@ __device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, 
     for (int off = 32; off > 0; off >>= 1) c += __shfl_down(c, off, 64);
     if (lane == 0) { sh_s[wave] = s; sh_c[wave] = c; }
     __syncthreads();
-    for (int b = threadIdx.x; b < kBins; b += kThreads) {
-        BinAcc acc{0.0, 0ull};
-        if (b == 0)
-            for (int w = 0; w < kWaves; ++w) { acc.sum += sh_s[w]; acc.cnt += sh_c[w]; }
-        ws->hist[blockIdx.x][b] = acc;
-    }
+    BinAcc acc{0.0, 0ull};
+    if (threadIdx.x == 0)
+        for (int w = 0; w < kWaves; ++w) { acc.sum += sh_s[w]; acc.cnt += sh_c[w]; }
+    __syncthreads();
+    return acc;
+}
+
+// One (sum, count) pair for bin 0 as the workgroup's whole histogram partial: every lane brings the
+// fp64 sum and the number of the elements it saw.
+__device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, Workspace* ws, int slot) {
+    const BinAcc total = block_sum_bin0(s, c);
+    for (int b = threadIdx.x; b < kBins; b += kThreads) ws->hist[slot][b] = b == 0 ? total : BinAcc{0.0, 0ull};
 }
 
 // K2 (+K3 when HIST): quantize to uint8, 4 codes packed per 32-bit store, and the 256-bin
@@ -31,10 +37,12 @@ __device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, 
 // 1 / scale is a finite non-zero number.  When 1 / scale is infinite or not a number (scale 0: an
 // all-zero tensor) every element has code 0 and the histogram is one sum; a zero 1 / scale (an
 // infinite scale: a single element) takes the fp64 histogram.
+// quantize_block is the pass itself for the calling workgroup's share of the tensor, given 1 / scale
+// (`narrow` is INT_MIN unless the statistics show a tensor crowded into a few codes), as workgroup
+// `slot` of a grid of G would run it.
 template <bool ALIGNED, bool NT, bool HIST, bool REVERSE, int POLICY>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
-                                                            int stats_parts, prime_qparams* qp_out, int zero_point,
-                                                            uint8_t* __restrict__ codes, Workspace* ws, int copies_shift) {
+__device__ __forceinline__ void quantize_block(const float* __restrict__ x, int64_t n, float inv, int narrow, int zero_point,
+                                               uint8_t* __restrict__ codes, Workspace* ws, int copies_shift, int slot, int G) {
     using M = Mem<ALIGNED, NT>;
     constexpr int kFpCopies = 8;
     union Hist {
@@ -43,12 +51,6 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
     };
     __shared__ std::conditional_t<HIST, Hist, int> hist_mem;      // no histogram memory without HIST
     Hist& hist = reinterpret_cast<Hist&>(hist_mem);
-    // the scale: given by value, or derived here from the statistics partials of the pass before
-    // (stats_parts < 0: the record a preceding kernel left in the workspace)
-    int narrow = INT_MIN;                // set when the statistics show a tensor crowded into a few codes
-    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &narrow)
-                      : stats_parts < 0 ? ws->qp.inv_scale
-                                        : 1.0f / scale_val;
     enum { kPlain, kFixed, kFp, kBin0 };
     const int mode = !HIST ? kPlain : !(__builtin_fabsf(inv) < __builtin_inff()) ? kBin0 : inv != 0.0f ? kFixed : kFp;
     const int shift = narrow != INT_MIN ? 3 : copies_shift;        // 8 = kMaxCopies
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
         constexpr int kMode = decltype(mode_t)::value;
         int since_flush = 0;
         const int flush_rounds = kMode == kFixed ? ResidualHist::flush_rounds(shift) : 0;
-        sweep_tiles<kUnroll, REVERSE>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+        sweep_tiles_of<kUnroll, REVERSE>(nvec, slot, G, [&](int64_t base, int64_t stride, auto full_t) {
             constexpr bool full = decltype(full_t)::value;
             const int64_t i0 = base + threadIdx.x;
             const Window out(codes + base * 4, (nvec - base) * 4);
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
                 since_flush = 0;
             }
         });
-        if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        if (slot == 0 && threadIdx.x < (n & 3)) {
             const int64_t i = (nvec << 2) + threadIdx.x;
             const float v = x[i];
             const int a = quantize_code(v, inv, zero_point);
@@ -135,14 +137,27 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
     else pass(std::integral_constant<int, kPlain>{});
     if (HIST) {
         if (mode == kFixed) {
-            rhist_store(hist.fixed, shift, inv, ws);
+            rhist_store(hist.fixed, shift, inv, ws, slot);
         } else if (mode == kFp) {
             __syncthreads();
-            hist_store(hist.fp, ws);
+            hist_store(hist.fp, ws, slot);
         } else {
-            hist_store_bin0(lane_sum, lane_cnt, ws);
+            hist_store_bin0(lane_sum, lane_cnt, ws, slot);
         }
     }
+}
+
+template <bool ALIGNED, bool NT, bool HIST, bool REVERSE, int POLICY>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
+                                                            int stats_parts, prime_qparams* qp_out, int zero_point,
+                                                            uint8_t* __restrict__ codes, Workspace* ws, int copies_shift) {
+    // the scale: given by value, or derived here from the statistics partials of the pass before
+    // (stats_parts < 0: the record a preceding kernel left in the workspace)
+    int narrow = INT_MIN;                // set when the statistics show a tensor crowded into a few codes
+    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &narrow)
+                      : stats_parts < 0 ? ws->qp.inv_scale
+                                        : 1.0f / scale_val;
+    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY>(x, n, inv, narrow, zero_point, codes, ws, copies_shift, blockIdx.x, gridDim.x);
 }
 
 // K3 alone: histogram of x under caller-supplied codes (average_buckets).  5 bytes per element.
@@ -183,7 +198,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const flo
         if (a < n_bins) hist_add(hist, a, x[i]);
     }
     __syncthreads();
-    hist_store(hist, ws);
+    hist_store(hist, ws, blockIdx.x);
 }
 
 // Second stage of the lookup build.  Workgroup j owns bins 4j .. 4j+3 (64 contiguous bytes

@@ -10,14 +10,16 @@ __global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace
     (void)block_scale_from_partials<kFinalThreads>(ws, nparts, n, out);
 }
 
-// K1: sum and sum of squares in fp64.  4 bytes per element.
+// The statistics partial of workgroup `slot` of a grid of G, computed by the calling workgroup and
+// stored in the workspace: fp64 sum and sum of squares of the rows that workgroup owns.
 template <bool ALIGNED, bool NT>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
+__device__ __forceinline__ void stats_partial(const float* __restrict__ x, int64_t n, int slot, int G, Workspace* ws) {
     using M = Mem<ALIGNED, NT>;
     const int64_t nvec = n >> 2;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep_tiles_of<kUnroll, false>(nvec, slot, G, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
+        const int64_t i0 = base + threadIdx.x;
         f4a v[kUnroll];
 #pragma unroll
         for (int j = 0; j < kUnroll; ++j) {
@@ -29,12 +31,18 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const fl
             if (j & 1) stats_add4(v[j], s1, q1); else stats_add4(v[j], s0, q0);
         }
     });
-    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    if (slot == 0 && threadIdx.x < (n & 3)) {
         const double v = x[(nvec << 2) + threadIdx.x];
         s0 += v;
         q0 = fma(v, v, q0);
     }
-    block_stats_store(s0 + s1, q0 + q1, ws);
+    block_stats_store(s0 + s1, q0 + q1, ws, slot);
+}
+
+// K1: sum and sum of squares in fp64.  4 bytes per element.
+template <bool ALIGNED, bool NT>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
+    stats_partial<ALIGNED, NT>(x, n, blockIdx.x, gridDim.x, ws);
 }
 
 // The norm as libtorch's CPU kernel accumulates it (the value compression.cpp:113 actually

@@ -30,6 +30,7 @@ namespace {
 #include "device_common.h"
 #include "kernels_statistics.h"
 #include "kernels_quantize.h"
+#include "kernels_small.h"
 #include "kernels_codes.h"
 #include "kernels_outer.h"
 
@@ -61,6 +62,7 @@ struct Options {
     int f32_store_policy = kStoreWriteThrough;          // fp32 outputs nobody reads back soon (dequantize, outer step)
     int f32_reread_store_policy = kStoreWriteThrough;   // fp32 outputs the next kernel reads back (ring step, first touch)
     int copy_store_policy = kStoreNt;                   // the plain copy (the byte counters' yardstick)
+    int64_t small_max_elems = int64_t(1) << 13;         // uniform_8bit_quantize takes one launch of one workgroup up to this many elements (0: never)
 };
 Options g_opt;
 
@@ -112,13 +114,13 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouch, kIdFirstTouchCodes, kIdCodeCount, kIdCodeTotal, kIdRequantPlan, kIdCodeRemap, kIdNormLiteral, kIdCount
+    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouch, kIdFirstTouchCodes, kIdCodeCount, kIdCodeTotal, kIdRequantPlan, kIdCodeRemap, kIdNormLiteral, kIdUniformSmall, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
     "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
     "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>", "div_kernel",
-    "first_touch_kernel", "first_touch_kernel<codes>", "code_count_kernel", "code_total_kernel", "requant_plan_kernel", "code_remap_kernel", "norm_literal_kernel"};
+    "first_touch_kernel", "first_touch_kernel<codes>", "code_count_kernel", "code_total_kernel", "requant_plan_kernel", "code_remap_kernel", "norm_literal_kernel", "uniform_small_kernel"};
 
 struct TimedLaunch {
     int id;
@@ -361,6 +363,9 @@ int prime_hip_set_option(const char* name, int value) {
         g_opt.large_read_min_elems = static_cast<int64_t>(value) << 20;
     } else if (!strcmp(name, "grid_cap")) {
         g_opt.grid_cap = value;
+    } else if (!strcmp(name, "small_max_elems")) {
+        if (value < 0) return fail(PRIME_EINVAL, "small_max_elems must be >= 0 (0: off)");
+        g_opt.small_max_elems = value;
     } else if (!strcmp(name, "reverse_second_pass")) {
         g_opt.reverse_second_pass = value != 0;
     } else if (!strcmp(name, "nt_load_min_mib")) {
@@ -384,6 +389,7 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "large_read_grid_eighths")) *value = g_opt.large_read_grid_eighths;
     else if (!strcmp(name, "large_read_min_mi_elems")) *value = static_cast<int>(g_opt.large_read_min_elems >> 20);
     else if (!strcmp(name, "grid_cap")) *value = g_opt.grid_cap;
+    else if (!strcmp(name, "small_max_elems")) *value = static_cast<int>(g_opt.small_max_elems);
     else if (!strcmp(name, "f32_store_policy")) *value = g_opt.f32_store_policy;
     else if (!strcmp(name, "f32_reread_store_policy")) *value = g_opt.f32_reread_store_policy;
     else if (!strcmp(name, "copy_store_policy")) *value = g_opt.copy_store_policy;
@@ -492,12 +498,31 @@ int prime_quantize_lookup_u8(const float* x, int64_t n, float scale, uint8_t* co
     return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
 }
 
-int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out, void* ws,
-                                prime_stream_t stream) {
-    if (bad_n(n) || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize: bad argument");
-    if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    Workspace* w = static_cast<Workspace*>(ws);
+}  // extern "C"
+
+namespace {
+
+// The single launch of one workgroup, when the tensor is small enough: at most small_max_elems
+// elements and a three-launch grid of one workgroup per row, at most kSmallSlots of them.
+bool small_applies(int64_t n) {
+    if (n <= 0 || n > g_opt.small_max_elems) return false;
+    const int64_t grid = grid_for(n, true);
+    const int64_t rows = (n / 4 + kThreads - 1) / kThreads;        // rows of whole vectors; the grid counts the ragged end too
+    return grid <= kSmallSlots && rows <= grid;
+}
+
+int run_uniform_small(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qp_out, Workspace* ws, hipStream_t st) {
+    const int rows = grid_for(n, true);
+    int shift = 0;
+    while ((1 << (shift + 1)) <= g_opt.hist_replicas) ++shift;
+    if (aligned_to(x, 16) && aligned_to(codes, 4))
+        launch(kIdUniformSmall, 9.0 * n, uniform_small_kernel<true>, 1, kThreads, st, x, n, rows, qp_out, codes, lut, ws, shift);
+    else
+        launch(kIdUniformSmall, 9.0 * n, uniform_small_kernel<false>, 1, kThreads, st, x, n, rows, qp_out, codes, lut, ws, shift);
+    return launch_check("uniform_small_kernel");
+}
+
+int uniform_three_launches(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out, Workspace* w, hipStream_t st) {
     if (n == 0) {
         if (int rc = run_stats(x, 0, qparams_out, w, st)) return rc;
         return run_lut_finalize(w, 0, lut, kBins, nullptr, st);
@@ -506,6 +531,25 @@ int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float
     if (int rc = run_stats_partials(x, n, w, st, &parts)) return rc;
     if (int rc = run_quantize(x, n, 0.0f, parts, qparams_out, kZeroPoint, codes, w, true, st, &grid, true)) return rc;
     return run_lut_finalize(w, grid, lut, kBins, nullptr, st);
+}
+
+int uniform_checked(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out, void* ws, prime_stream_t stream,
+                    bool may_take_one_launch = true) {
+    if (bad_n(n) || (n > 0 && (!x || !codes)) || !lut) return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize: bad argument");
+    if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Workspace* w = static_cast<Workspace*>(ws);
+    if (may_take_one_launch && small_applies(n)) return run_uniform_small(x, n, codes, lut, qparams_out, w, st);
+    return uniform_three_launches(x, n, codes, lut, qparams_out, w, st);
+}
+
+}  // namespace
+
+extern "C" {
+
+int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out, void* ws,
+                                prime_stream_t stream) {
+    return uniform_checked(x, n, codes, lut, qparams_out, ws, stream);
 }
 
 int prime_uniform_8bit_quantize_noalloc(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out,
@@ -548,8 +592,8 @@ int prime_uniform_8bit_quantize_buckets(const float* const* xs, const int64_t* n
         if (!workspaces[k]) return fail(PRIME_EWORKSPACE, "prime_uniform_8bit_quantize_buckets: a workspace is null");
     for (int64_t i = 0; i < count; ++i) {
         const int k = static_cast<int>(i % n_streams);
-        if (int rc = prime_uniform_8bit_quantize(xs[i], ns[i], codes[i], luts + i * kBins, qparams_out ? qparams_out + i : nullptr,
-                                                 workspaces[k], streams[k]))
+        if (int rc = uniform_checked(xs[i], ns[i], codes[i], luts + i * kBins, qparams_out ? qparams_out + i : nullptr,
+                                     workspaces[k], streams[k]))
             return rc;
     }
     return 0;

@@ -480,6 +480,67 @@ def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle,
         _lib.set_option(option, old)
 
 
+def _small_inputs(n, rng):
+    """What the kernel has a branch for: ordinary data, a tensor crowded into a few codes, all zeros
+    (every code 0), products beyond the fixed-point range, a not-a-number, a huge scale."""
+    normal = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    with np.errstate(over="ignore"):                              # the overflow to infinity is wanted
+        huge = (rng.standard_normal(n) * 3e38).astype(np.float32)
+    out = {"normal": normal, "near one": (1 + rng.standard_normal(n) * 1e-4).astype(np.float32),
+           "zeros": np.zeros(n, np.float32), "huge": huge, "large": np.full(n, 3e38, np.float32)}
+    if n >= 64:
+        far = normal.copy()
+        far[rng.integers(0, n, size=3)] = np.float32(40.0)       # about 4e4 standard deviations out
+        out["outliers"] = far
+        nan = normal.copy()
+        nan[n // 2] = np.nan
+        out["nan"] = nan
+    return out
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 1023, 4092, 4095, 4096, 4097, 4099, 8191, 8192, 8193, 12288, 12289, 16380, 16383, 16384])
+def test_one_launch_for_a_small_tensor_equals_the_three_launches_bit_for_bit(abi, n):
+    # small tensors take one launch of one workgroup that stands in for each workgroup of the
+    # three-launch grid in turn: codes, table and the whole statistics record must be those of the
+    # three launches bit for bit, at the sizes where the number of stand-ins changes, with and
+    # without a ragged end
+    rng = np.random.default_rng(n)
+    saved = _lib.get_option("small_max_elems")
+    assert saved == 1 << 13
+    try:
+        for label, x in _small_inputs(n, rng).items():
+            for shift in (0, 1) if n in (4097, 16383) else (0,):
+                buf = torch.zeros(n + 8, dtype=torch.float32, device=abi.dev)
+                xt = buf[shift:shift + n]
+                xt.copy_(torch.from_numpy(x))
+                _lib.set_option("small_max_elems", 0)
+                _lib.profile_begin()
+                want = abi.uniform(xt)
+                torch.cuda.synchronize()
+                assert "uniform_small_kernel" not in _lib.profile_end()
+                announce(f"one launch n={n} {label} shift={shift}")
+                _lib.set_option("small_max_elems", 1 << 14)      # the most the kernel is built for: four rows
+                for rep in range(2):
+                    _lib.profile_begin()
+                    got = abi.uniform(xt)
+                    torch.cuda.synchronize()
+                    assert list(_lib.profile_end()) == ["uniform_small_kernel"]
+                    assert torch.equal(got[0], want[0]), (label, rep)
+                    assert torch.equal(got[1].view(torch.int32), want[1].view(torch.int32)), (label, rep)
+                    assert torch.equal(got[2].view(torch.int64), want[2].view(torch.int64)), (label, rep)
+    finally:
+        _lib.set_option("small_max_elems", saved)
+
+
+def test_the_default_limit_of_the_one_launch_path(abi):
+    for n, small in ((1, True), (8192, True), (8193, False), (16384, False), (40000, False), (1 << 20, False)):
+        x = torch.randn(n, device=abi.dev)
+        _lib.profile_begin()
+        abi.uniform(x)
+        torch.cuda.synchronize()
+        assert ("uniform_small_kernel" in _lib.profile_end()) == small, n
+
+
 def test_results_do_not_depend_on_scheduling(abi):
     announce("determinism")
     x = torch.randn(3_000_001, device=abi.dev) * 1e-3
