@@ -86,6 +86,48 @@ def test_ring_reduce_step_2p26_chunks(abi):
         del want, acc
 
 
+def test_config2_all_22_layer_buckets(abi):
+    # benchmark configuration 2 in full: 22 per-layer buckets of 51,380,224 elements, Student-t(3) * 1e-4
+    # (heavy tails: the clip bins fill), quantized bucket by bucket; every bucket is checked on the
+    # device through what holds at any size: the scale formula on the fp64 norm, codes recomputed
+    # from that scale, bin populations, the table against fp64 bin means, the round trip
+    n, layers = 4 * 2048 * 2048 + 3 * 2048 * 5632, 22
+    g = torch.Generator(device=abi.dev).manual_seed(2)
+    for layer in range(layers):
+        # Student-t(3) = normal / sqrt(chi2(3) / 3)
+        z = torch.randn(n, device=abi.dev, generator=g)
+        chi = (torch.randn(3, n, device=abi.dev, generator=g) ** 2).sum(0)
+        x = (z / torch.sqrt(chi / 3.0) * 1e-4).float()
+        del z, chi
+        if layer % 4 == 0:
+            announce(f"cfg2 layer {layer}")
+        codes, lut, qp = abi.uniform(x)
+        q = abi.qparams(qp)
+        sumsq = float((x.double() ** 2).sum())
+        want = np.float32(6.0 * (float(np.float32(np.sqrt(sumsq))) / np.sqrt(n - 1)) / 256.0)
+        assert abs(float(q["scale"]) - float(want)) <= 1e-6 * float(want), layer
+        # codes from the scale the kernel derived: round half away from zero, +128, clamp (compression.cpp:23-24)
+        p = x * (torch.tensor(1.0, device=abi.dev) / torch.tensor(float(q["scale"]), device=abi.dev))
+        whole = torch.trunc(p)                                     # p - whole is exact: no p + 0.5 that could round up
+        rounded = whole + ((p - whole).abs() >= 0.5) * torch.sign(p)
+        ref_codes = (rounded + 128).clamp(0, 255).to(torch.uint8)
+        del whole, rounded
+        assert torch.equal(codes, ref_codes), (layer, int((codes != ref_codes).sum()))
+        cnt = torch.bincount(codes.int(), minlength=256)
+        assert int(cnt.sum()) == n
+        assert int(cnt[0]) > n // 1000 and int(cnt[255]) > n // 1000      # the tails clip
+        sums = torch.bincount(codes.int(), weights=x.double(), minlength=256)
+        mean = torch.where(cnt > 0, sums / cnt.clamp(min=1), torch.zeros_like(sums))
+        floor = torch.tensor(float(q["scale"]), device=abi.dev, dtype=torch.float64)
+        assert float(((lut.double() - mean).abs() / torch.maximum(mean.abs(), floor)).max()) <= 1e-6, layer
+        out = torch.empty_like(x)
+        abi.dequant(out, lut, codes, add=False)
+        assert torch.equal(out, lut[codes.long()]), layer
+        inside = (codes > 0) & (codes < 255)
+        assert float((out - x)[inside].abs().max()) <= float(q["scale"]), layer
+        del x, p, ref_codes, out, inside
+
+
 def test_config4_shard_all_42_buckets(abi):
     # benchmark configuration 4 in full: 1.25e9 elements (5 GB) as 42 buckets, the last 32 longer, N(0, 5e-4)
     # with 0.01 % of entries at +-50 sigma; quantize + lookup + dequantize per bucket, checked through
