@@ -427,6 +427,27 @@ def main() -> int:
                           "kernels": {k: {"avg_us": round(us, 2), "algo_GBps": round(b / us / 1e3, 1)} for k, (us, b) in per28.items()}}
             if name == "uniform_8bit_quantize (a1)":
                 uni_prof = per28
+        # What this device's memory delivers to the simplest kernels at the same size, for scale: reading
+        # only (the statistics pass above), a plain copy, writing only (torch's fill).  HBM moves reads and
+        # writes over one bus in turn, so a kernel that does both is bounded by the sum of the two times.
+        def event_timed(fn):
+            for r in range(args.warmup):
+                fn(r)
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+            for r, (a, b) in enumerate(evs):
+                a.record()
+                fn(r)
+                b.record()
+            torch.cuda.synchronize()
+            return sum(a.elapsed_time(b) for a, b in evs) / len(evs) * 1e3 - event_overhead_us
+        copy_us = event_timed(lambda r: _lib.check(lib.prime_copy_bytes(o28s[r % 3].data_ptr(), xs28[r % 3].data_ptr(), n28 * 4, st), "copy"))
+        fill_us = event_timed(lambda r: o28s[r % 3].fill_(1.0))
+        yard = {"read_only_stats_kernel": {"GBps": rows["stats (norm)"]["GBps"], "frac_of_hbm_peak": rows["stats (norm)"]["frac_of_hbm_peak"]}
+                if "stats (norm)" in rows else None,
+                "copy_kernel_1GiB_to_1GiB": {"us": round(copy_us, 2), "GBps": round(8 * n28 / copy_us / 1e3, 1),
+                                             "frac_of_hbm_peak": round(8 * n28 / copy_us / 1e3 / HBM_PEAK_GBS, 4)},
+                "write_only_torch_fill_1GiB": {"us": round(fill_us, 2), "GBps": round(4 * n28 / fill_us / 1e3, 1),
+                                               "frac_of_hbm_peak": round(4 * n28 / fill_us / 1e3 / HBM_PEAK_GBS, 4)}}
         dom_us, dom_bytes = uni_prof["quantize_kernel+hist"]
         uni, ring28 = rows["uniform_8bit_quantize (a1)"], rows.get("ring reduce step (a4 + a1)", {})
         out["tensor_2p28"] = {
@@ -438,6 +459,7 @@ def main() -> int:
             "ring_reduce_step": {"value": ring28["GBps"], "unit": "GB/s", "ms": round(ring28["us"] / 1e3, 4),
                                  "frac_of_hbm_peak": ring28["frac_of_hbm_peak"]} if ring28 else None,
             "operations": rows,
+            "memory_yardsticks": yard,
         }
         out["roofline"] = {
             "bound": "hbm",

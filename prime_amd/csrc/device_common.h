@@ -322,7 +322,7 @@ __device__ __forceinline__ void hist_add(LdsHist<R>& h, int code, float x) {
 // code c lies d = x * inv - (c - 128) bins from the centre of its bin (|d| <= 1/2 unless c is 0 or
 // 255, where the clipped elements collect); the bin's sum of x is ((c - 128) * count + sum of d) / inv.
 // d comes from one fused multiply-add (a single rounding of the exact x * inv - k) and is added as the
-// integer round(d * 2^22) + 2^31 in bits [47:0] of the slot, with 1 in bits [63:48]: count and sum
+// integer floor(d * 2^22 + 1/2) + 2^31 in bits [47:0] of the slot, with 1 in bits [63:48]: count and sum
 // in one atomic, integer sums that do not depend on the order of the additions.  Per element the
 // table carries an error below 2^-23 of a bin width.  Elements with |x * inv| > 628 (or not a number)
 // are beyond the range of the 32-bit residual: they count with residual 0 and their x goes to a pair of
@@ -357,10 +357,21 @@ __device__ __forceinline__ void rhist_zero(ResidualHist& h, int shift) {
     }
 }
 
-// round(d * 2^22) of the residual of x in the bin of `code`; meaningless (and replaced) for far elements
+// floor(v + 1/2) as an integer, in one instruction (computed exactly: no sum that could round).
+__device__ __forceinline__ int round_half_up(float v) {
+    int r;
+    asm("v_cvt_rpi_i32_f32 %0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+
+// The residual d of x from the centre `centre` (= code - 128, as a float) of its bin, in units of
+// 2^-22 bin: floor(d * 2^22 + 1/2), d from one fused multiply-add.  Meaningless (and replaced) for
+// far elements.
+__device__ __forceinline__ int residual_units(float x, float inv, float centre) {
+    return round_half_up(__builtin_fmaf(x, inv, -centre) * kResidualOne);
+}
 __device__ __forceinline__ int residual_fixed(float x, float inv, int code) {
-    const float d = __builtin_fmaf(x, inv, -static_cast<float>(code - kZeroPoint));
-    return static_cast<int>(__builtin_rintf(d * kResidualOne));
+    return residual_units(x, inv, static_cast<float>(code - kZeroPoint));
 }
 
 // `copy` = the lane's copy index, threadIdx.x & ((1 << shift) - 1)
@@ -389,32 +400,44 @@ __device__ __forceinline__ float round_centre(float q) {
 // The four elements of one vector in the fused pass: their packed codes (returned) and their
 // histogram entries (no barrier inside: lanes may skip it).  Products within kFarBins take the short
 // instruction sequence; a vector with a product beyond it, or not a number, takes the general one.
+// Short sequence, per element: the centre k of the bin as a float (round_centre), then k + 1.5 * 2^23
+// + 128 as a float, whose bit pattern is a constant plus the code: the low byte is the code for the
+// packed word, and the whole pattern shifted left addresses the slot (the constant is taken out of
+// the lane's base offset, modulo 2^32), so that the code never exists as an integer of its own.
 __device__ __forceinline__ uint32_t rhist_quantize4(ResidualHist& h, int shift, int copy, const f4a v, float inv) {
     const float qa = v.x * inv, qb = v.y * inv, qc = v.z * inv, qd = v.w * inv;
     const bool ra = !(__builtin_fabsf(qa) <= kFarBins), rb = !(__builtin_fabsf(qb) <= kFarBins),
                rc = !(__builtin_fabsf(qc) <= kFarBins), rd = !(__builtin_fabsf(qd) <= kFarBins);
-    int a, b, c, d, fa, fb, fc, fd;
     if (!(ra | rb | rc | rd)) {
+        constexpr float kMagic = 12582912.0f + kZeroPoint;            // 1.5 * 2^23 + 128: bits 0x4B400080 + (code - 128)
+        constexpr uint32_t kMagicBits = 0x4B400000u;
         const float ka = round_centre(qa), kb = round_centre(qb), kc = round_centre(qc), kd = round_centre(qd);
-        a = static_cast<int>(ka) + kZeroPoint;
-        b = static_cast<int>(kb) + kZeroPoint;
-        c = static_cast<int>(kc) + kZeroPoint;
-        d = static_cast<int>(kd) + kZeroPoint;
-        fa = static_cast<int>(__builtin_rintf(__builtin_fmaf(v.x, inv, -ka) * kResidualOne));
-        fb = static_cast<int>(__builtin_rintf(__builtin_fmaf(v.y, inv, -kb) * kResidualOne));
-        fc = static_cast<int>(__builtin_rintf(__builtin_fmaf(v.z, inv, -kc) * kResidualOne));
-        fd = static_cast<int>(__builtin_rintf(__builtin_fmaf(v.w, inv, -kd) * kResidualOne));
-    } else {
-        a = quantize_code(v.x, inv, kZeroPoint);
-        b = quantize_code(v.y, inv, kZeroPoint);
-        c = quantize_code(v.z, inv, kZeroPoint);
-        d = quantize_code(v.w, inv, kZeroPoint);
-        fa = fb = fc = fd = 0;
-        if (ra) rhist_add_far(h, a, v.x); else fa = residual_fixed(v.x, inv, a);
-        if (rb) rhist_add_far(h, b, v.y); else fb = residual_fixed(v.y, inv, b);
-        if (rc) rhist_add_far(h, c, v.z); else fc = residual_fixed(v.z, inv, c);
-        if (rd) rhist_add_far(h, d, v.w); else fd = residual_fixed(v.w, inv, d);
+        const uint32_t ua = __float_as_uint(ka + kMagic), ub = __float_as_uint(kb + kMagic),
+                       uc = __float_as_uint(kc + kMagic), ud = __float_as_uint(kd + kMagic);      // kMagicBits + code
+        const int s3 = shift + 3;                                     // a slot is 8 bytes
+        uint32_t base = (static_cast<uint32_t>(copy) << 3) - (kMagicBits << s3);
+        asm("" : "+v"(base));             // opaque: keeps the constant out of every element's address arithmetic
+        char* slots = reinterpret_cast<char*>(h.slot);
+        auto add = [&](uint32_t u, int units) {
+            const unsigned long long val = (1ull << 48) | static_cast<unsigned long long>(static_cast<unsigned>(units) ^ 0x80000000u);
+            __hip_atomic_fetch_add(reinterpret_cast<unsigned long long*>(slots + ((u << s3) + base)), val, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+        };
+        add(ua, residual_units(v.x, inv, ka));
+        add(ub, residual_units(v.y, inv, kb));
+        add(uc, residual_units(v.z, inv, kc));
+        add(ud, residual_units(v.w, inv, kd));
+        const uint32_t lo = __builtin_amdgcn_perm(ub, ua, 0x0c0c0400u);   // code a | code b << 8
+        const uint32_t hi = __builtin_amdgcn_perm(ud, uc, 0x0c0c0400u);
+        return lo | (hi << 16);
     }
+    const int a = quantize_code(v.x, inv, kZeroPoint), b = quantize_code(v.y, inv, kZeroPoint),
+              c = quantize_code(v.z, inv, kZeroPoint), d = quantize_code(v.w, inv, kZeroPoint);
+    int fa = 0, fb = 0, fc = 0, fd = 0;
+    if (ra) rhist_add_far(h, a, v.x); else fa = residual_fixed(v.x, inv, a);
+    if (rb) rhist_add_far(h, b, v.y); else fb = residual_fixed(v.y, inv, b);
+    if (rc) rhist_add_far(h, c, v.z); else fc = residual_fixed(v.z, inv, c);
+    if (rd) rhist_add_far(h, d, v.w); else fd = residual_fixed(v.w, inv, d);
     rhist_add(h, shift, copy, a, fa);
     rhist_add(h, shift, copy, b, fb);
     rhist_add(h, shift, copy, c, fc);
