@@ -223,18 +223,22 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_remap_kernel(con
 // is divided by `divisor` before it is stored and counted: chunk.div_(world_size) of
 // ReduceOp::AVG (collectives.cpp:155-159) folded into the last accumulation of a chunk.
 // POLICY is the cache policy of the fp32 stores.
-template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut,
-                                                           const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
-                                                           float divisor) {
+// ONESHOT (never with STATS, whose partials are per workgroup of a small grid): one workgroup of
+// kShotThreads lanes per tile instead of a loop.
+template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT = false>
+__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd)
+void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
+                    float divisor) {
+    static_assert(!(ONESHOT && STATS), "statistics partials need the small grid of the looping sweep");
     using M = Mem<ALIGNED, NT>;
+    constexpr int T = ONESHOT ? kShotThreads : kThreads;
     __shared__ float s_lut[kBins];
-    for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
+    for (int b = threadIdx.x; b < kBins; b += T) s_lut[b] = lut[b];
     __syncthreads();
     const int64_t nvec = n >> 2;
-    constexpr int U = DIV ? kDivUnroll : kUnroll;
+    constexpr int U = ONESHOT ? kShotUnroll : DIV ? kDivUnroll : kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    sweep_tiles<U>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+    walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         const Window win(out + base * 4, (nvec - base) * 16);

@@ -10,12 +10,13 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
 }
 
 // chunk /= world_size for ReduceOp::AVG (collectives.cpp:155-159): an fp32 division in place.
-template <bool ALIGNED, int POLICY>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void div_kernel(float* __restrict__ x, int64_t n, float d) {
+template <bool ALIGNED, int POLICY, bool ONESHOT = false>
+__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void div_kernel(float* __restrict__ x, int64_t n, float d) {
     using M = Mem<ALIGNED, false>;
     const int64_t nvec = n >> 2;
-    constexpr int U = kDivUnroll;
-    sweep_tiles<U>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+    constexpr int T = ONESHOT ? kShotThreads : kThreads;
+    constexpr int U = ONESHOT ? kShotUnroll : kDivUnroll;
+    walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         const Window win(x + base * 4, (nvec - base) * 16);
@@ -44,14 +45,14 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void div_kernel(float* __r
 // (src/zeroband/diloco.py:93-101): grad = outer_param - inner_param, then the whole flat buffer
 // divided by the world size; an fp32 subtraction and an fp32 division per element.
 // 12 bytes per element.
-template <bool ALIGNED, bool NT, int POLICY>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer,
-                                                                                   const float* __restrict__ inner, int64_t n,
-                                                                                   float world_size, float* __restrict__ out) {
+template <bool ALIGNED, bool NT, int POLICY, bool ONESHOT = false>
+__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer, const float* __restrict__ inner, int64_t n,
+                                            float world_size, float* __restrict__ out) {
     using M = Mem<ALIGNED, NT>;
     const int64_t nvec = n >> 2;
-    constexpr int U = kDivUnroll;
-    sweep_tiles<U>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+    constexpr int T = ONESHOT ? kShotThreads : kThreads;
+    constexpr int U = ONESHOT ? kShotUnroll : kDivUnroll;
+    walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         const Window win(out + base * 4, (nvec - base) * 16);
@@ -167,28 +168,27 @@ __device__ __forceinline__ void outer_sgd_one(float& p, float& buf, float g, flo
 // the inner model (sync_inner_model, :137-144) in the same pass.  The gradient is fp32
 // (24 bytes per element) or, with CODES, uint8 codes and their lookup table (21 bytes per
 // element, and the dequantize pass is saved).
-template <bool CODES, bool ALIGNED, bool NT, int POLICY>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom,
-                                                                              const float* __restrict__ grad,
-                                                                              const uint8_t* __restrict__ codes,
-                                                                              const float* __restrict__ lut,
-                                                                              float* __restrict__ inner, int64_t n, float neg_lr,
-                                                                              float mu, int first) {
+template <bool CODES, bool ALIGNED, bool NT, int POLICY, bool ONESHOT = false>
+__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom, const float* __restrict__ grad,
+                                       const uint8_t* __restrict__ codes, const float* __restrict__ lut, float* __restrict__ inner,
+                                       int64_t n, float neg_lr, float mu, int first) {
     using M = Mem<ALIGNED, NT>;
+    constexpr int T = ONESHOT ? kShotThreads : kThreads;
+    constexpr int U = ONESHOT ? kShotUnroll : kUnroll;
     __shared__ float s_lut[kBins];
     if (CODES) {
-        for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
+        for (int b = threadIdx.x; b < kBins; b += T) s_lut[b] = lut[b];
         __syncthreads();
     }
     const int64_t nvec = n >> 2;
-    sweep_tiles(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+    walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         const Window wp(param + base * 4, (nvec - base) * 16), wm(mom + base * 4, (nvec - base) * 16),
             wi(inner ? inner + base * 4 : nullptr, inner ? (nvec - base) * 16 : 0);
-        f4a p[kUnroll], m[kUnroll], g[kUnroll];
+        f4a p[U], m[U], g[U];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             const bool ok = full || i < nvec;
             p[j] = ok ? M::ldf4(param, i) : f4a{0.f, 0.f, 0.f, 0.f};
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void outer_step_kernel(flo
             }
         }
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             if (full || i < nvec) {
 #pragma unroll
@@ -236,21 +236,23 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void outer_step_kernel(flo
     }
 }
 
-template <int POLICY>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
+template <int POLICY, bool ONESHOT = false>
+__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
     using M = Mem<true, true>;
-    sweep_tiles(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+    constexpr int T = ONESHOT ? kShotThreads : kThreads;
+    constexpr int U = ONESHOT ? kShotUnroll : kUnroll;
+    walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         const Window win(dst + base, (nvec - base) * 16);
-        f4a v[kUnroll];
+        f4a v[U];
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             if (full || i < nvec) v[j] = M::ldf4(reinterpret_cast<const float*>(src), i);
         }
 #pragma unroll
-        for (int j = 0; j < kUnroll; ++j) {
+        for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             if (full || i < nvec) win.template st128<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 16u, v[j]);
         }

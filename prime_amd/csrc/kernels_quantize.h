@@ -160,6 +160,40 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
     quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY>(x, n, inv, narrow, zero_point, codes, ws, copies_shift, blockIdx.x, gridDim.x);
 }
 
+// K2 with the scale given and no histogram (quantize_per_tensor_uint8, compression.cpp:9-43), one
+// workgroup per tile: a pass that keeps nothing between tiles does not need the loop.
+template <int POLICY>
+__global__ __launch_bounds__(kShotThreads, 8) void quantize_shot_kernel(const float* __restrict__ x, int64_t n, float scale_val, int zero_point,
+                                                                    uint8_t* __restrict__ codes) {
+    using M = Mem<true, true>;
+    const float inv = 1.0f / scale_val;
+    const int64_t nvec = n >> 2;
+    walk_tiles<kShotThreads, kShotUnroll, true>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+        constexpr bool full = decltype(full_t)::value;
+        const int64_t i0 = base + threadIdx.x;
+        const Window out(codes + base * 4, (nvec - base) * 4);
+        f4a v[kShotUnroll];
+#pragma unroll
+        for (int j = 0; j < kShotUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < kShotUnroll; ++j) {
+            const int64_t i = i0 + j * stride;
+            if (full || i < nvec) {
+                const uint32_t a = quantize_code(v[j].x, inv, zero_point), b = quantize_code(v[j].y, inv, zero_point),
+                               c = quantize_code(v[j].z, inv, zero_point), d = quantize_code(v[j].w, inv, zero_point);
+                out.template st32<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 4u, a | (b << 8) | (c << 16) | (d << 24));
+            }
+        }
+    });
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        codes[i] = static_cast<uint8_t>(quantize_code(x[i], inv, zero_point));
+    }
+}
+
 // K3 alone: histogram of x under caller-supplied codes (average_buckets).  5 bytes per element.
 template <bool ALIGNED, int R>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const float* __restrict__ x, const uint8_t* __restrict__ codes,

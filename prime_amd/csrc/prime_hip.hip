@@ -62,6 +62,9 @@ struct Options {
     int f32_store_policy = kStoreWriteThrough;          // fp32 outputs nobody reads back soon (dequantize, outer step)
     int f32_reread_store_policy = kStoreWriteThrough;   // fp32 outputs the next kernel reads back (ring step, first touch)
     int copy_store_policy = kStoreNt;                   // the plain copy (the byte counters' yardstick)
+    int one_shot = 1;                                   // kernels that keep nothing between tiles: one workgroup per tile instead of a loop
+    int64_t one_shot_min_elems = int64_t(1) << 16;      // ... from this many elements up
+    int one_shot_store_policy = kStoreNt;               // cache policy of their fp32 stores
     int64_t small_max_elems = int64_t(1) << 13;         // uniform_8bit_quantize takes one launch of one workgroup up to this many elements (0: never)
 };
 Options g_opt;
@@ -99,6 +102,13 @@ int grid_for(int64_t n, bool reads = false) {
     if (g_opt.grid_cap > 0 && cap > g_opt.grid_cap) cap = g_opt.grid_cap;
     return static_cast<int>(tiles < cap ? tiles : cap);
 }
+
+// One workgroup per tile for a kernel launched ONESHOT.
+int shot_grid(int64_t nvec) {
+    const int64_t tile = static_cast<int64_t>(kShotThreads) * kShotUnroll;
+    return static_cast<int>((nvec + tile - 1) / tile);
+}
+inline bool one_shot(int64_t n) { return g_opt.one_shot && n >= g_opt.one_shot_min_elems; }
 
 inline bool use_nt(int64_t n) { return (n >> 18) >= g_opt.nt_load_min_mib; }   // n floats = n / 2^18 MiB
 
@@ -227,6 +237,13 @@ int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_
     if (hist && zp != kZeroPoint) return fail(PRIME_EINVAL, "the fused quantize + lookup pass has zero point 128");
     const int grid = grid_for(n, true);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
+    if (!hist && stats_parts == 0 && al && one_shot(n)) {
+        with_policy(g_opt.code_store_policy, [&](auto P) {
+            launch(kIdQuantize, 5.0 * n, quantize_shot_kernel<decltype(P)::value>, shot_grid(n >> 2), kShotThreads, st, x, n, scale, zp, codes);
+        });
+        if (grid_out) *grid_out = 0;
+        return launch_check("quantize_shot_kernel");
+    }
     const bool rev = second_pass && g_opt.reverse_second_pass;
     if (!hist) launch_quantize_r<false>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     else launch_quantize_r<true>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
@@ -247,9 +264,21 @@ int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins
 template <bool ADD, bool STATS, bool DIV, int POLICY>
 void launch_dequant(int id, double bytes, int grid, hipStream_t st, float* out, const float* lut, const uint8_t* codes, int64_t n,
                     Workspace* ws, float divisor) {
-    if (!(aligned_to(out, 16) && aligned_to(codes, 4)))
+    if (!(aligned_to(out, 16) && aligned_to(codes, 4))) {
         launch(id, bytes, dequant_kernel<ADD, STATS, false, false, DIV, kStorePlain>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
-    else if (use_nt(n))
+        return;
+    }
+    if constexpr (!STATS) {
+        if (one_shot(n)) {
+            // accumulating in place is the one case that does better with write-through stores (380 against 388 us at 2^28)
+            with_policy(ADD ? g_opt.f32_store_policy : g_opt.one_shot_store_policy, [&](auto P) {
+                launch(id, bytes, dequant_kernel<ADD, false, true, true, DIV, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, out, lut,
+                       codes, n, ws, divisor);
+            });
+            return;
+        }
+    }
+    if (use_nt(n))
         launch(id, bytes, dequant_kernel<ADD, STATS, true, true, DIV, POLICY>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
     else
         launch(id, bytes, dequant_kernel<ADD, STATS, true, false, DIV, POLICY>, grid, kThreads, st, out, lut, codes, n, ws, divisor);
@@ -264,9 +293,9 @@ int run_dequant(float* out, const float* lut, const uint8_t* codes, int64_t n, W
     const int id = STATS ? (ADD ? kIdDequantAddStats : kIdDequantSetStats) : (ADD ? kIdDequantAdd : kIdDequantSet);
     const double bytes = (ADD ? 9.0 : 5.0) * n;
     const int pol = STATS ? g_opt.f32_reread_store_policy : g_opt.f32_store_policy;
-    if (pol == kStoreNt) launch_dequant<ADD, STATS, DIV, kStoreNt>(id, bytes, grid, st, out, lut, codes, n, ws, divisor);
-    else if (pol == kStoreWriteThrough) launch_dequant<ADD, STATS, DIV, kStoreWriteThrough>(id, bytes, grid, st, out, lut, codes, n, ws, divisor);
-    else launch_dequant<ADD, STATS, DIV, kStorePlain>(id, bytes, grid, st, out, lut, codes, n, ws, divisor);
+    with_policy(pol, [&](auto policy) {
+        launch_dequant<ADD, STATS, DIV, decltype(policy)::value>(id, bytes, grid, st, out, lut, codes, n, ws, divisor);
+    });
     if (grid_out) *grid_out = grid;
     return launch_check("dequant_kernel");
 }
@@ -363,6 +392,12 @@ int prime_hip_set_option(const char* name, int value) {
         g_opt.large_read_min_elems = static_cast<int64_t>(value) << 20;
     } else if (!strcmp(name, "grid_cap")) {
         g_opt.grid_cap = value;
+    } else if (!strcmp(name, "one_shot")) {
+        g_opt.one_shot = value != 0;
+    } else if (!strcmp(name, "one_shot_store_policy")) {
+        if (value != kStorePlain && value != kStoreNt && value != kStoreWriteThrough)
+            return fail(PRIME_EINVAL, "a store policy must be 0 (plain), 2 (non-temporal) or 16 (write-through)");
+        g_opt.one_shot_store_policy = value;
     } else if (!strcmp(name, "small_max_elems")) {
         if (value < 0) return fail(PRIME_EINVAL, "small_max_elems must be >= 0 (0: off)");
         g_opt.small_max_elems = value;
@@ -389,6 +424,8 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "large_read_grid_eighths")) *value = g_opt.large_read_grid_eighths;
     else if (!strcmp(name, "large_read_min_mi_elems")) *value = static_cast<int>(g_opt.large_read_min_elems >> 20);
     else if (!strcmp(name, "grid_cap")) *value = g_opt.grid_cap;
+    else if (!strcmp(name, "one_shot")) *value = g_opt.one_shot;
+    else if (!strcmp(name, "one_shot_store_policy")) *value = g_opt.one_shot_store_policy;
     else if (!strcmp(name, "small_max_elems")) *value = static_cast<int>(g_opt.small_max_elems);
     else if (!strcmp(name, "f32_store_policy")) *value = g_opt.f32_store_policy;
     else if (!strcmp(name, "f32_reread_store_policy")) *value = g_opt.f32_reread_store_policy;
@@ -694,7 +731,11 @@ int prime_div_f32(float* x, int64_t n, float divisor, prime_stream_t stream) {
     if (bad_n(n) || (n > 0 && !x)) return fail(PRIME_EINVAL, "prime_div_f32: bad argument");
     if (n == 0) return 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (aligned_to(x, 16))
+    if (aligned_to(x, 16) && one_shot(n))
+        with_policy(g_opt.one_shot_store_policy, [&](auto P) {
+            launch(kIdDiv, 8.0 * n, div_kernel<true, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, x, n, divisor);
+        });
+    else if (aligned_to(x, 16))
         with_policy(g_opt.f32_store_policy, [&](auto P) {
             launch(kIdDiv, 8.0 * n, div_kernel<true, decltype(P)::value>, grid_for(n), kThreads, st, x, n, divisor);
         });
@@ -709,7 +750,13 @@ int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n,
     if (n == 0) return 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int grid = grid_for(n);
-    if (aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(out, 16))
+    const bool pg_aligned = aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(out, 16);
+    if (pg_aligned && one_shot(n))
+        with_policy(g_opt.one_shot_store_policy, [&](auto P) {
+            launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<true, true, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, outer,
+                   inner, n, world_size, out);
+        });
+    else if (pg_aligned)
         with_policy(g_opt.f32_store_policy, [&](auto P) {
             if (use_nt(n))
                 launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<true, true, decltype(P)::value>, grid, kThreads, st, outer, inner, n, world_size, out);
@@ -783,7 +830,12 @@ int prime_outer_sgd_nesterov_f32(float* param, float* momentum_buf, const float*
     const double bytes = (inner_out ? 24.0 : 20.0) * n;
     const uint8_t* no_codes = nullptr;
     const float* no_lut = nullptr;
-    if (al)
+    if (al && one_shot(n))
+        with_policy(g_opt.one_shot_store_policy, [&](auto P) {
+            launch(kIdOuterStep, bytes, outer_step_kernel<false, true, true, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, param,
+                   momentum_buf, grad, no_codes, no_lut, inner_out, n, -lr, momentum, first_step);
+        });
+    else if (al)
         with_policy(g_opt.f32_store_policy, [&](auto P) {
             if (use_nt(n))
                 launch(kIdOuterStep, bytes, outer_step_kernel<false, true, true, decltype(P)::value>, grid, kThreads, st, param, momentum_buf,
@@ -808,7 +860,12 @@ int prime_outer_sgd_nesterov_u8(float* param, float* momentum_buf, const uint8_t
     const bool al = aligned_to(param, 16) && aligned_to(momentum_buf, 16) && aligned_to(codes, 4) && aligned_to(inner_out, 16);
     const double bytes = (inner_out ? 21.0 : 17.0) * n;
     const float* no_grad = nullptr;
-    if (al)
+    if (al && one_shot(n))
+        with_policy(g_opt.one_shot_store_policy, [&](auto P) {
+            launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, true, true, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, param,
+                   momentum_buf, no_grad, codes, lut, inner_out, n, -lr, momentum, first_step);
+        });
+    else if (al)
         with_policy(g_opt.f32_store_policy, [&](auto P) {
             if (use_nt(n))
                 launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, true, true, decltype(P)::value>, grid, kThreads, st, param,
@@ -831,8 +888,12 @@ int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t
     const int64_t nvec = n_bytes >> 4;
     const int grid = grid_for(nvec * 4);
     with_policy(g_opt.copy_store_policy, [&](auto P) {
-        launch(kIdCopy, 2.0 * n_bytes, copy_kernel<decltype(P)::value>, grid, kThreads, static_cast<hipStream_t>(stream),
-               static_cast<f4a*>(dst), static_cast<const f4a*>(src), nvec);
+        if (one_shot(nvec * 4))
+            launch(kIdCopy, 2.0 * n_bytes, copy_kernel<decltype(P)::value, true>, shot_grid(nvec), kShotThreads, static_cast<hipStream_t>(stream),
+                   static_cast<f4a*>(dst), static_cast<const f4a*>(src), nvec);
+        else
+            launch(kIdCopy, 2.0 * n_bytes, copy_kernel<decltype(P)::value>, grid, kThreads, static_cast<hipStream_t>(stream),
+                   static_cast<f4a*>(dst), static_cast<const f4a*>(src), nvec);
     });
     return launch_check("copy_kernel");
 }

@@ -453,7 +453,8 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
 @pytest.mark.parametrize("option,values", [("hist_replicas", (1, 2, 4, 8)), ("blocks_per_cu", (1, 2, 3, 4)),
                                            ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20)),
                                            ("code_store_policy", (0, 2, 16)), ("f32_reread_store_policy", (0, 2, 16)),
-                                           ("reverse_second_pass", (0, 1))])
+                                           ("reverse_second_pass", (0, 1)), ("one_shot", (0, 1)),
+                                           ("one_shot_store_policy", (0, 2, 16))])
 def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle, option, values):
     # the options change scheduling and cache hints only: codes, scale and lookup must not move,
     # on ordinary data, on a tensor crowded into a few codes, and through a ring step
@@ -539,6 +540,87 @@ def test_the_default_limit_of_the_one_launch_path(abi):
         abi.uniform(x)
         torch.cuda.synchronize()
         assert ("uniform_small_kernel" in _lib.profile_end()) == small, n
+
+
+@pytest.mark.parametrize("n", [65536, 65537, 700_001, (1 << 21) + 511, (1 << 21) + 513])
+def test_one_workgroup_per_tile_equals_the_looping_launch(abi, oracle, n):
+    # the kernels that keep nothing from tile to tile run as one 256-lane workgroup per tile from
+    # 65536 elements up; their results must be those of the looping launch bit for bit, and the
+    # oracle's, at sizes that end inside a tile, on a tile boundary and one vector past it
+    import ctypes
+
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    y = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    codes_np = rng.integers(0, 256, n, dtype=np.uint8)
+    lut_np = np.sort(rng.standard_normal(256).astype(np.float32)) * 1e-2
+    lib, st = abi.lib, abi.st
+    xt, yt, ct, lt = abi.to_dev(x), abi.to_dev(y), abi.to_dev(codes_np), abi.to_dev(lut_np)
+
+    def run_all():
+        out = {}
+        q = abi.quantize(xt, 3.1e-5)
+        out["quantize"] = q
+        d = torch.empty(n, device=abi.dev)
+        abi.dequant(d, lt, ct, add=False)
+        out["set"] = d
+        a = xt.clone()
+        abi.dequant(a, lt, ct, add=True)
+        out["add"] = a
+        v = xt.clone()
+        _lib.check(lib.prime_div_f32(v.data_ptr(), n, ctypes.c_float(7.0), st), "div")
+        out["div"] = v
+        pg = torch.empty(n, device=abi.dev)
+        _lib.check(lib.prime_pseudo_gradient_f32(xt.data_ptr(), yt.data_ptr(), n, ctypes.c_float(8.0), pg.data_ptr(), st), "pg")
+        out["pseudo gradient"] = pg
+        for name, first in (("outer step, first", 1), ("outer step", 0)):
+            p, m, inner = xt.clone(), yt.clone(), torch.empty(n, device=abi.dev)
+            _lib.check(lib.prime_outer_sgd_nesterov_f32(p.data_ptr(), m.data_ptr(), pg.data_ptr(), inner.data_ptr(), n, ctypes.c_float(0.7),
+                                                        ctypes.c_float(0.9), first, st), name)
+            out[name] = torch.stack([p, m, inner])
+            p, m, inner = xt.clone(), yt.clone(), torch.empty(n, device=abi.dev)
+            _lib.check(lib.prime_outer_sgd_nesterov_u8(p.data_ptr(), m.data_ptr(), ct.data_ptr(), lt.data_ptr(), inner.data_ptr(), n,
+                                                       ctypes.c_float(0.7), ctypes.c_float(0.9), first, st), name)
+            out[name + ", codes"] = torch.stack([p, m, inner])
+        if n % 4 == 0:
+            c = torch.empty(n, device=abi.dev)
+            _lib.check(lib.prime_copy_bytes(c.data_ptr(), xt.data_ptr(), 4 * n, st), "copy")
+            out["copy"] = c
+        torch.cuda.synchronize()
+        return out
+
+    saved = _lib.get_option("one_shot")
+    try:
+        announce(f"one workgroup per tile n={n}")
+        _lib.set_option("one_shot", 1)
+        _lib.profile_begin()
+        shot = run_all()
+        prof = _lib.profile_end()
+        _lib.set_option("one_shot", 0)
+        loop = run_all()
+    finally:
+        _lib.set_option("one_shot", saved)
+    assert set(prof) >= {"quantize_kernel", "dequant_kernel<set>", "dequant_kernel<add>", "div_kernel", "pseudo_gradient_kernel", "outer_step_kernel"}
+    for name in shot:
+        assert torch.equal(shot[name].view(torch.int32) if shot[name].dtype == torch.float32 else shot[name],
+                           loop[name].view(torch.int32) if loop[name].dtype == torch.float32 else loop[name]), name
+    oc = oracle.quantize_per_tensor_uint8(x, np.float32(3.1e-5), 128)
+    assert np.array_equal(shot["quantize"].cpu().numpy(), oc)
+    assert np.array_equal(shot["set"].cpu().numpy(), lut_np[codes_np])
+    want = x.copy()
+    oracle.index_add(want, lut_np, codes_np)
+    assert np.array_equal(shot["add"].cpu().numpy(), want)
+    assert np.array_equal(shot["div"].cpu().numpy(), x / np.float32(7.0))
+    assert np.array_equal(shot["pseudo gradient"].cpu().numpy(), oracle.pseudo_gradient(x, y, 8.0))
+    for first, name in ((True, "outer step, first"), (False, "outer step")):
+        p, m = x.copy(), y.copy()
+        oracle.outer_sgd_nesterov(p, m, oracle.pseudo_gradient(x, y, 8.0), 0.7, 0.9, first)
+        got = shot[name].cpu().numpy()
+        assert np.array_equal(got[0], p) and np.array_equal(got[1], m) and np.array_equal(got[2], p), name
+        p, m = x.copy(), y.copy()
+        oracle.outer_sgd_nesterov(p, m, lut_np[codes_np], 0.7, 0.9, first)
+        got = shot[name + ", codes"].cpu().numpy()
+        assert np.array_equal(got[0], p) and np.array_equal(got[1], m) and np.array_equal(got[2], p), name
 
 
 def test_results_do_not_depend_on_scheduling(abi):
