@@ -40,17 +40,18 @@ __device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, 
 // quantize_block is the pass itself for the calling workgroup's share of the tensor, given 1 / scale
 // (`narrow` is INT_MIN unless the statistics show a tensor crowded into a few codes), as workgroup
 // `slot` of a grid of G would run it.
+// The workgroup's histogram memory: the fixed-point histogram or, for a zero 1 / scale, the fp64 one.
+constexpr int kFpCopies = 8;
+union QuantHist {
+    ResidualHist fixed;
+    LdsHist<kFpCopies> fp;
+};
+
 template <bool ALIGNED, bool NT, bool HIST, bool REVERSE, int POLICY>
 __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int64_t n, float inv, int narrow, int zero_point,
-                                               uint8_t* __restrict__ codes, Workspace* ws, int copies_shift, int slot, int G) {
+                                               uint8_t* __restrict__ codes, Workspace* ws, int copies_shift, int slot, int G,
+                                               QuantHist& hist) {
     using M = Mem<ALIGNED, NT>;
-    constexpr int kFpCopies = 8;
-    union Hist {
-        ResidualHist fixed;
-        LdsHist<kFpCopies> fp;
-    };
-    __shared__ std::conditional_t<HIST, Hist, int> hist_mem;      // no histogram memory without HIST
-    Hist& hist = reinterpret_cast<Hist&>(hist_mem);
     enum { kPlain, kFixed, kFp, kBin0 };
     const int mode = !HIST ? kPlain : !(__builtin_fabsf(inv) < __builtin_inff()) ? kBin0 : inv != 0.0f ? kFixed : kFp;
     const int shift = narrow != INT_MIN ? 3 : copies_shift;        // 8 = kMaxCopies
@@ -157,7 +158,9 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
     const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &narrow)
                       : stats_parts < 0 ? ws->qp.inv_scale
                                         : 1.0f / scale_val;
-    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY>(x, n, inv, narrow, zero_point, codes, ws, copies_shift, blockIdx.x, gridDim.x);
+    __shared__ std::conditional_t<HIST, QuantHist, int> hist_mem;      // no histogram memory without HIST
+    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY>(x, n, inv, narrow, zero_point, codes, ws, copies_shift, blockIdx.x, gridDim.x,
+                                                       reinterpret_cast<QuantHist&>(hist_mem));
 }
 
 // K2 with the scale given and no histogram (quantize_per_tensor_uint8, compression.cpp:9-43), one

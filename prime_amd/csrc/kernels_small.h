@@ -32,12 +32,7 @@ __global__ __launch_bounds__(kThreads) void uniform_small_kernel(const float* __
                                                                  prime_qparams* qp_out, uint8_t* __restrict__ codes,
                                                                  float* __restrict__ lut, Workspace* ws, int copies_shift) {
     using M = Mem<ALIGNED, false>;
-    constexpr int kFpCopies = 8;
-    union Hist {
-        ResidualHist fixed;
-        LdsHist<kFpCopies> fp;
-    };
-    __shared__ Hist hist;
+    __shared__ QuantHist hist;
     __shared__ double sh_s[kSmallSlots][kWaves];
     __shared__ double sh_q[kSmallSlots][kWaves];
     __shared__ double sh_part_s[kSmallSlots];
