@@ -50,7 +50,13 @@ const char* prime_hip_last_error(void);
  * that re-reads a tensor walks it from its end), "hist_replicas" (copies
  * of each LDS histogram bin in the fused quantize pass: 1, 2, 4, 8), "nt_load_min_mib" (tensors at least this large
  * are read with non-temporal loads in their first pass), "nt_second_min_mib" (the same for the
- * quantize pass that reads a tensor for the last time).  Returns 0 if the name is known.  The
+ * quantize pass that reads a tensor for the last time), "one_shot" (kernels that keep nothing from
+ * tile to tile - dequantize, plain quantize, divide, pseudo-gradient, outer step, copy - run as one
+ * 256-lane workgroup per tile from 65536 elements up instead of a loop) and "one_shot_store_policy"
+ * (cache policy of their stores), "small_max_elems" (uniform_8bit_quantize of at most this many
+ * elements, and at most four rows of 4096, takes one launch of one workgroup; 0: never),
+ * "grid_cap" (upper bound on the workgroups of a looping kernel, for experiments; 0: none).
+ * No option changes a result.  Returns 0 if the name is known.  The
  * options are process-wide and read at launch time: set them before work is enqueued, not
  * concurrently with it. */
 int prime_hip_set_option(const char* name, int value);
