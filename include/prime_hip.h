@@ -48,7 +48,8 @@ const char* prime_hip_last_error(void);
  * policy of the stores of codes, of fp32 outputs, of fp32 outputs the next kernel reads back, of
  * the plain copy: 0 write-back, 2 non-temporal, 16 write-through), "reverse_second_pass" (the pass
  * that re-reads a tensor walks it from its end), "hist_replicas" (copies
- * of each LDS histogram bin in the fused quantize pass: 1, 2, 4, 8), "nt_load_min_mib" (tensors at least this large
+ * of each LDS histogram bin in the fused quantize pass: 1, 2, 4, 8), "average_replicas" (the same for
+ * average_buckets' histogram: 1, 2, 4, 8, 16), "nt_load_min_mib" (tensors at least this large
  * are read with non-temporal loads in their first pass), "nt_second_min_mib" (the same for the
  * quantize pass that reads a tensor for the last time), "one_shot" (kernels that keep nothing from
  * tile to tile - dequantize, plain quantize, divide, pseudo-gradient, outer step, copy - run as one

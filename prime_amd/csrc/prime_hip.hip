@@ -55,6 +55,7 @@ struct Options {
     int64_t large_read_min_elems = int64_t(1) << 27;
     int nt_load_min_mib = 512;      // tensors of at least this many MiB are loaded with the non-temporal hint
     int nt_second_min_mib = 0;      // the same for the quantize pass that re-reads a tensor: its last use, always hinted
+    int average_replicas = 8;       // 1, 2, 4, 8 or 16 copies of each LDS bin of average_buckets' fp64 histogram
     int hist_replicas = 4;          // 1, 2, 4 or 8 copies of each LDS bin of the fused quantize pass
     int code_store_policy = kStoreNt;   // cache policy of the code stores (0 plain, 2 nt, 16 write-through)
     int reverse_second_pass = 1;    // the pass that re-reads a tensor walks it from its end
@@ -376,6 +377,10 @@ int prime_hip_set_option(const char* name, int value) {
         if (value != 1 && value != 2 && value != 4 && value != 8)
             return fail(PRIME_EINVAL, "hist_replicas must be 1, 2, 4 or 8");
         g_opt.hist_replicas = value;
+    } else if (!strcmp(name, "average_replicas")) {
+        if (value != 1 && value != 2 && value != 4 && value != 8 && value != 16)
+            return fail(PRIME_EINVAL, "average_replicas must be 1, 2, 4, 8 or 16");
+        g_opt.average_replicas = value;
     } else if (!strcmp(name, "code_store_policy")) {
         if (value != kStorePlain && value != kStoreNt && value != kStoreWriteThrough)
             return fail(PRIME_EINVAL, "code_store_policy must be 0 (plain), 2 (non-temporal) or 16 (write-through)");
@@ -423,6 +428,7 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "reverse_second_pass")) *value = g_opt.reverse_second_pass;
     else if (!strcmp(name, "large_read_grid_eighths")) *value = g_opt.large_read_grid_eighths;
     else if (!strcmp(name, "large_read_min_mi_elems")) *value = static_cast<int>(g_opt.large_read_min_elems >> 20);
+    else if (!strcmp(name, "average_replicas")) *value = g_opt.average_replicas;
     else if (!strcmp(name, "grid_cap")) *value = g_opt.grid_cap;
     else if (!strcmp(name, "one_shot")) *value = g_opt.one_shot;
     else if (!strcmp(name, "one_shot_store_policy")) *value = g_opt.one_shot_store_policy;
@@ -514,10 +520,19 @@ int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64
     if (n > 0) {
         grid = grid_for(n, true);
         const int nb = static_cast<int>(n_bins < kBins ? n_bins : kBins);
-        if (aligned_to(x, 16) && aligned_to(codes, 4))
-            launch(kIdHist, 5.0 * n, hist_kernel<true, 8>, grid, kThreads, st, x, codes, n, nb, w);
-        else
-            launch(kIdHist, 5.0 * n, hist_kernel<false, 8>, grid, kThreads, st, x, codes, n, nb, w);
+        const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
+        auto go = [&](auto copies) {
+            constexpr int R = decltype(copies)::value;
+            if (al) launch(kIdHist, 5.0 * n, hist_kernel<true, R>, grid, kThreads, st, x, codes, n, nb, w);
+            else launch(kIdHist, 5.0 * n, hist_kernel<false, R>, grid, kThreads, st, x, codes, n, nb, w);
+        };
+        switch (g_opt.average_replicas) {
+            case 1: go(std::integral_constant<int, 1>{}); break;
+            case 2: go(std::integral_constant<int, 2>{}); break;
+            case 4: go(std::integral_constant<int, 4>{}); break;
+            case 16: go(std::integral_constant<int, 16>{}); break;
+            default: go(std::integral_constant<int, 8>{}); break;
+        }
         if (int rc = launch_check("hist_kernel")) return rc;
     }
     return run_lut_finalize(w, grid, lut, n_bins, counts, st);

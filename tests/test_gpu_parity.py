@@ -450,7 +450,7 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
     assert np.all(np.abs(le - ref_lut)[both] <= (3 * abs(rel) + 2e-5) * np.maximum(np.abs(ref_lut[both]), float(q["scale"])))
 
 
-@pytest.mark.parametrize("option,values", [("hist_replicas", (1, 2, 4, 8)), ("blocks_per_cu", (1, 2, 3, 4)),
+@pytest.mark.parametrize("option,values", [("hist_replicas", (1, 2, 4, 8)), ("average_replicas", (1, 2, 4, 8, 16)), ("blocks_per_cu", (1, 2, 3, 4)),
                                            ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20)),
                                            ("code_store_policy", (0, 2, 16)), ("f32_reread_store_policy", (0, 2, 16)),
                                            ("reverse_second_pass", (0, 1)), ("one_shot", (0, 1)),
