@@ -27,19 +27,32 @@ __device__ __forceinline__ float lut_entry_of_rows(const BinAcc (&part)[kSmallSl
 
 // `rows` <= kSmallSlots is the grid the three-launch sequence uses for this tensor: one workgroup per
 // row of whole vectors (the last of them may be left with the ragged end only, or with nothing).
-template <bool ALIGNED>
-__global__ __launch_bounds__(kThreads) void uniform_small_kernel(const float* __restrict__ x, int64_t n, int rows,
+// SRC says where the values come from: the tensor as it stands (uniform_8bit_quantize), or a ring
+// step's first pass folded in - x = lut_in[codes_in] (gather step), x += lut_in[codes_in] (reduce
+// step), the same divided by `divisor` (the last accumulation of an averaged chunk) - with the
+// updated values written back, as dequant_kernel<.., STATS, ..> does ahead of the quantize pass.
+enum SmallSource { kSmallTensor = 0, kSmallSet = 1, kSmallAdd = 2, kSmallAddDiv = 3 };
+
+template <bool ALIGNED, int SRC>
+__global__ __launch_bounds__(kThreads) void uniform_small_kernel(float* __restrict__ x, int64_t n, int rows,
                                                                  prime_qparams* qp_out, uint8_t* __restrict__ codes,
-                                                                 float* __restrict__ lut, Workspace* ws, int copies_shift) {
+                                                                 float* __restrict__ lut, Workspace* ws, int copies_shift,
+                                                                 const uint8_t* codes_in, const float* lut_in,
+                                                                 float divisor) {
     using M = Mem<ALIGNED, false>;
     __shared__ QuantHist hist;
     __shared__ double sh_s[kSmallSlots][kWaves];
     __shared__ double sh_q[kSmallSlots][kWaves];
     __shared__ double sh_part_s[kSmallSlots];
     __shared__ double sh_part_q[kSmallSlots];
+    __shared__ float s_lut[SRC == kSmallTensor ? 1 : kBins];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t nvec = n >> 2;
     const int tail = static_cast<int>(n & 3);
+    if (SRC != kSmallTensor) {
+        for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut_in[b];
+        __syncthreads();
+    }
 
     // the lane's vector of every row, and its element of the ragged end
     f4a v[kSmallSlots];
@@ -48,10 +61,36 @@ __global__ __launch_bounds__(kThreads) void uniform_small_kernel(const float* __
     for (int r = 0; r < kSmallSlots; ++r) {
         const int64_t i = static_cast<int64_t>(r) * kThreads + threadIdx.x;
         has[r] = r < rows && i < nvec;
-        v[r] = has[r] ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+        v[r] = f4a{0.f, 0.f, 0.f, 0.f};
+        if (SRC == kSmallTensor || SRC == kSmallAdd || SRC == kSmallAddDiv) {
+            if (has[r]) v[r] = M::ldf4(x, i);
+        }
+        if (SRC != kSmallTensor && has[r]) {
+            const uint32_t c = M::ldu32(codes_in, i);
+            f4a l;
+            l.x = s_lut[c & 255];
+            l.y = s_lut[(c >> 8) & 255];
+            l.z = s_lut[(c >> 16) & 255];
+            l.w = s_lut[c >> 24];
+            if (SRC == kSmallSet) v[r] = l;
+            else v[r] = l + v[r];
+            if (SRC == kSmallAddDiv) v[r] = v[r] / divisor;
+            M::stf4(x, i, v[r], false);
+        }
     }
     const bool has_tail = static_cast<int>(threadIdx.x) < tail;
-    const float tail_v = has_tail ? x[(nvec << 2) + threadIdx.x] : 0.0f;
+    float tail_v = 0.0f;
+    if (has_tail) {
+        const int64_t i = (nvec << 2) + threadIdx.x;
+        if (SRC == kSmallTensor) {
+            tail_v = x[i];
+        } else {
+            tail_v = s_lut[codes_in[i]];
+            if (SRC != kSmallSet) tail_v += x[i];
+            if (SRC == kSmallAddDiv) tail_v = tail_v / divisor;
+            x[i] = tail_v;
+        }
+    }
 
     // statistics: per row what stats_partial computes for the workgroup of that row
 #pragma unroll

@@ -109,7 +109,8 @@ int shot_grid(int64_t nvec) {
     const int64_t tile = static_cast<int64_t>(kShotThreads) * kShotUnroll;
     return static_cast<int>((nvec + tile - 1) / tile);
 }
-inline bool one_shot(int64_t n) { return g_opt.one_shot && n >= g_opt.one_shot_min_elems; }
+// (a dispatch counts its work-items in 32 bits: beyond 2^34 elements the looping kernels take over)
+inline bool one_shot(int64_t n) { return g_opt.one_shot && n >= g_opt.one_shot_min_elems && n <= (int64_t(1) << 34); }
 
 inline bool use_nt(int64_t n) { return (n >> 18) >= g_opt.nt_load_min_mib; }   // n floats = n / 2^18 MiB
 
@@ -563,15 +564,24 @@ bool small_applies(int64_t n) {
     return grid <= kSmallSlots && rows <= grid;
 }
 
-int run_uniform_small(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qp_out, Workspace* ws, hipStream_t st) {
+template <int SRC>
+int run_small(float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qp_out, Workspace* ws, hipStream_t st,
+              const uint8_t* codes_in, const float* lut_in, float divisor) {
     const int rows = grid_for(n, true);
     int shift = 0;
     while ((1 << (shift + 1)) <= g_opt.hist_replicas) ++shift;
-    if (aligned_to(x, 16) && aligned_to(codes, 4))
-        launch(kIdUniformSmall, 9.0 * n, uniform_small_kernel<true>, 1, kThreads, st, x, n, rows, qp_out, codes, lut, ws, shift);
+    if (aligned_to(x, 16) && aligned_to(codes, 4) && aligned_to(codes_in, 4))
+        launch(kIdUniformSmall, (SRC == kSmallTensor ? 9.0 : SRC == kSmallSet ? 10.0 : 14.0) * n, uniform_small_kernel<true, SRC>, 1, kThreads, st, x, n,
+               rows, qp_out, codes, lut, ws, shift, codes_in, lut_in, divisor);
     else
-        launch(kIdUniformSmall, 9.0 * n, uniform_small_kernel<false>, 1, kThreads, st, x, n, rows, qp_out, codes, lut, ws, shift);
+        launch(kIdUniformSmall, (SRC == kSmallTensor ? 9.0 : SRC == kSmallSet ? 10.0 : 14.0) * n, uniform_small_kernel<false, SRC>, 1, kThreads, st, x, n,
+               rows, qp_out, codes, lut, ws, shift, codes_in, lut_in, divisor);
     return launch_check("uniform_small_kernel");
+}
+
+int run_uniform_small(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qp_out, Workspace* ws, hipStream_t st) {
+    // (the kernel only reads the tensor when it is the source)
+    return run_small<kSmallTensor>(const_cast<float*>(x), n, codes, lut, qp_out, ws, st, nullptr, nullptr, 1.0f);
 }
 
 int uniform_three_launches(const float* x, int64_t n, uint8_t* codes, float* lut, prime_qparams* qparams_out, Workspace* w, hipStream_t st) {
@@ -708,6 +718,11 @@ int ring_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_
     if (n == 0) {
         if (int rc = run_stats(chunk, 0, qparams_out, w, st)) return rc;
         return run_lut_finalize(w, 0, lut_out, kBins, nullptr, st);
+    }
+    if (small_applies(n)) {               // one launch of one workgroup, the same results bit for bit
+        if (!ADD) return run_small<kSmallSet>(chunk, n, codes_out, lut_out, qparams_out, w, st, codes_in, lut_in, 1.0f);
+        if (divisor != 1.0f) return run_small<kSmallAddDiv>(chunk, n, codes_out, lut_out, qparams_out, w, st, codes_in, lut_in, divisor);
+        return run_small<kSmallAdd>(chunk, n, codes_out, lut_out, qparams_out, w, st, codes_in, lut_in, 1.0f);
     }
     int grid = 0;
     if (ADD && divisor != 1.0f) {

@@ -533,6 +533,53 @@ def test_one_launch_for_a_small_tensor_equals_the_three_launches_bit_for_bit(abi
         _lib.set_option("small_max_elems", saved)
 
 
+@pytest.mark.parametrize("n", [1, 3, 5, 1023, 4095, 4096, 4097, 4099, 8191, 8192])
+def test_one_launch_ring_steps_on_small_chunks_equal_the_three_launches_bit_for_bit(abi, oracle, n):
+    # reduce step, gather step and the dividing reduce step on chunks of up to 8192 elements: one
+    # launch of one workgroup; accumulator, codes, table and statistics record must be those of the
+    # three launches bit for bit, and the accumulator the oracle's
+    rng = np.random.default_rng(1000 + n)
+    acc0 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    codes_np = rng.integers(0, 256, n, dtype=np.uint8)
+    lut_np = (np.sort(rng.standard_normal(256)) * 2e-3).astype(np.float32)
+    saved = _lib.get_option("small_max_elems")
+    cases = {"reduce": dict(), "gather": dict(gather=True), "reduce and divide": dict(divisor=3.0), "divide by one": dict(divisor=1.0)}
+    try:
+        for shift in (0, 1) if n in (4097, 8191) else (0,):
+            for label, kw in cases.items():
+                announce(f"small ring step {label} n={n} shift={shift}")
+                out = {}
+                for mode, limit in (("three launches", 0), ("one launch", saved)):
+                    _lib.set_option("small_max_elems", limit)
+                    buf = torch.zeros(n + 8, dtype=torch.float32, device=abi.dev)
+                    acc = buf[shift:shift + n]
+                    acc.copy_(torch.from_numpy(acc0))
+                    cbuf = torch.zeros(n + 8, dtype=torch.uint8, device=abi.dev)
+                    cin = cbuf[shift:shift + n]
+                    cin.copy_(torch.from_numpy(codes_np))
+                    _lib.profile_begin()
+                    c, l, q = abi.ring_step(acc, cin, abi.to_dev(lut_np), **kw)
+                    torch.cuda.synchronize()
+                    prof = _lib.profile_end()
+                    assert ("uniform_small_kernel" in prof) == (limit > 0) and len(prof) == (1 if limit else 3), (mode, list(prof))
+                    out[mode] = (acc.clone(), c, l, q)
+                a, b = out["three launches"], out["one launch"]
+                assert torch.equal(a[0].view(torch.int32), b[0].view(torch.int32)), label
+                assert torch.equal(a[1], b[1]), label
+                assert torch.equal(a[2].view(torch.int32), b[2].view(torch.int32)), label
+                assert torch.equal(a[3].view(torch.int64), b[3].view(torch.int64)), label
+                want = acc0.copy()
+                if kw.get("gather"):
+                    want = lut_np[codes_np]
+                else:
+                    oracle.index_add(want, lut_np, codes_np)
+                    if kw.get("divisor", 1.0) != 1.0:
+                        want = want / np.float32(kw["divisor"])
+                assert np.array_equal(b[0].cpu().numpy(), want), label
+    finally:
+        _lib.set_option("small_max_elems", saved)
+
+
 def test_the_default_limit_of_the_one_launch_path(abi):
     for n, small in ((1, True), (8192, True), (8193, False), (16384, False), (40000, False), (1 << 20, False)):
         x = torch.randn(n, device=abi.dev)
