@@ -135,9 +135,27 @@ struct Window {
     }
 };
 
+// The value of lane i + N of the same row of 16 lanes (N < 16), by data-parallel primitives: no LDS
+// traffic, unlike a shuffle.  Lanes whose source lies outside their row get an unspecified value.
+template <int N>
+__device__ __forceinline__ double row_down(double v) {
+    const long long b = __double_as_longlong(v);
+    const int lo = static_cast<int>(b), hi = static_cast<int>(b >> 32);
+    const int lo2 = __builtin_amdgcn_update_dpp(lo, lo, 0x100 + N, 0xf, 0xf, false);     // row_shl:N
+    const int hi2 = __builtin_amdgcn_update_dpp(hi, hi, 0x100 + N, 0xf, 0xf, false);
+    return __longlong_as_double((static_cast<long long>(hi2) << 32) | static_cast<unsigned>(lo2));
+}
+
+// Sum over the wavefront, valid in lane 0: lane i adds lane i + 32, then i + 16, 8, 4, 2, 1 (a fixed
+// tree, so the result depends on the values alone).  Lane 0 only ever takes from lanes below 16 in
+// the last four steps, which therefore stay inside a row.
 __device__ __forceinline__ double wave_sum(double v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    v += __shfl_down(v, 32, 64);
+    v += __shfl_down(v, 16, 64);
+    v += row_down<8>(v);
+    v += row_down<4>(v);
+    v += row_down<2>(v);
+    v += row_down<1>(v);
     return v;
 }
 
@@ -393,15 +411,18 @@ __device__ __forceinline__ int residual_fixed(float x, float inv, int code) {
     return residual_units(x, inv, static_cast<float>(code - kZeroPoint));
 }
 
-// `copy` = the lane's copy index, threadIdx.x & ((1 << shift) - 1)
-__device__ __forceinline__ void rhist_add(ResidualHist& h, int shift, int copy, int code, int fixed) {
+// `copy` = the lane's copy index, threadIdx.x & ((1 << shift) - 1).  H is ResidualHist or any struct
+// with its `slot`, `far_sum` and `far_cnt` members.
+template <typename H>
+__device__ __forceinline__ void rhist_add(H& h, int shift, int copy, int code, int fixed) {
     const unsigned long long v = (1ull << 48) | static_cast<unsigned long long>(static_cast<unsigned>(fixed) ^ 0x80000000u);
     __hip_atomic_fetch_add(&h.slot[(code << shift) + copy], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
 __device__ __forceinline__ bool is_far(float x, float inv) { return !(__builtin_fabsf(x * inv) <= kFarBins); }
 
-__device__ __forceinline__ void rhist_add_far(ResidualHist& h, int code, float x) {
+template <typename H>
+__device__ __forceinline__ void rhist_add_far(H& h, int code, float x) {
     const int side = code == kBins - 1, c = threadIdx.x & (kFarCopies - 1);
     __hip_atomic_fetch_add(&h.far_sum[side][c], static_cast<double>(x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     __hip_atomic_fetch_add(&h.far_cnt[side][c], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -423,7 +444,8 @@ __device__ __forceinline__ float round_centre(float q) {
 // + 128 as a float, whose bit pattern is a constant plus the code: the low byte is the code for the
 // packed word, and the whole pattern shifted left addresses the slot (the constant is taken out of
 // the lane's base offset, modulo 2^32), so that the code never exists as an integer of its own.
-__device__ __forceinline__ uint32_t rhist_quantize4(ResidualHist& h, int shift, int copy, const f4a v, float inv) {
+template <typename H>
+__device__ __forceinline__ uint32_t rhist_quantize4(H& h, int shift, int copy, const f4a v, float inv) {
     const float qa = v.x * inv, qb = v.y * inv, qc = v.z * inv, qd = v.w * inv;
     const bool ra = !(__builtin_fabsf(qa) <= kFarBins), rb = !(__builtin_fabsf(qb) <= kFarBins),
                rc = !(__builtin_fabsf(qc) <= kFarBins), rd = !(__builtin_fabsf(qd) <= kFarBins);
@@ -481,22 +503,35 @@ __device__ __forceinline__ void rhist_flush(ResidualHist& h, int shift) {
     __syncthreads();
 }
 
-// Bin b of the workgroup's partial, after a last flush: the bin's sum of x in fp64 and its count.
-__device__ __forceinline__ BinAcc rhist_bin(const ResidualHist& h, float inv, int b) {
-    const unsigned long long cnt = h.wide_cnt[b];
-    unsigned long long far_n = 0;
-    double far_s = 0.0;
+// A bin's entry of a workgroup's partial from its integer totals: the count, the sum of the residuals
+// in units of 2^-22 bin, and for the two clip bins the far elements' count and fp64 sum of x.
+__device__ __forceinline__ BinAcc rhist_entry(unsigned long long cnt, long long units, unsigned long long far_n, double far_s, float inv, int b) {
+    const double centre = static_cast<double>(static_cast<long long>(cnt - far_n) * (b - kZeroPoint));
+    const double bins = centre + static_cast<double>(units) * (1.0 / kResidualOne);
+    BinAcc acc;
+    acc.sum = bins / static_cast<double>(inv) + far_s;
+    acc.cnt = cnt;
+    return acc;
+}
+
+// The far elements of bin b (0 or 255), their copies added in order.
+template <typename H>
+__device__ __forceinline__ void rhist_far_of(const H& h, int b, unsigned long long& far_n, double& far_s) {
+    far_n = 0;
+    far_s = 0.0;
     if (b == 0 || b == kBins - 1) {
         const int side = b != 0;
 #pragma unroll
         for (int c = 0; c < kFarCopies; ++c) { far_n += h.far_cnt[side][c]; far_s += h.far_sum[side][c]; }
     }
-    const double centre = static_cast<double>(static_cast<long long>(cnt - far_n) * (b - kZeroPoint));
-    const double bins = centre + static_cast<double>(h.wide_sum[b]) * (1.0 / kResidualOne);
-    BinAcc acc;
-    acc.sum = bins / static_cast<double>(inv) + far_s;
-    acc.cnt = cnt;
-    return acc;
+}
+
+// Bin b of the workgroup's partial, after a last flush: the bin's sum of x in fp64 and its count.
+__device__ __forceinline__ BinAcc rhist_bin(const ResidualHist& h, float inv, int b) {
+    unsigned long long far_n;
+    double far_s;
+    rhist_far_of(h, b, far_n, far_s);
+    return rhist_entry(h.wide_cnt[b], h.wide_sum[b], far_n, far_s, inv, b);
 }
 
 // The workgroup's partial as workgroup `slot`, 4 KiB contiguous.

@@ -10,7 +10,16 @@
 // Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
 
 constexpr int kSmallSlots = 4;
-static_assert(kThreads >= kBins && kSmallSlots <= 4, "the table's tree is written for four rows, one bin per lane");
+constexpr int kSmallShift = 1;          // two LDS copies of each bin per row (any number gives the same integer sums)
+static_assert(kThreads == 1024 && kBins == 256 && kSmallSlots == 4, "lane -> (row, bin) covers four rows of 256 bins; the tree is written for four rows");
+
+// One row's fixed-point histogram: a row adds at most 4 * kThreads + 3 elements, so no slot can
+// overflow its 16-bit count and the slots are read out directly, without the 64-bit accumulators.
+struct SmallRowHist {
+    unsigned long long slot[kBins << kSmallShift];
+    double far_sum[2][kFarCopies];
+    unsigned far_cnt[2][kFarCopies];
+};
 
 __device__ __forceinline__ BinAcc binacc_add(BinAcc a, BinAcc b) { return BinAcc{a.sum + b.sum, a.cnt + b.cnt}; }
 
@@ -40,7 +49,12 @@ __global__ __launch_bounds__(kThreads) void uniform_small_kernel(float* __restri
                                                                  const uint8_t* codes_in, const float* lut_in,
                                                                  float divisor) {
     using M = Mem<ALIGNED, false>;
-    __shared__ QuantHist hist;
+    union Hists {
+        QuantHist one;                    // row by row, when the histogram is not the fixed-point one
+        SmallRowHist row[kSmallSlots];    // all rows side by side
+    };
+    __shared__ Hists hists;
+    QuantHist& hist = hists.one;
     __shared__ double sh_s[kSmallSlots][kWaves];
     __shared__ double sh_q[kSmallSlots][kWaves];
     __shared__ double sh_part_s[kSmallSlots];
@@ -92,21 +106,37 @@ __global__ __launch_bounds__(kThreads) void uniform_small_kernel(float* __restri
         }
     }
 
-    // statistics: per row what stats_partial computes for the workgroup of that row
+    // statistics: per row what stats_partial computes for the workgroup of that row; the rows that
+    // exist are reduced side by side (their shuffle chains overlap), the others not at all
+    auto stats_of = [&](auto count) {
+        constexpr int N = decltype(count)::value;
+        double s[N], q[N];
 #pragma unroll
-    for (int r = 0; r < kSmallSlots; ++r) {
-        if (r >= rows) continue;         // uniform over the workgroup
-        double s = 0.0, q = 0.0;
-        stats_add4(v[r], s, q);
-        if (r == 0 && has_tail) {
-            const double t = tail_v;
-            s += t;
-            q = fma(t, t, q);
+        for (int r = 0; r < N; ++r) {
+            s[r] = 0.0;
+            q[r] = 0.0;
+            stats_add4(v[r], s[r], q[r]);
+            if (r == 0 && has_tail) {
+                const double t = tail_v;
+                s[r] += t;
+                q[r] = fma(t, t, q[r]);
+            }
+            s[r] += 0.0;                  // the second accumulator pair of the streaming kernel stays at zero
+            q[r] += 0.0;
         }
-        s = wave_sum(s + 0.0);           // the second accumulator pair of the streaming kernel stays at zero
-        q = wave_sum(q + 0.0);
-        if (lane == 0) { sh_s[r][wave] = s; sh_q[r][wave] = q; }
-    }
+#pragma unroll
+        for (int r = 0; r < N; ++r) {                 // independent chains: the compiler overlaps them
+            s[r] = wave_sum(s[r]);
+            q[r] = wave_sum(q[r]);
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < N; ++r) { sh_s[r][wave] = s[r]; sh_q[r][wave] = q[r]; }
+        }
+    };
+    if (rows <= 1) stats_of(std::integral_constant<int, 1>{});
+    else if (rows == 2) stats_of(std::integral_constant<int, 2>{});
+    else stats_of(std::integral_constant<int, kSmallSlots>{});
     __syncthreads();
     if (static_cast<int>(threadIdx.x) < rows) {
         double S = sh_s[threadIdx.x][0], Q = sh_q[threadIdx.x][0];
@@ -123,71 +153,116 @@ __global__ __launch_bounds__(kThreads) void uniform_small_kernel(float* __restri
     const double pb = (0.0 + (mine ? sh_part_q[threadIdx.x & (kSmallSlots - 1)] : 0.0)) + 0.0;
     const float inv = block_scale_reduce<kThreads>(pa, pb, ws, n, qp_out, &narrow);
 
-    // codes and histogram, row by row; the modes are those of quantize_block
+    // codes and histogram; the modes are those of quantize_block
     enum { kFixed, kFp, kBin0 };
     const int mode = !(__builtin_fabsf(inv) < __builtin_inff()) ? kBin0 : inv != 0.0f ? kFixed : kFp;
-    const int shift = narrow != INT_MIN ? 3 : copies_shift;
-    const int copy = threadIdx.x & ((1 << shift) - 1);
     BinAcc part[kSmallSlots];
-    for (int r = 0; r < kSmallSlots; ++r) part[r] = BinAcc{0.0, 0ull};
 #pragma unroll
-    for (int r = 0; r < kSmallSlots; ++r) {
-        if (r < rows) {                   // uniform over the workgroup
+    for (int r = 0; r < kSmallSlots; ++r) part[r] = BinAcc{0.0, 0ull};
+    const int64_t ti = (nvec << 2) + threadIdx.x;
+    if (mode == kFixed) {
+        // all rows at once, each into its own histogram
+        unsigned long long* all = &hists.row[0].slot[0];
+        for (int i = threadIdx.x; i < rows * static_cast<int>(sizeof(SmallRowHist) / 8); i += kThreads) all[i] = 0ull;   // zero bits are 0.0 and 0u too
+        __syncthreads();
+        const int copy = threadIdx.x & ((1 << kSmallShift) - 1);
+#pragma unroll
+        for (int r = 0; r < kSmallSlots; ++r) {
             const int64_t i = static_cast<int64_t>(r) * kThreads + threadIdx.x;
-            const int64_t ti = (nvec << 2) + threadIdx.x;
-            if (mode == kFixed) {
-                rhist_zero(hist.fixed, shift);
+            if (has[r]) M::stu32(codes, i, rhist_quantize4(hists.row[r], kSmallShift, copy, v[r], inv));
+        }
+        if (has_tail) {
+            const int a = quantize_code(tail_v, inv, kZeroPoint);
+            codes[ti] = static_cast<uint8_t>(a);
+            const bool far = is_far(tail_v, inv);
+            if (far) rhist_add_far(hists.row[0], a, tail_v);
+            rhist_add(hists.row[0], kSmallShift, copy, a, far ? 0 : residual_fixed(tail_v, inv, a));
+        }
+        __syncthreads();
+        // lane -> (row, bin): the bin's entry of that row's partial, left where the bin's slots were
+        const int bin = threadIdx.x & (kBins - 1);
+#pragma unroll
+        for (int pass = 0; pass < kSmallSlots * kBins / kThreads; ++pass) {
+            const int r = pass * (kThreads / kBins) + (threadIdx.x >> 8);
+            if (r >= rows) continue;      // uniform over the wavefront
+            SmallRowHist& h = hists.row[r];
+            unsigned long long cnt = 0, sum = 0;
+#pragma unroll
+            for (int c = 0; c < (1 << kSmallShift); ++c) {
+                const unsigned long long s = h.slot[(bin << kSmallShift) + c];
+                cnt += s >> 48;
+                sum += s & 0xffffffffffffull;
+            }
+            unsigned long long far_n;
+            double far_s;
+            rhist_far_of(h, bin, far_n, far_s);
+            const BinAcc e = rhist_entry(cnt, static_cast<long long>(sum) - static_cast<long long>(cnt << 31), far_n, far_s, inv, bin);
+            static_assert(kSmallShift >= 1, "an entry takes the place of two slots");
+            h.slot[(bin << kSmallShift)] = static_cast<unsigned long long>(__double_as_longlong(e.sum));
+            h.slot[(bin << kSmallShift) + 1] = e.cnt;
+        }
+        __syncthreads();
+        if (threadIdx.x < kBins) {
+#pragma unroll
+            for (int r = 0; r < kSmallSlots; ++r) {
+                if (r < rows) {
+                    part[r].sum = __longlong_as_double(static_cast<long long>(hists.row[r].slot[(bin << kSmallShift)]));
+                    part[r].cnt = hists.row[r].slot[(bin << kSmallShift) + 1];
+                }
+            }
+        }
+    } else {
+        // row by row through one histogram (rare: a zero or non-finite 1 / scale)
+        auto set_part = [&](int r, BinAcc e) {
+#pragma unroll
+            for (int k = 0; k < kSmallSlots; ++k)
+                if (r == k) part[k] = e;
+        };
+        for (int r = 0; r < rows; ++r) {
+            const int64_t i = static_cast<int64_t>(r) * kThreads + threadIdx.x;
+            f4a vr = v[0];
+            bool hr = has[0];
+#pragma unroll
+            for (int k = 1; k < kSmallSlots; ++k)
+                if (r == k) { vr = v[k]; hr = has[k]; }
+            int a = 0, b = 0, c = 0, d = 0;
+            if (hr) {
+                a = quantize_code(vr.x, inv, kZeroPoint);
+                b = quantize_code(vr.y, inv, kZeroPoint);
+                c = quantize_code(vr.z, inv, kZeroPoint);
+                d = quantize_code(vr.w, inv, kZeroPoint);
+                M::stu32(codes, i, static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) | (static_cast<uint32_t>(c) << 16) |
+                                       (static_cast<uint32_t>(d) << 24));
+            }
+            const bool tail_here = r == 0 && has_tail;
+            const int ta = tail_here ? quantize_code(tail_v, inv, kZeroPoint) : 0;
+            if (tail_here) codes[ti] = static_cast<uint8_t>(ta);
+            if (mode == kFp) {
+                hist_zero(hist.fp);
                 __syncthreads();
-                if (has[r]) M::stu32(codes, i, rhist_quantize4(hist.fixed, shift, copy, v[r], inv));
-                if (r == 0 && has_tail) {
-                    const int a = quantize_code(tail_v, inv, kZeroPoint);
-                    codes[ti] = static_cast<uint8_t>(a);
-                    const bool far = is_far(tail_v, inv);
-                    if (far) rhist_add_far(hist.fixed, a, tail_v);
-                    rhist_add(hist.fixed, shift, copy, a, far ? 0 : residual_fixed(tail_v, inv, a));
+                if (hr) {
+                    hist_add(hist.fp, a, vr.x);
+                    hist_add(hist.fp, b, vr.y);
+                    hist_add(hist.fp, c, vr.z);
+                    hist_add(hist.fp, d, vr.w);
                 }
-                rhist_flush(hist.fixed, shift);
-                if (threadIdx.x < kBins) part[r] = rhist_bin(hist.fixed, inv, threadIdx.x);
+                if (tail_here) hist_add(hist.fp, ta, tail_v);
                 __syncthreads();
-            } else {
-                int a = 0, b = 0, c = 0, d = 0;
-                if (has[r]) {
-                    a = quantize_code(v[r].x, inv, kZeroPoint);
-                    b = quantize_code(v[r].y, inv, kZeroPoint);
-                    c = quantize_code(v[r].z, inv, kZeroPoint);
-                    d = quantize_code(v[r].w, inv, kZeroPoint);
-                    M::stu32(codes, i, static_cast<uint32_t>(a) | (static_cast<uint32_t>(b) << 8) | (static_cast<uint32_t>(c) << 16) |
-                                           (static_cast<uint32_t>(d) << 24));
+                if (threadIdx.x < kBins) set_part(r, hist_bin(hist.fp, threadIdx.x));
+                __syncthreads();
+            } else {                      // every code is 0: one sum, lanes then wavefronts in the order of hist_store_bin0
+                double ls = 0.0;
+                unsigned long long lc = 0;
+                if (hr) {
+                    ls += static_cast<double>(vr.x);
+                    ls += static_cast<double>(vr.y);
+                    ls += static_cast<double>(vr.z);
+                    ls += static_cast<double>(vr.w);
+                    lc += 4;
                 }
-                const int ta = (r == 0 && has_tail) ? quantize_code(tail_v, inv, kZeroPoint) : 0;
-                if (r == 0 && has_tail) codes[ti] = static_cast<uint8_t>(ta);
-                if (mode == kFp) {
-                    hist_zero(hist.fp);
-                    __syncthreads();
-                    if (has[r]) {
-                        hist_add(hist.fp, a, v[r].x);
-                        hist_add(hist.fp, b, v[r].y);
-                        hist_add(hist.fp, c, v[r].z);
-                        hist_add(hist.fp, d, v[r].w);
-                    }
-                    if (r == 0 && has_tail) hist_add(hist.fp, ta, tail_v);
-                    __syncthreads();
-                    if (threadIdx.x < kBins) part[r] = hist_bin(hist.fp, threadIdx.x);
-                    __syncthreads();
-                } else {                  // every code is 0: one sum, lanes then wavefronts in the order of hist_store_bin0
-                    double ls = 0.0;
-                    unsigned long long lc = 0;
-                    if (has[r]) {
-                        ls += static_cast<double>(v[r].x);
-                        ls += static_cast<double>(v[r].y);
-                        ls += static_cast<double>(v[r].z);
-                        ls += static_cast<double>(v[r].w);
-                        lc += 4;
-                    }
-                    if (r == 0 && has_tail) { ls += static_cast<double>(tail_v); lc += 1; }
-                    const BinAcc total = block_sum_bin0(ls, lc);
-                    if (threadIdx.x == 0) part[r] = total;
-                }
+                if (tail_here) { ls += static_cast<double>(tail_v); lc += 1; }
+                const BinAcc total = block_sum_bin0(ls, lc);
+                if (threadIdx.x == 0) set_part(r, total);
             }
         }
     }

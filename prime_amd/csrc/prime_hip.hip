@@ -66,7 +66,7 @@ struct Options {
     int one_shot = 1;                                   // kernels that keep nothing between tiles: one workgroup per tile instead of a loop
     int64_t one_shot_min_elems = int64_t(1) << 16;      // ... from this many elements up
     int one_shot_store_policy = kStoreNt;               // cache policy of their fp32 stores
-    int64_t small_max_elems = int64_t(1) << 13;         // uniform_8bit_quantize takes one launch of one workgroup up to this many elements (0: never)
+    int64_t small_max_elems = int64_t(1) << 14;         // uniform_8bit_quantize takes one launch of one workgroup up to this many elements (0: never)
 };
 Options g_opt;
 

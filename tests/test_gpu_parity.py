@@ -507,7 +507,7 @@ def test_one_launch_for_a_small_tensor_equals_the_three_launches_bit_for_bit(abi
     # without a ragged end
     rng = np.random.default_rng(n)
     saved = _lib.get_option("small_max_elems")
-    assert saved == 1 << 13
+    assert saved == 1 << 14
     try:
         for label, x in _small_inputs(n, rng).items():
             for shift in (0, 1) if n in (4097, 16383) else (0,):
@@ -520,7 +520,7 @@ def test_one_launch_for_a_small_tensor_equals_the_three_launches_bit_for_bit(abi
                 torch.cuda.synchronize()
                 assert "uniform_small_kernel" not in _lib.profile_end()
                 announce(f"one launch n={n} {label} shift={shift}")
-                _lib.set_option("small_max_elems", 1 << 14)      # the most the kernel is built for: four rows
+                _lib.set_option("small_max_elems", saved)
                 for rep in range(2):
                     _lib.profile_begin()
                     got = abi.uniform(xt)
@@ -533,7 +533,7 @@ def test_one_launch_for_a_small_tensor_equals_the_three_launches_bit_for_bit(abi
         _lib.set_option("small_max_elems", saved)
 
 
-@pytest.mark.parametrize("n", [1, 3, 5, 1023, 4095, 4096, 4097, 4099, 8191, 8192])
+@pytest.mark.parametrize("n", [1, 3, 5, 1023, 4095, 4096, 4097, 4099, 8191, 8192, 12291, 16384])
 def test_one_launch_ring_steps_on_small_chunks_equal_the_three_launches_bit_for_bit(abi, oracle, n):
     # reduce step, gather step and the dividing reduce step on chunks of up to 8192 elements: one
     # launch of one workgroup; accumulator, codes, table and statistics record must be those of the
@@ -545,7 +545,7 @@ def test_one_launch_ring_steps_on_small_chunks_equal_the_three_launches_bit_for_
     saved = _lib.get_option("small_max_elems")
     cases = {"reduce": dict(), "gather": dict(gather=True), "reduce and divide": dict(divisor=3.0), "divide by one": dict(divisor=1.0)}
     try:
-        for shift in (0, 1) if n in (4097, 8191) else (0,):
+        for shift in (0, 1) if n in (4097, 8191, 12291) else (0,):
             for label, kw in cases.items():
                 announce(f"small ring step {label} n={n} shift={shift}")
                 out = {}
@@ -581,7 +581,7 @@ def test_one_launch_ring_steps_on_small_chunks_equal_the_three_launches_bit_for_
 
 
 def test_the_default_limit_of_the_one_launch_path(abi):
-    for n, small in ((1, True), (8192, True), (8193, False), (16384, False), (40000, False), (1 << 20, False)):
+    for n, small in ((1, True), (8192, True), (16384, True), (16385, False), (40000, False), (1 << 20, False)):
         x = torch.randn(n, device=abi.dev)
         _lib.profile_begin()
         abi.uniform(x)
