@@ -157,6 +157,8 @@ def bench_excerpt(path: str) -> str:
             out.append(f"  {key}: value={d[key]['value']} GB/s frac_of_hbm_peak={d[key]['frac_of_hbm_peak']} ms_per_hop={d[key]['ms_per_hop']}")
             for k, v in d[key]["kernels"].items():
                 out.append(f"    {k:30s} avg_us={v['avg_us']:9.2f} algo_GBps={v['algo_GBps']}")
+    if "other_configs" in d:
+        out.append("  other_configs: " + json.dumps(d["other_configs"]))
     if "diloco_outer_step" in d:
         out.append("  diloco_outer_step: " + json.dumps({k: v for k, v in d["diloco_outer_step"].items() if k != "workload"}))
     return "\n".join(out)
