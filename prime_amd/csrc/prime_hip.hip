@@ -62,10 +62,13 @@ struct Options {
     int grid_cap = 0;               // experiment: upper bound on the workgroups of a streaming kernel (0: none)
     int f32_store_policy = kStoreWriteThrough;          // fp32 outputs nobody reads back soon (dequantize, outer step)
     int f32_reread_store_policy = kStoreWriteThrough;   // fp32 outputs the next kernel reads back (ring step, first touch)
-    int copy_store_policy = kStoreNt;                   // the plain copy (the byte counters' yardstick)
+    int copy_store_policy = kStoreWriteThrough;         // the plain copy (the byte counters' yardstick)
     int one_shot = 1;                                   // kernels that keep nothing between tiles: one workgroup per tile instead of a loop
     int64_t one_shot_min_elems = int64_t(1) << 16;      // ... from this many elements up
-    int one_shot_store_policy = kStoreNt;               // cache policy of their fp32 stores
+    // cache policy of their fp32 stores.  Write-through: as fast as non-temporal from 2^27 elements up (the outer
+    // step alone loses 2-3 %) and well ahead below (dequantize set at 2^24: 10.5 against 17 us; pseudo-gradient at
+    // 2^26: 109 against 128 us)
+    int one_shot_store_policy = kStoreWriteThrough;
     int64_t small_max_elems = int64_t(1) << 14;         // uniform_8bit_quantize takes one launch of one workgroup up to this many elements (0: never)
 };
 Options g_opt;
@@ -272,8 +275,7 @@ void launch_dequant(int id, double bytes, int grid, hipStream_t st, float* out, 
     }
     if constexpr (!STATS) {
         if (one_shot(n)) {
-            // accumulating in place is the one case that does better with write-through stores (380 against 388 us at 2^28)
-            with_policy(ADD ? g_opt.f32_store_policy : g_opt.one_shot_store_policy, [&](auto P) {
+            with_policy(g_opt.one_shot_store_policy, [&](auto P) {
                 launch(id, bytes, dequant_kernel<ADD, false, true, true, DIV, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, out, lut,
                        codes, n, ws, divisor);
             });
