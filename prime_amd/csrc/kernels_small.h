@@ -10,7 +10,7 @@
 // Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
 
 constexpr int kSmallSlots = 4;
-constexpr int kSmallShift = 1;          // two LDS copies of each bin per row (any number gives the same integer sums)
+constexpr int kSmallShift = 2;          // four LDS copies of each bin per row (any number gives the same integer sums)
 static_assert(kThreads == 1024 && kBins == 256 && kSmallSlots == 4, "lane -> (row, bin) covers four rows of 256 bins; the tree is written for four rows");
 
 // One row's fixed-point histogram: a row adds at most 4 * kThreads + 3 elements, so no slot can
