@@ -20,7 +20,10 @@
 #endif
 
 constexpr int kThreads = PRIME_THREADS;   // wavefronts of 64
-constexpr int kBatchThreads = 512;       // workgroup of the one-tensor-per-workgroup kernel
+#ifndef PRIME_BATCH_THREADS
+#define PRIME_BATCH_THREADS 512
+#endif
+constexpr int kBatchThreads = PRIME_BATCH_THREADS;   // workgroup of the one-tensor-per-workgroup kernel
 constexpr int kWaves = kThreads / 64;
 constexpr int kBins = 256;               // compression.cpp:5
 constexpr int kZeroPoint = 128;          // compression.cpp:107
