@@ -388,9 +388,10 @@ struct ResidualHist {
 };
 static_assert(65535 / (kThreads * 4 * kUnroll) - 2 >= 1, "a slot must hold more than three rounds of a whole workgroup");
 
+template <int T = kThreads>          // T = lanes of the calling workgroup
 __device__ __forceinline__ void rhist_zero(ResidualHist& h, int shift) {
-    for (int i = threadIdx.x; i < (kBins << shift); i += kThreads) h.slot[i] = 0ull;
-    for (int i = threadIdx.x; i < kBins; i += kThreads) { h.wide_sum[i] = 0; h.wide_cnt[i] = 0ull; }
+    for (int i = threadIdx.x; i < (kBins << shift); i += T) h.slot[i] = 0ull;
+    for (int i = threadIdx.x; i < kBins; i += T) { h.wide_sum[i] = 0; h.wide_cnt[i] = 0ull; }
     if (threadIdx.x < 2 * kFarCopies) {
         h.far_sum[threadIdx.x / kFarCopies][threadIdx.x % kFarCopies] = 0.0;
         h.far_cnt[threadIdx.x / kFarCopies][threadIdx.x % kFarCopies] = 0u;
