@@ -993,7 +993,12 @@ def test_entry_points_replay_from_a_hip_graph(abi, oracle):
                 c, l, qp = g_abi.uniform(x)
                 c2, l2, qp2 = g_abi.ring_step(acc, c, l)
                 c3, l3, qp3 = g_abi.requantize_codes(c2, l2)
-                res.append((c, l, qp, c2, l2, qp2, c3, l3, qp3))
+                # the kernels that run as one workgroup per tile (from 65536 elements up)
+                d = torch.empty_like(x)
+                g_abi.dequant(d, l, c, add=False)
+                g_abi.dequant(d, l2, c2, add=True)
+                c4 = g_abi.quantize(x, 3.0e-4)
+                res.append((c, l, qp, c2, l2, qp2, c3, l3, qp3, d, c4))
             return res
 
         for x, acc in zip(xs, accs):
@@ -1015,7 +1020,7 @@ def test_entry_points_replay_from_a_hip_graph(abi, oracle):
         announce(f"graph replay {replay}")
         graph.replay()
         torch.cuda.synchronize()
-        for (c, l, qp, c2, l2, qp2, c3, l3, qp3), a, b, acc in zip(outs, hx, ha, accs):
+        for (c, l, qp, c2, l2, qp2, c3, l3, qp3, d, c4), a, b, acc in zip(outs, hx, ha, accs):
             q = abi.qparams(qp)
             assert q["scale"] == oracle.scale_exact(a)
             oc, _, _ = oracle.uniform_8bit_quantize(a, "given", scale=float(q["scale"]))
@@ -1027,6 +1032,10 @@ def test_entry_points_replay_from_a_hip_graph(abi, oracle):
             oc2, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q2["scale"]))
             assert q2["scale"] == oracle.scale_exact(want) and np.array_equal(c2.cpu().numpy(), oc2)
             _check_requantized(abi, oracle, c2, l2, c3, l3, qp3)
+            want_d = l.cpu().numpy()[oc]
+            oracle.index_add(want_d, l2.cpu().numpy(), oc2)
+            assert np.array_equal(d.cpu().numpy(), want_d)
+            assert np.array_equal(c4.cpu().numpy(), oracle.quantize_per_tensor_uint8(a, np.float32(3.0e-4), 128))
 
 
 @pytest.mark.parametrize("shift", [0, 1, 3])
