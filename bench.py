@@ -12,7 +12,7 @@ generator (seed = layer index) and are resident in HBM before the timed region.
 The single JSON line printed at the end carries
   value          algorithmic GB/s of quantize+lookup (9 bytes per element: x read twice, codes
                  written once) over the whole step, wall clock between two synchronisations, with
-                 the buckets dealt over three HIP streams (--streams); one_stream is the same work
+                 the buckets dealt over two HIP streams (--streams); one_stream is the same work
                  strictly bucket after bucket
   roofline       the dominant kernel (quantize + histogram, 5 bytes per element) on a 2^28-element
                  tensor (1 GiB, four times the last-level cache, so what it reads comes from HBM),
@@ -198,7 +198,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--streams", type=int, default=3,
+    ap.add_argument("--streams", type=int, default=2,
                     help="HIP streams the buckets are spread over in the timed region (1 = strictly one after another)")
     ap.add_argument("--legs", default="buckets,t28,ring,outer,diloco,configs,staging",
                     help="comma list of buckets (carries value), t28 (carries roofline and the per-operation rows), ring, "
@@ -694,7 +694,7 @@ def main() -> int:
         del x1, c1, o1
 
         # config 4: 1.25e9 elements in 42 buckets (29,761,904 each, the last 32 longer), N(0, 5e-4) with
-        # 0.01 % of entries at +-50 sigma; quantize + lookup over three streams, then dequantize
+        # 0.01 % of entries at +-50 sigma; quantize + lookup over --streams streams, then dequantize
         sizes4 = [29_761_904] * 41 + [29_761_904 + 32]
         xs4 = []
         for b, nb4 in enumerate(sizes4):

@@ -56,6 +56,8 @@ const char* prime_hip_last_error(void);
  * 256-lane workgroup per tile from 65536 elements up instead of a loop) and "one_shot_store_policy"
  * (cache policy of their stores), "small_max_elems" (uniform_8bit_quantize of at most this many
  * elements, and at most four rows of 4096, takes one launch of one workgroup; 0: never),
+ * "two_row_below_mi_elems" (the statistics and quantize kernels take tiles of two rows of 4096
+ * elements instead of four on tensors below this many Mi elements; 0: never),
  * "grid_cap" (upper bound on the workgroups of a looping kernel, for experiments; 0: none).
  * No option changes a result.  Returns 0 if the name is known.  The
  * options are process-wide and read at launch time: set them before work is enqueued, not
@@ -145,8 +147,8 @@ int prime_uniform_8bit_quantize_literal(const float* x, int64_t n, uint8_t* code
 
 /* Large buckets, pipelined: bucket i is quantized as prime_uniform_8bit_quantize would, on
  * streams[i % n_streams] with workspaces[i % n_streams], so that the statistics pass of one
- * bucket overlaps the quantize pass and the launch ramps of its neighbours (three streams
- * give +18 % on 205 MB buckets).  This is the loop over per-layer buckets of
+ * bucket overlaps the quantize pass and the launch ramps of its neighbours (two streams
+ * give +5 % on 205 MB buckets, more of them less).  This is the loop over per-layer buckets of
  * Diloco.sync_pseudo_gradient (src/zeroband/diloco.py:108-110) without the network in between.
  * xs, ns, codes, workspaces and streams are host arrays; luts is count x 256 on the device and
  * qparams_out (optional) count records.  The caller orders the streams against its own work. */

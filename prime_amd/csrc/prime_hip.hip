@@ -70,6 +70,10 @@ struct Options {
     // 2^26: 109 against 128 us)
     int one_shot_store_policy = kStoreWriteThrough;
     int64_t small_max_elems = int64_t(1) << 14;         // uniform_8bit_quantize takes one launch of one workgroup up to this many elements (0: never)
+    // the statistics and quantize kernels take tiles of two rows instead of four below this many elements (0: never):
+    // a 51 M-element bucket 74.5 against 78.4 us for the three launches, 2^26 elements 93.5 against 97.4;
+    // from 2^27 up four rows win (2^27: 196 against 207 us, 2^28: 378 against 404)
+    int64_t two_row_below_elems = int64_t(1) << 27;
 };
 Options g_opt;
 
@@ -115,6 +119,9 @@ int shot_grid(int64_t nvec) {
 // (a dispatch counts its work-items in 32 bits: beyond 2^34 elements the looping kernels take over)
 inline bool one_shot(int64_t n) { return g_opt.one_shot && n >= g_opt.one_shot_min_elems && n <= (int64_t(1) << 34); }
 
+// after_writer: the kernel before wrote the tensor (ring step, pseudo-gradient) instead of reading it: half the limit
+// (ring step of 2^26 elements: the quantize pass 51 us with four rows, 62 with two; of 2^25: 27.4 and 26.4)
+inline bool two_row_tiles(int64_t n, bool after_writer = false) { return (after_writer ? 2 * n : n) < g_opt.two_row_below_elems; }
 inline bool use_nt(int64_t n) { return (n >> 18) >= g_opt.nt_load_min_mib; }   // n floats = n / 2^18 MiB
 
 inline bool aligned_to(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
@@ -186,12 +193,13 @@ int run_stats_finalize(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
 // First stage only: returns the number of partials through *parts.
 int run_stats_partials(const float* x, int64_t n, Workspace* ws, hipStream_t st, int* parts) {
     const int grid = grid_for(n, true);
+    const bool two = two_row_tiles(n);
     if (!aligned_to(x, 16))
         launch(kIdStats, 4.0 * n, stats_kernel<false, false>, grid, kThreads, st, x, n, ws);
     else if (use_nt(n))
-        launch(kIdStats, 4.0 * n, stats_kernel<true, true>, grid, kThreads, st, x, n, ws);
+        launch(kIdStats, 4.0 * n, two ? stats_kernel<true, true, 2> : stats_kernel<true, true>, grid, kThreads, st, x, n, ws);
     else
-        launch(kIdStats, 4.0 * n, stats_kernel<true, false>, grid, kThreads, st, x, n, ws);
+        launch(kIdStats, 4.0 * n, two ? stats_kernel<true, false, 2> : stats_kernel<true, false>, grid, kThreads, st, x, n, ws);
     *parts = grid;
     return launch_check("stats_kernel");
 }
@@ -203,7 +211,7 @@ int run_stats(const float* x, int64_t n, prime_qparams* out, Workspace* ws, hipS
 }
 
 template <bool HIST, bool REVERSE, int POLICY>
-void launch_quantize_p(bool al, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
+void launch_quantize_p(bool al, bool two, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
                        prime_qparams* qp_out, int zp, uint8_t* codes, Workspace* ws) {
     const int id = HIST ? kIdQuantizeHist : kIdQuantize;
     int shift = 0;
@@ -211,15 +219,17 @@ void launch_quantize_p(bool al, int grid, hipStream_t st, const float* x, int64_
     if (!al)
         launch(id, 5.0 * n, quantize_kernel<false, false, HIST, REVERSE, kStorePlain>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
     else if ((n >> 18) >= g_opt.nt_second_min_mib)      // the quantize pass is always the last reader of the tensor
-        launch(id, 5.0 * n, quantize_kernel<true, true, HIST, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
+        launch(id, 5.0 * n, two ? quantize_kernel<true, true, HIST, REVERSE, POLICY, 2> : quantize_kernel<true, true, HIST, REVERSE, POLICY>,
+               grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
     else
-        launch(id, 5.0 * n, quantize_kernel<true, false, HIST, REVERSE, POLICY>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
+        launch(id, 5.0 * n, two ? quantize_kernel<true, false, HIST, REVERSE, POLICY, 2> : quantize_kernel<true, false, HIST, REVERSE, POLICY>,
+               grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift);
 }
 
 template <bool HIST>
-void launch_quantize_r(bool al, bool reverse, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
+void launch_quantize_r(bool al, bool two, bool reverse, int grid, hipStream_t st, const float* x, int64_t n, float scale, int stats_parts,
                        prime_qparams* qp_out, int zp, uint8_t* codes, Workspace* ws) {
-#define PRIME_Q(REV, POL) launch_quantize_p<HIST, REV, POL>(al, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws)
+#define PRIME_Q(REV, POL) launch_quantize_p<HIST, REV, POL>(al, two, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws)
     const int pol = g_opt.code_store_policy;
     if (reverse) {
         if (pol == kStoreNt) PRIME_Q(true, kStoreNt);
@@ -238,7 +248,7 @@ void launch_quantize_r(bool al, bool reverse, int grid, hipStream_t st, const fl
 // number of histogram partials written.  second_pass: the tensor has just been streamed by the
 // kernel before this one, so walk it from its end (what the last-level cache still holds comes first).
 int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_qparams* qp_out, int zp, uint8_t* codes,
-                 Workspace* ws, bool hist, hipStream_t st, int* grid_out, bool second_pass = false) {
+                 Workspace* ws, bool hist, hipStream_t st, int* grid_out, bool second_pass = false, bool after_writer = false) {
     if (hist && zp != kZeroPoint) return fail(PRIME_EINVAL, "the fused quantize + lookup pass has zero point 128");
     const int grid = grid_for(n, true);
     const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
@@ -250,8 +260,9 @@ int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_
         return launch_check("quantize_shot_kernel");
     }
     const bool rev = second_pass && g_opt.reverse_second_pass;
-    if (!hist) launch_quantize_r<false>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
-    else launch_quantize_r<true>(al, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    const bool two = two_row_tiles(n, after_writer);
+    if (!hist) launch_quantize_r<false>(al, two, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
+    else launch_quantize_r<true>(al, two, rev, grid, st, x, n, scale, stats_parts, qp_out, zp, codes, ws);
     if (grid_out) *grid_out = grid;
     return launch_check("quantize_kernel");
 }
@@ -409,6 +420,9 @@ int prime_hip_set_option(const char* name, int value) {
     } else if (!strcmp(name, "small_max_elems")) {
         if (value < 0) return fail(PRIME_EINVAL, "small_max_elems must be >= 0 (0: off)");
         g_opt.small_max_elems = value;
+    } else if (!strcmp(name, "two_row_below_mi_elems")) {
+        if (value < 0 || value > 8192) return fail(PRIME_EINVAL, "two_row_below_mi_elems must be in [0, 8192] (0: off)");
+        g_opt.two_row_below_elems = static_cast<int64_t>(value) << 20;
     } else if (!strcmp(name, "reverse_second_pass")) {
         g_opt.reverse_second_pass = value != 0;
     } else if (!strcmp(name, "nt_load_min_mib")) {
@@ -436,6 +450,7 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "one_shot")) *value = g_opt.one_shot;
     else if (!strcmp(name, "one_shot_store_policy")) *value = g_opt.one_shot_store_policy;
     else if (!strcmp(name, "small_max_elems")) *value = static_cast<int>(g_opt.small_max_elems);
+    else if (!strcmp(name, "two_row_below_mi_elems")) *value = static_cast<int>(g_opt.two_row_below_elems >> 20);
     else if (!strcmp(name, "f32_store_policy")) *value = g_opt.f32_store_policy;
     else if (!strcmp(name, "f32_reread_store_policy")) *value = g_opt.f32_reread_store_policy;
     else if (!strcmp(name, "copy_store_policy")) *value = g_opt.copy_store_policy;
@@ -732,7 +747,7 @@ int ring_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_
     } else {
         if (int rc = run_dequant<ADD, true>(chunk, lut_in, codes_in, n, w, st, &grid)) return rc;
     }
-    if (int rc = run_quantize(chunk, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid, true)) return rc;
+    if (int rc = run_quantize(chunk, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid, true, true)) return rc;
     return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
 }
 
@@ -847,7 +862,7 @@ int prime_ring_first_touch(const float* outer, const float* inner, int64_t n, fl
                    no_codes, no_lut, 1.0f, grad_out, w);
     }
     if (int rc = launch_check("first_touch_kernel")) return rc;
-    if (int rc = run_quantize(grad_out, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid, true)) return rc;
+    if (int rc = run_quantize(grad_out, n, 0.0f, grid, qparams_out, kZeroPoint, codes_out, w, true, st, &grid, true, true)) return rc;
     return run_lut_finalize(w, grid, lut_out, kBins, nullptr, st);
 }
 

@@ -516,7 +516,7 @@ outer_sgd_nesterov_codes_ = torch.ops.prime.outer_sgd_nesterov_codes_
 # Pipelined quantization of many large buckets (the per-layer loop of
 # Diloco.sync_pseudo_gradient, src/zeroband/diloco.py:108-110, without the network in between).
 
-PIPELINE_STREAMS = 3     # measured best on MI355X for 205 MB buckets (1: 5.7, 2: 6.3, 3: 6.8, 4: 6.0 TB/s)
+PIPELINE_STREAMS = 2     # measured best on MI355X for 205 MB buckets (1: 6.14, 2: 6.46, 3: 6.34, 4: 6.23, 6: 6.28 TB/s)
 _side_streams: Dict[int, list] = {}
 
 

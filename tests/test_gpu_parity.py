@@ -454,7 +454,7 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
                                            ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20)),
                                            ("code_store_policy", (0, 2, 16)), ("f32_reread_store_policy", (0, 2, 16)),
                                            ("reverse_second_pass", (0, 1)), ("one_shot", (0, 1)),
-                                           ("one_shot_store_policy", (0, 2, 16))])
+                                           ("one_shot_store_policy", (0, 2, 16)), ("two_row_below_mi_elems", (0, 128))])
 def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle, option, values):
     # the options change scheduling and cache hints only: codes, scale and lookup must not move,
     # on ordinary data, on a tensor crowded into a few codes, and through a ring step
