@@ -140,3 +140,18 @@ def test_ring_over_a_real_gloo_group_one_process_per_rank(dev, oracle, tmp_path,
         err_old = np.linalg.norm(cpu[r] - exact)
         assert abs(err_new - err_old) / math.sqrt(n) < 0.5            # tests/test_c/test_collectives.py:57
         assert abs(err_new - err_old) / math.sqrt(n) < 0.02
+
+
+@pytest.mark.parametrize("W", [2, 4])
+def test_all_reduce_timing_script_with_uint8_compression(dev, W):
+    # scripts/all_reduce.py of the reference with compression "uint8": rand(1, N) per rank, the ranks share
+    # the GPU; the sum of W uniform(0, 1) tensors after 8-bit hops stays within a few quantization steps
+    from tests.test_host import _run_ranks
+
+    announce(f"all_reduce_bench uint8 W={W}")
+    line = _run_ranks(["--size_model", "1000003", "--n_iters", "2", "--compression", "uint8", "--check"], world=W)
+    assert line["ranks"] == W and line["compression"] == "uint8"
+    assert line["size_model"] == 1000003 - 1000003 % (2 * W)          # src/zeroband/collectives.py:83
+    # one hop's step is 6 * rms / 256 of what it carries; W - 1 accumulations and two more round trips
+    assert line["rms_error"] < (W + 1) * 6.0 * line["rms_of_sum"] / 256
+    assert line["MBps"] > 0

@@ -163,3 +163,44 @@ def test_short_rounding_sequence_equals_roundf_on_every_float_in_its_range(tmp_p
     res = subprocess.run([str(exe)], capture_output=True, text=True)
     assert res.returncode == 0, res.stdout
     assert "checked 2285502466 mismatches 0" in res.stdout
+
+
+def _run_ranks(args, world, timeout=150):
+    """One child process per rank of `python -m prime_amd.all_reduce_bench`, rendezvous on localhost."""
+    import json
+    import os
+    import socket
+    import subprocess
+    import sys
+
+    with socket.socket() as sock:
+        sock.bind(("127.0.0.1", 0))
+        port = sock.getsockname()[1]
+    root = Path(__file__).resolve().parents[1]
+    procs = []
+    for r in range(world):
+        env = dict(os.environ, PYTHONPATH=str(root), RANK=str(r), WORLD_SIZE=str(world), MASTER_ADDR="127.0.0.1",
+                   MASTER_PORT=str(port), GLOO_SOCKET_IFNAME="lo")
+        procs.append(subprocess.Popen([sys.executable, "-u", "-m", "prime_amd.all_reduce_bench", *args], cwd=str(root), env=env,
+                                      stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+    outs = []
+    try:
+        for pr in procs:
+            out, _ = pr.communicate(timeout=timeout)
+            outs.append(out)
+    finally:
+        for pr in procs:
+            if pr.poll() is None:
+                pr.kill()
+    for r, pr in enumerate(procs):
+        assert pr.returncode == 0, f"rank {r} failed:\n{outs[r][-3000:]}"
+    lines = [ln for ln in outs[0].splitlines() if ln.startswith("{")]
+    assert len(lines) == 1, outs[0][-2000:]
+    return json.loads(lines[0])
+
+
+def test_all_reduce_timing_script_without_compression_on_two_host_ranks():
+    # the reference's scripts/all_reduce.py with compression "no": the tensor stays on the host
+    line = _run_ranks(["--size_model", "100001", "--n_iters", "2", "--compression", "no", "--check"], world=2)
+    assert line["ranks"] == 2 and line["size_model"] == 100001 and line["compression"] == "no"
+    assert line["MBps"] > 0 and line["rms_error"] < 1e-6
