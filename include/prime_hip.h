@@ -58,6 +58,8 @@ const char* prime_hip_last_error(void);
  * elements, and at most four rows of 4096, takes one launch of one workgroup; 0: never),
  * "two_row_below_mi_elems" (the statistics and quantize kernels take tiles of two rows of 4096
  * elements instead of four on tensors below this many Mi elements; 0: never),
+ * "set_four_rows_max_mi_elems" (the one-workgroup-per-tile dequantize set takes tiles of four rows of
+ * 1024 elements instead of two on tensors of at most this many Mi elements; 0: never),
  * "grid_cap" (upper bound on the workgroups of a looping kernel, for experiments; 0: none).
  * No option changes a result.  Returns 0 if the name is known.  The
  * options are process-wide and read at launch time: set them before work is enqueued, not

@@ -31,7 +31,10 @@ constexpr int kMaxGrid = 2048;           // per-workgroup partial slots in the w
 constexpr int kUnroll = PRIME_UNROLL;
 constexpr int kDivUnroll = PRIME_UNROLL > 2 ? 2 : PRIME_UNROLL;   // vectors per step in the kernels that divide
 constexpr int kShotThreads = 256;        // workgroup of a one-tile-per-workgroup launch
-constexpr int kShotUnroll = 2;           // rows of its tile
+#ifndef PRIME_SHOT_UNROLL
+#define PRIME_SHOT_UNROLL 2
+#endif
+constexpr int kShotUnroll = PRIME_SHOT_UNROLL;   // rows of its tile
 // wavefronts per SIMD the streaming kernels are compiled for (4 SIMDs per compute unit, at
 // most 8 wavefronts each): bounds their register use so that PRIME_BLOCKS_PER_CU workgroups fit
 constexpr int kWavesPerSimd = (PRIME_THREADS / 64) * PRIME_BLOCKS_PER_CU / 4 > 8 ? 8

@@ -225,7 +225,9 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_remap_kernel(con
 // POLICY is the cache policy of the fp32 stores.
 // ONESHOT (never with STATS, whose partials are per workgroup of a small grid): one workgroup of
 // kShotThreads lanes per tile instead of a loop.
-template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT = false>
+// SHOT_ROWS: rows of a ONESHOT workgroup's tile.  The plain set does best with four up to 2^25 elements (2^23: 6.2
+// against 7.5 us, 2^24: 13.1 against 15.4 us) and with two beyond (2^26: 54 against 58 us, 2^28: 211 against 242 us).
+template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT = false, int SHOT_ROWS = kShotUnroll>
 __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd)
 void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
                     float divisor) {
@@ -233,10 +235,18 @@ void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, cons
     using M = Mem<ALIGNED, NT>;
     constexpr int T = ONESHOT ? kShotThreads : kThreads;
     __shared__ float s_lut[kBins];
-    for (int b = threadIdx.x; b < kBins; b += T) s_lut[b] = lut[b];
-    __syncthreads();
+    // The table goes to LDS once per workgroup, first thing.  A workgroup of the plain set that lives
+    // for one tile issues the tile's loads before that, so that the table's trip to L2 runs beside the
+    // codes' trip to memory instead of in front of it (2^28 elements: 210 instead of 233 us; with the
+    // accumulator's loads in flight as well the order makes no difference or costs 1 %).
+    constexpr bool kLateFill = ONESHOT && !ADD;
+    auto fill_lut = [&] {
+        for (int b = threadIdx.x; b < kBins; b += T) s_lut[b] = lut[b];
+        __syncthreads();
+    };
+    if (!kLateFill) fill_lut();
     const int64_t nvec = n >> 2;
-    constexpr int U = ONESHOT ? kShotUnroll : DIV ? kDivUnroll : kUnroll;
+    constexpr int U = ONESHOT ? SHOT_ROWS : DIV ? kDivUnroll : kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
     walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
@@ -251,6 +261,7 @@ void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, cons
             c[j] = ok ? M::ldu32(codes, i) : 0u;
             if (ADD) a[j] = ok ? M::ldf4(out, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
+        if (kLateFill) fill_lut();        // every workgroup of such a launch has a tile: the barrier is uniform
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;

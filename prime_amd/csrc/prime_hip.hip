@@ -74,6 +74,7 @@ struct Options {
     // a 51 M-element bucket 74.5 against 78.4 us for the three launches, 2^26 elements 93.5 against 97.4;
     // from 2^27 up four rows win (2^27: 196 against 207 us, 2^28: 378 against 404)
     int64_t two_row_below_elems = int64_t(1) << 27;
+    int64_t set_four_rows_max_elems = int64_t(1) << 25;  // the one-workgroup-per-tile dequantize set takes tiles of four rows up to this many elements (0: never)
 };
 Options g_opt;
 
@@ -112,8 +113,8 @@ int grid_for(int64_t n, bool reads = false) {
 }
 
 // One workgroup per tile for a kernel launched ONESHOT.
-int shot_grid(int64_t nvec) {
-    const int64_t tile = static_cast<int64_t>(kShotThreads) * kShotUnroll;
+int shot_grid(int64_t nvec, int rows = kShotUnroll) {
+    const int64_t tile = static_cast<int64_t>(kShotThreads) * rows;
     return static_cast<int>((nvec + tile - 1) / tile);
 }
 // (a dispatch counts its work-items in 32 bits: beyond 2^34 elements the looping kernels take over)
@@ -287,8 +288,12 @@ void launch_dequant(int id, double bytes, int grid, hipStream_t st, float* out, 
     if constexpr (!STATS) {
         if (one_shot(n)) {
             with_policy(g_opt.one_shot_store_policy, [&](auto P) {
-                launch(id, bytes, dequant_kernel<ADD, false, true, true, DIV, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, out, lut,
-                       codes, n, ws, divisor);
+                if (!ADD && n <= g_opt.set_four_rows_max_elems)
+                    launch(id, bytes, dequant_kernel<ADD, false, true, true, DIV, decltype(P)::value, true, 4>, shot_grid(n >> 2, 4), kShotThreads, st,
+                           out, lut, codes, n, ws, divisor);
+                else
+                    launch(id, bytes, dequant_kernel<ADD, false, true, true, DIV, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, out, lut,
+                           codes, n, ws, divisor);
             });
             return;
         }
@@ -423,6 +428,9 @@ int prime_hip_set_option(const char* name, int value) {
     } else if (!strcmp(name, "two_row_below_mi_elems")) {
         if (value < 0 || value > 8192) return fail(PRIME_EINVAL, "two_row_below_mi_elems must be in [0, 8192] (0: off)");
         g_opt.two_row_below_elems = static_cast<int64_t>(value) << 20;
+    } else if (!strcmp(name, "set_four_rows_max_mi_elems")) {
+        if (value < 0 || value > 8192) return fail(PRIME_EINVAL, "set_four_rows_max_mi_elems must be in [0, 8192] (0: off)");
+        g_opt.set_four_rows_max_elems = static_cast<int64_t>(value) << 20;
     } else if (!strcmp(name, "reverse_second_pass")) {
         g_opt.reverse_second_pass = value != 0;
     } else if (!strcmp(name, "nt_load_min_mib")) {
@@ -451,6 +459,7 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "one_shot_store_policy")) *value = g_opt.one_shot_store_policy;
     else if (!strcmp(name, "small_max_elems")) *value = static_cast<int>(g_opt.small_max_elems);
     else if (!strcmp(name, "two_row_below_mi_elems")) *value = static_cast<int>(g_opt.two_row_below_elems >> 20);
+    else if (!strcmp(name, "set_four_rows_max_mi_elems")) *value = static_cast<int>(g_opt.set_four_rows_max_elems >> 20);
     else if (!strcmp(name, "f32_store_policy")) *value = g_opt.f32_store_policy;
     else if (!strcmp(name, "f32_reread_store_policy")) *value = g_opt.f32_reread_store_policy;
     else if (!strcmp(name, "copy_store_policy")) *value = g_opt.copy_store_policy;

@@ -454,7 +454,8 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
                                            ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20)),
                                            ("code_store_policy", (0, 2, 16)), ("f32_reread_store_policy", (0, 2, 16)),
                                            ("reverse_second_pass", (0, 1)), ("one_shot", (0, 1)),
-                                           ("one_shot_store_policy", (0, 2, 16)), ("two_row_below_mi_elems", (0, 128))])
+                                           ("one_shot_store_policy", (0, 2, 16)), ("two_row_below_mi_elems", (0, 128)),
+                                           ("set_four_rows_max_mi_elems", (0, 32))])
 def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle, option, values):
     # the options change scheduling and cache hints only: codes, scale and lookup must not move,
     # on ordinary data, on a tensor crowded into a few codes, and through a ring step
@@ -643,6 +644,15 @@ def test_one_workgroup_per_tile_equals_the_looping_launch(abi, oracle, n):
         _lib.profile_begin()
         shot = run_all()
         prof = _lib.profile_end()
+        rows = _lib.get_option("set_four_rows_max_mi_elems")
+        try:                                         # the set takes four-row tiles at these sizes: its two-row variant as well
+            _lib.set_option("set_four_rows_max_mi_elems", 0)
+            two_rows = torch.empty(n, device=abi.dev)
+            abi.dequant(two_rows, lt, ct, add=False)
+            torch.cuda.synchronize()
+        finally:
+            _lib.set_option("set_four_rows_max_mi_elems", rows)
+        assert rows == 32 and torch.equal(two_rows.view(torch.int32), shot["set"].view(torch.int32))
         _lib.set_option("one_shot", 0)
         loop = run_all()
     finally:
