@@ -236,8 +236,10 @@ int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n,
  *                   rank's own chunks, :155-159; 1.0f skips the division)
  *   (codes_out, lut_out) = uniform_8bit_quantize(grad_out)                  (:138 / :162)
  * codes_in == NULL is the quantization of a chunk that is sent before anything is received
- * (steps 1 and 2).  17 bytes per element against 12 + 9 for prime_pseudo_gradient_f32 followed
- * by prime_uniform_8bit_quantize, and 18 against 12 + 14 with a received message. */
+ * (steps 1 and 2): prime_pseudo_gradient_f32 followed by prime_uniform_8bit_quantize, which on
+ * this device beat a pass that takes the statistics along (12 + 9 bytes per element in 197 us
+ * against 17 in 211 us at 2^26 elements).  With a received message the fused pass moves 18 bytes
+ * per element against 12 + 14 and is 15 % faster. */
 int prime_ring_first_touch(const float* outer, const float* inner, int64_t n, float world_size,
                            const uint8_t* codes_in, const float* lut_in, float divisor, float* grad_out,
                            uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out, void* ws,

@@ -86,7 +86,9 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
 // otherwise read it back.  With CODES the received message is accumulated,
 // acc = grad + lut[codes] (collectives.cpp:128-133), and with a divisor other than 1 the sum is
 // divided (ReduceOp::AVG, :155-159).  The fp64 sum and sum of squares of what is stored are the
-// statistics of the quantization that follows.  12 bytes per element, 13 with codes.
+// statistics of the quantization that follows.  12 bytes per element, 13 with codes.  (Only the
+// variant with CODES is launched: without a message the pseudo-gradient as one workgroup per tile
+// followed by the statistics kernel is faster than this loop.)
 template <bool CODES, bool ALIGNED, bool NT, int POLICY>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(const float* __restrict__ outer,
                                                                                const float* __restrict__ inner, int64_t n,
