@@ -66,8 +66,7 @@ struct Options {
     int one_shot = 1;                                   // kernels that keep nothing between tiles: one workgroup per tile instead of a loop
     int64_t one_shot_min_elems = int64_t(1) << 16;      // ... from this many elements up
     // cache policy of their fp32 stores.  Write-through: as fast as non-temporal from 2^27 elements up (the outer
-    // step alone loses 2-3 %) and well ahead below (dequantize set at 2^24: 10.5 against 17 us; pseudo-gradient at
-    // 2^26: 109 against 128 us)
+    // step alone loses 2-3 %) and well ahead below (pseudo-gradient at 2^26: 109 against 128 us)
     int one_shot_store_policy = kStoreWriteThrough;
     int64_t small_max_elems = int64_t(1) << 14;         // uniform_8bit_quantize takes one launch of one workgroup up to this many elements (0: never)
     // the statistics and quantize kernels take tiles of two rows instead of four below this many elements (0: never):
