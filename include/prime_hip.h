@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define PRIME_HIP_ABI_VERSION 1
+#define PRIME_HIP_ABI_VERSION 2
 
 #define PRIME_EINVAL (-1)   /* null pointer, negative size, bad n_bins ... */
 #define PRIME_EWORKSPACE (-2) /* workspace missing, too small or not initialised */
@@ -60,8 +60,15 @@ const char* prime_hip_last_error(void);
  * elements instead of four on tensors below this many Mi elements; 0: never),
  * "set_four_rows_max_mi_elems" (the one-workgroup-per-tile dequantize set takes tiles of four rows of
  * 1024 elements instead of two on tensors of at most this many Mi elements; 0: never),
- * "grid_cap" (upper bound on the workgroups of a looping kernel, for experiments; 0: none).
- * No option changes a result.  Returns 0 if the name is known.  The
+ * "segment_blocks_per_cu" (workgroups per compute unit that the quantize pass of a segmented launch
+ * shares out among its tensors), "grid_cap" (upper bound on the workgroups of a looping kernel, for
+ * experiments; 0: none).
+ * Cache policies, load hints, the one-workgroup-per-tile and one-launch variants, the number of LDS
+ * copies and segment_blocks_per_cu never change a result.  The options that change the number of
+ * workgroups of the statistics pass or its tile shape (blocks_per_cu, grid_cap, large_read_*,
+ * two_row_below_mi_elems) change the order in which the fp64 sums are added: codes and scale have been
+ * equal on all tested data, but a sum may move in its last bit and, rarely, a scale with it.
+ * Returns 0 if the name is known.  The
  * options are process-wide and read at launch time: set them before work is enqueued, not
  * concurrently with it. */
 int prime_hip_set_option(const char* name, int value);
@@ -214,6 +221,44 @@ int prime_requantize_codes(const uint8_t* codes_in, const float* lut_in, int64_t
 int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_t n,
                            uint8_t* codes_out, float* lut_out, prime_qparams* qparams_out,
                            void* ws, prime_stream_t stream);
+
+/* ---- segmented launches: many mid-size tensors, three kernel launches in all ----
+ * The ring all-reduce of one layer bucket cuts it into 2 * world_size chunks (collectives.cpp:89-90)
+ * and Diloco.sync_pseudo_gradient visits one bucket after the other (src/zeroband/diloco.py:108-110),
+ * so the tensors this path really sees are chunks of 1-4 M elements, where three kernel boundaries
+ * per tensor cost more than the data.  These entry points take `count` tensors as host arrays of
+ * device pointers and sizes, give every tensor as many workgroups as its size wants, and run the
+ * whole set in three launches per group of 64 tensors: statistics (or a ring step's first pass),
+ * quantize + histogram, lookup tables.  Tensor i's results (codes[i], luts + 256 * i,
+ * qparams_out[i]) equal what the one-tensor entry point returns for it, bit for bit (the lookup
+ * entries of a tensor whose 1 / scale is zero or not finite, and bins 0 / 255 of a tensor with
+ * values beyond 628 bins in several workgroups, may differ in their last bit: they are sums of
+ * fp64 values in an order that depends on the launch).  Tensors that are empty or not aligned for
+ * vector access (tensor 16 bytes, codes 4) take the one-tensor path inside the call.  The pointer
+ * and size arrays are host memory and are read before the call returns; luts is count x 256 floats
+ * and qparams_out (optional) count records on the device.  One workspace, as for the calls above. */
+int prime_uniform_8bit_quantize_segmented(const float* const* xs, const int64_t* ns, int64_t count,
+                                          uint8_t* const* codes, float* luts, prime_qparams* qparams_out,
+                                          void* ws, prime_stream_t stream);
+
+/* prime_ring_reduce_step on count chunks: what the world_size ranks of a lock-stepped ring do in one
+ * step of the reduce-scatter (collectives.cpp:124-138), or one rank on the chunks of several buckets. */
+int prime_ring_reduce_step_segmented(float* const* accs, const uint8_t* const* codes_in,
+                                     const float* const* luts_in, const int64_t* ns, int64_t count,
+                                     uint8_t* const* codes_out, float* luts_out, prime_qparams* qparams_out,
+                                     void* ws, prime_stream_t stream);
+
+/* prime_ring_reduce_div_step on count chunks, one divisor for all (collectives.cpp:124-133,155-162). */
+int prime_ring_reduce_div_step_segmented(float* const* accs, const uint8_t* const* codes_in,
+                                         const float* const* luts_in, const int64_t* ns, int64_t count,
+                                         float divisor, uint8_t* const* codes_out, float* luts_out,
+                                         prime_qparams* qparams_out, void* ws, prime_stream_t stream);
+
+/* prime_ring_gather_step on count chunks (collectives.cpp:200-215). */
+int prime_ring_gather_step_segmented(float* const* chunks, const uint8_t* const* codes_in,
+                                     const float* const* luts_in, const int64_t* ns, int64_t count,
+                                     uint8_t* const* codes_out, float* luts_out, prime_qparams* qparams_out,
+                                     void* ws, prime_stream_t stream);
 
 /* x[i] = x[i] / divisor in place: chunk.div_(world_size) of the ring's ReduceOp::AVG,
  * collectives.cpp:155-159. */

@@ -10,7 +10,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libprime_hip.so"
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class QParams(ctypes.Structure):
@@ -70,6 +70,10 @@ SIGNATURES = {
     "prime_ring_reduce_step": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "prime_ring_gather_step": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "prime_ring_reduce_div_step": (ctypes.c_int, [_vp, _vp, _vp, _i64, _f32, _vp, _vp, _vp, _vp, _vp]),
+    "prime_uniform_8bit_quantize_segmented": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "prime_ring_reduce_step_segmented": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "prime_ring_reduce_div_step_segmented": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _f32, _vp, _vp, _vp, _vp, _vp]),
+    "prime_ring_gather_step_segmented": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp]),
     "prime_div_f32": (ctypes.c_int, [_vp, _i64, _f32, _vp]),
     "prime_pseudo_gradient_f32": (ctypes.c_int, [_vp, _vp, _i64, _f32, _vp, _vp]),
     "prime_ring_first_touch": (ctypes.c_int, [_vp, _vp, _i64, _f32, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -134,8 +138,9 @@ def profile_begin() -> None:
 
 def profile_end() -> dict:
     """{kernel name: {"launches", "total_ms", "algo_bytes"}} since profile_begin (synchronises)."""
-    buf = (KernelTime * 32)()
+    cap = 64
+    buf = (KernelTime * cap)()
     n = ctypes.c_int()
-    check(load().prime_hip_profile_end(buf, 32, ctypes.byref(n)), "profile_end")
+    check(load().prime_hip_profile_end(buf, cap, ctypes.byref(n)), "profile_end")
     return {buf[i].name.decode(): {"launches": buf[i].launches, "total_ms": buf[i].total_ms,
-                                   "algo_bytes": buf[i].algo_bytes} for i in range(min(n.value, 32))}
+                                   "algo_bytes": buf[i].algo_bytes} for i in range(min(n.value, cap))}

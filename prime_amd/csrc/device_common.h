@@ -43,9 +43,39 @@ constexpr int kFinalThreads = 1024;      // workgroup size of the second-stage k
 constexpr int kLutBinsPerBlock = 4;      // bins one second-stage workgroup reduces (64 bytes per partial)
 constexpr int64_t kMaxElems = int64_t(1) << 40;   // per-workgroup counts are 32-bit
 
+constexpr int kSegMax = 64;              // tensors of one segmented launch (their descriptors travel as kernel arguments)
+
+// One bin of a workgroup's histogram partial, 16 bytes, in one of two forms.  BinAcc: the fp64 sum
+// of the bin's elements and their number.  BinPart (the fixed-point histogram of the fused quantize
+// pass): the integer sum of the elements' residuals from the centre of the bin, in units of 2^-22 of
+// a bin width, and their number.  Integer partials add up to the same totals whichever workgroup saw
+// which element, so the table built from them does not depend on how the tensor was dealt out.
 struct BinAcc {
     double sum;
     unsigned long long cnt;
+};
+struct BinPart {
+    long long units;
+    unsigned long long cnt;
+};
+// The elements of a workgroup that lie beyond the range of the fixed-point residual (they all have
+// code 0 or 255): their number and the fp64 sum of their values, per side.
+struct FarPart {
+    double sum[2];
+    unsigned long long cnt[2];
+};
+// Which of the two forms the partials of the launch before have, and the 1 / scale their residuals refer to.
+enum { kHistFp = 0, kHistFixed = 1 };
+struct HistInfo {
+    float inv;
+    int mode;
+};
+
+// What one tensor of a segmented launch leaves between the kernels.
+struct SegRecord {
+    prime_qparams qp;
+    HistInfo info;
+    int pad[2];
 };
 
 // Every kernel stores its per-workgroup partial results here with plain stores; the kernel
@@ -54,12 +84,22 @@ struct Workspace {
     prime_qparams qp;                    // scale of the tensor in flight
     uint32_t code_map[kBins / 4];        // old code -> new code of a requantization in the code domain
     unsigned long long code_total[kBins];   // population of each code over the whole tensor
+    HistInfo hist_info;                  // form of the histogram partials below
+    unsigned tile_counter;               // next tile of the part of a pass that is dealt out on demand
+    unsigned pad;
     double part_sum[kMaxGrid];
     double part_sq[kMaxGrid];
-    union {
+    FarPart far[kMaxGrid];
+    union alignas(16) {
         BinAcc hist[kMaxGrid][kBins];    // 4 KiB per workgroup
+        BinPart hist_fixed[kMaxGrid][kBins];
         uint32_t code_cnt[kMaxGrid][kBins];   // per-workgroup populations of each code value
     };
+    // segmented launches: per tensor the record and the statistics partials of as many workgroups as
+    // the one-tensor entry point would launch for it; the histogram partials share the rows above
+    SegRecord seg[kSegMax];
+    double seg_part_sum[kSegMax][kMaxGrid];
+    double seg_part_sq[kSegMax][kMaxGrid];
 };
 
 typedef float f4a __attribute__((ext_vector_type(4)));   // 16-byte aligned
@@ -197,7 +237,7 @@ __device__ __forceinline__ void finalize_from_norm(float norm, double sum, doubl
 
 // Workgroup reduction of (sum, sumsq) in a fixed order; the workgroup's partial goes to the
 // workspace for stats_finalize_kernel.
-__device__ __forceinline__ void block_stats_store(double s, double q, Workspace* ws, int slot) {
+__device__ __forceinline__ void block_stats_store(double s, double q, double* part_sum, double* part_sq, int slot) {
     __shared__ double sh_s[kWaves];
     __shared__ double sh_q[kWaves];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -209,9 +249,12 @@ __device__ __forceinline__ void block_stats_store(double s, double q, Workspace*
         double S = sh_s[0], Q = sh_q[0];
 #pragma unroll
         for (int w = 1; w < kWaves; ++w) { S += sh_s[w]; Q += sh_q[w]; }
-        ws->part_sum[slot] = S;
-        ws->part_sq[slot] = Q;
+        part_sum[slot] = S;
+        part_sq[slot] = Q;
     }
+}
+__device__ __forceinline__ void block_stats_store(double s, double q, Workspace* ws, int slot) {
+    block_stats_store(s, q, ws->part_sum, ws->part_sq, slot);
 }
 
 // True when the tensor's spread is below about two bins: std < 0.05 rms, from the fp64 sums.
@@ -225,12 +268,13 @@ __device__ __forceinline__ bool narrow_distribution(double sum, double sumsq, in
 
 // Second stage of the statistics run by a whole workgroup of the consuming kernel: every
 // workgroup adds the same partials in the same order, so all of them derive the same scale
-// bit for bit and no separate launch is needed.  Returns 1 / scale; workgroup 0 publishes
-// the record.
+// bit for bit and no separate launch is needed.  Returns 1 / scale; the workgroup with `publish`
+// set stores the record to `rec` and, if given, `out`.
 // The reduction itself: lane i brings the partial sums of workgroup i (and of i + THREADS, ...)
 // already added up as a (sum) and b (sum of squares).
 template <int THREADS>
-__device__ __forceinline__ float block_scale_reduce(double a, double b, Workspace* ws, int64_t n, prime_qparams* out, int* hot_base) {
+__device__ __forceinline__ float block_scale_reduce(double a, double b, int64_t n, bool publish, prime_qparams* rec, prime_qparams* out,
+                                                    int* hot_base) {
     __shared__ double sh_s[THREADS / 64];
     __shared__ double sh_q[THREADS / 64];
     __shared__ float sh_inv;
@@ -249,8 +293,8 @@ __device__ __forceinline__ float block_scale_reduce(double a, double b, Workspac
         sh_inv = qp.inv_scale;
         sh_hot = narrow_distribution(S, Q, n) ? quantize_code(static_cast<float>(S / static_cast<double>(n)), qp.inv_scale, kZeroPoint) - 1
                                               : INT_MIN;
-        if (blockIdx.x == 0) {
-            ws->qp = qp;
+        if (publish) {
+            *rec = qp;
             if (out) *out = qp;
         }
     }
@@ -260,20 +304,26 @@ __device__ __forceinline__ float block_scale_reduce(double a, double b, Workspac
 }
 
 template <int THREADS>
-__device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
-                                                           int* hot_base = nullptr) {
+__device__ __forceinline__ float block_scale_from_partials(const double* part_sum, const double* part_sq, int nparts, int64_t n,
+                                                           bool publish, prime_qparams* rec, prime_qparams* out, int* hot_base = nullptr) {
     constexpr int kIters = (kMaxGrid + THREADS - 1) / THREADS;
     double ps[kIters], pq[kIters];
 #pragma unroll
     for (int k = 0; k < kIters; ++k) {       // all loads in flight at once
         const int i = threadIdx.x + k * THREADS;
-        ps[k] = i < nparts ? ws->part_sum[i] : 0.0;
-        pq[k] = i < nparts ? ws->part_sq[i] : 0.0;
+        ps[k] = i < nparts ? part_sum[i] : 0.0;
+        pq[k] = i < nparts ? part_sq[i] : 0.0;
     }
     double a = 0.0, b = 0.0;
 #pragma unroll
     for (int k = 0; k < kIters; ++k) { a += ps[k]; b += pq[k]; }
-    return block_scale_reduce<THREADS>(a, b, ws, n, out, hot_base);
+    return block_scale_reduce<THREADS>(a, b, n, publish, rec, out, hot_base);
+}
+
+template <int THREADS>
+__device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
+                                                           int* hot_base = nullptr) {
+    return block_scale_from_partials<THREADS>(ws->part_sum, ws->part_sq, nparts, n, blockIdx.x == 0, &ws->qp, out, hot_base);
 }
 
 // Work distribution of the streaming kernels.  The tensor is cut into rows of kThreads
@@ -315,15 +365,20 @@ __device__ __forceinline__ void sweep_tiles(int64_t nvec, Body&& body) {
 // elements a plain copy takes 322 us instead of 358 us, 4 bytes in / 16 bytes out 204 us instead of
 // 240 us (256 lanes, two rows).  Otherwise the looping sweep above (T must be kThreads).
 template <int T, int U, bool ONESHOT, typename Body>
-__device__ __forceinline__ void walk_tiles(int64_t nvec, Body&& body) {
+__device__ __forceinline__ void walk_tiles_of(int64_t nvec, int64_t slot, int64_t G, Body&& body) {
     if constexpr (ONESHOT) {
-        const int64_t base = static_cast<int64_t>(blockIdx.x) * (T * U);
+        const int64_t base = slot * (T * U);
         if (base + T * U <= nvec) body(base, static_cast<int64_t>(T), std::true_type{});
         else if (base < nvec) body(base, static_cast<int64_t>(T), std::false_type{});
     } else {
         static_assert(ONESHOT || T == kThreads, "the looping sweep is laid out for kThreads lanes");
-        sweep_tiles<U, false>(nvec, body);
+        sweep_tiles_of<U, false>(nvec, slot, G, body);
     }
+}
+
+template <int T, int U, bool ONESHOT, typename Body>
+__device__ __forceinline__ void walk_tiles(int64_t nvec, Body&& body) {
+    walk_tiles_of<T, U, ONESHOT>(nvec, blockIdx.x, gridDim.x, body);
 }
 
 template <int U = kUnroll, typename Body>
@@ -494,9 +549,10 @@ __device__ __forceinline__ uint32_t rhist_quantize4(H& h, int shift, int copy, c
 }
 
 // Move the slots into the 64-bit accumulators.  Called by all lanes of the workgroup (two barriers).
+template <int T = kThreads>
 __device__ __forceinline__ void rhist_flush(ResidualHist& h, int shift) {
     __syncthreads();
-    for (int b = threadIdx.x; b < kBins; b += kThreads) {
+    for (int b = threadIdx.x; b < kBins; b += T) {
         unsigned long long cnt = 0, sum = 0;
         for (int r = 0; r < (1 << shift); ++r) {
             const unsigned long long v = h.slot[(b << shift) + r];
@@ -510,41 +566,38 @@ __device__ __forceinline__ void rhist_flush(ResidualHist& h, int shift) {
     __syncthreads();
 }
 
-// A bin's entry of a workgroup's partial from its integer totals: the count, the sum of the residuals
-// in units of 2^-22 bin, and for the two clip bins the far elements' count and fp64 sum of x.
-__device__ __forceinline__ BinAcc rhist_entry(unsigned long long cnt, long long units, unsigned long long far_n, double far_s, float inv, int b) {
+// The fp64 sum of a bin's elements from the integer totals over the whole tensor: the count, the sum
+// of the residuals in units of 2^-22 bin (as hi * 2^32 + lo: the sum of the partials' upper and of their
+// lower halves, so that no 64-bit total can overflow) and, for the two clip bins, the far elements'
+// count and fp64 sum.  One conversion from exact integers: the same value however the tensor was dealt out.
+__device__ __forceinline__ double fixed_bin_sum(unsigned long long cnt, long long units_hi, unsigned long long units_lo,
+                                                unsigned long long far_n, double far_s, float inv, int b) {
     const double centre = static_cast<double>(static_cast<long long>(cnt - far_n) * (b - kZeroPoint));
-    const double bins = centre + static_cast<double>(units) * (1.0 / kResidualOne);
-    BinAcc acc;
-    acc.sum = bins / static_cast<double>(inv) + far_s;
-    acc.cnt = cnt;
-    return acc;
+    const double units = static_cast<double>(units_hi) * 4294967296.0 + static_cast<double>(units_lo);
+    return (centre + units * (1.0 / kResidualOne)) / static_cast<double>(inv) + far_s;
+}
+__device__ __forceinline__ long long units_hi(long long units) { return units >> 32; }
+__device__ __forceinline__ unsigned long long units_lo(long long units) { return static_cast<unsigned long long>(units) & 0xffffffffull; }
+
+__device__ __forceinline__ float mean_entry(double sum, unsigned long long cnt) {      // compression.cpp:99-101
+    return cnt ? static_cast<float>(sum / static_cast<double>(cnt)) : 0.0f;
 }
 
-// The far elements of bin b (0 or 255), their copies added in order.
+// The far elements of side `side` (0: bin 0, 1: bin 255), their copies added in order.
 template <typename H>
-__device__ __forceinline__ void rhist_far_of(const H& h, int b, unsigned long long& far_n, double& far_s) {
+__device__ __forceinline__ void rhist_far_side(const H& h, int side, unsigned long long& far_n, double& far_s) {
     far_n = 0;
     far_s = 0.0;
-    if (b == 0 || b == kBins - 1) {
-        const int side = b != 0;
 #pragma unroll
-        for (int c = 0; c < kFarCopies; ++c) { far_n += h.far_cnt[side][c]; far_s += h.far_sum[side][c]; }
-    }
+    for (int c = 0; c < kFarCopies; ++c) { far_n += h.far_cnt[side][c]; far_s += h.far_sum[side][c]; }
 }
 
-// Bin b of the workgroup's partial, after a last flush: the bin's sum of x in fp64 and its count.
-__device__ __forceinline__ BinAcc rhist_bin(const ResidualHist& h, float inv, int b) {
-    unsigned long long far_n;
-    double far_s;
-    rhist_far_of(h, b, far_n, far_s);
-    return rhist_entry(h.wide_cnt[b], h.wide_sum[b], far_n, far_s, inv, b);
-}
-
-// The workgroup's partial as workgroup `slot`, 4 KiB contiguous.
-__device__ __forceinline__ void rhist_store(ResidualHist& h, int shift, float inv, Workspace* ws, int slot) {
-    rhist_flush(h, shift);
-    for (int b = threadIdx.x; b < kBins; b += kThreads) ws->hist[slot][b] = rhist_bin(h, inv, b);
+// The workgroup's partial: 4 KiB of integer bin totals to `row`, the far elements to `far`.
+template <int T = kThreads>
+__device__ __forceinline__ void rhist_store(ResidualHist& h, int shift, BinPart* __restrict__ row, FarPart* __restrict__ far) {
+    rhist_flush<T>(h, shift);
+    for (int b = threadIdx.x; b < kBins; b += T) row[b] = BinPart{h.wide_sum[b], h.wide_cnt[b]};
+    if (threadIdx.x < 2) rhist_far_side(h, threadIdx.x, far->cnt[threadIdx.x], far->sum[threadIdx.x]);
 }
 
 // Register-side accumulators for a tensor whose values crowd into a few codes (a constant, or
@@ -607,6 +660,6 @@ __device__ __forceinline__ BinAcc hist_bin(const LdsHist<R>& h, int b) {
 // Store the workgroup's histogram as the partial of workgroup `slot`: one 16-byte store per lane,
 // 4 KiB contiguous per workgroup.
 template <int R>
-__device__ __forceinline__ void hist_store(LdsHist<R>& h, Workspace* ws, int slot) {
-    for (int b = threadIdx.x; b < kBins; b += kThreads) ws->hist[slot][b] = hist_bin(h, b);
+__device__ __forceinline__ void hist_store(LdsHist<R>& h, BinAcc* __restrict__ row) {
+    for (int b = threadIdx.x; b < kBins; b += kThreads) row[b] = hist_bin(h, b);
 }

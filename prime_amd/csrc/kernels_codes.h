@@ -227,14 +227,14 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_remap_kernel(con
 // kShotThreads lanes per tile instead of a loop.
 // SHOT_ROWS: rows of a ONESHOT workgroup's tile.  The plain set does best with four up to 2^25 elements (2^23: 6.2
 // against 7.5 us, 2^24: 13.1 against 15.4 us) and with two beyond (2^26: 54 against 58 us, 2^28: 211 against 242 us).
-template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT = false, int SHOT_ROWS = kShotUnroll>
-__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd)
-void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
-                    float divisor) {
+// dequant_block is the pass for the calling workgroup as workgroup `slot` of a grid of G would run it
+// (s_lut: 256 floats of LDS; the statistics partial goes to part_sum[slot] / part_sq[slot]).
+template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT, int SHOT_ROWS>
+__device__ __forceinline__ void dequant_block(float* __restrict__ out, const float* __restrict__ lut, const uint8_t* __restrict__ codes,
+                                              int64_t n, double* part_sum, double* part_sq, float divisor, int slot, int G, float* s_lut) {
     static_assert(!(ONESHOT && STATS), "statistics partials need the small grid of the looping sweep");
     using M = Mem<ALIGNED, NT>;
     constexpr int T = ONESHOT ? kShotThreads : kThreads;
-    __shared__ float s_lut[kBins];
     // The table goes to LDS once per workgroup, first thing.  A workgroup of the plain set that lives
     // for one tile issues the tile's loads before that, so that the table's trip to L2 runs beside the
     // codes' trip to memory instead of in front of it (2^28 elements: 210 instead of 233 us; with the
@@ -248,7 +248,7 @@ void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, cons
     const int64_t nvec = n >> 2;
     constexpr int U = ONESHOT ? SHOT_ROWS : DIV ? kDivUnroll : kUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+    walk_tiles_of<T, U, ONESHOT>(nvec, slot, G, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         const Window win(out + base * 4, (nvec - base) * 16);
@@ -281,7 +281,7 @@ void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, cons
             }
         }
     });
-    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    if (slot == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
         float v = s_lut[codes[i]];
         if (ADD) v += out[i];
@@ -293,5 +293,14 @@ void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, cons
             q0 = fma(d, d, q0);
         }
     }
-    if (STATS) block_stats_store(s0 + s1, q0 + q1, ws, blockIdx.x);
+    if (STATS) block_stats_store(s0 + s1, q0 + q1, part_sum, part_sq, slot);
+}
+
+template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT = false, int SHOT_ROWS = kShotUnroll>
+__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd)
+void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
+                    float divisor) {
+    __shared__ float s_lut[kBins];
+    dequant_block<ADD, STATS, ALIGNED, NT, DIV, POLICY, ONESHOT, SHOT_ROWS>(out, lut, codes, n, STATS ? ws->part_sum : nullptr,
+                                                                           STATS ? ws->part_sq : nullptr, divisor, blockIdx.x, gridDim.x, s_lut);
 }

@@ -24,9 +24,22 @@ __device__ __forceinline__ BinAcc block_sum_bin0(double s, unsigned long long c)
 
 // One (sum, count) pair for bin 0 as the workgroup's whole histogram partial: every lane brings the
 // fp64 sum and the number of the elements it saw.
-__device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, Workspace* ws, int slot) {
+__device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, BinAcc* __restrict__ row) {
     const BinAcc total = block_sum_bin0(s, c);
-    for (int b = threadIdx.x; b < kBins; b += kThreads) ws->hist[slot][b] = b == 0 ? total : BinAcc{0.0, 0ull};
+    for (int b = threadIdx.x; b < kBins; b += kThreads) row[b] = b == 0 ? total : BinAcc{0.0, 0ull};
+}
+
+// Where a workgroup of the quantize pass leaves its histogram partial: 256 bin entries (BinPart when
+// the histogram is the fixed-point one, BinAcc otherwise), the far elements, and - from the workgroup
+// with `first` set - the form of the partials for the kernel that reads them.
+struct HistOut {
+    BinAcc* row;
+    FarPart* far;
+    HistInfo* info;
+    bool first;
+};
+__device__ __forceinline__ HistOut hist_out_of(Workspace* ws, int slot) {
+    return HistOut{ws ? ws->hist[slot] : nullptr, ws ? &ws->far[slot] : nullptr, ws ? &ws->hist_info : nullptr, slot == 0};
 }
 
 // K2 (+K3 when HIST): quantize to uint8, 4 codes packed per 32-bit store, and the 256-bin
@@ -49,7 +62,7 @@ union QuantHist {
 
 template <bool ALIGNED, bool NT, bool HIST, bool REVERSE, int POLICY, int U = kUnroll>
 __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int64_t n, float inv, int narrow, int zero_point,
-                                               uint8_t* __restrict__ codes, Workspace* ws, int copies_shift, int slot, int G,
+                                               uint8_t* __restrict__ codes, const HistOut out_part, int copies_shift, int slot, int G,
                                                QuantHist& hist) {
     using M = Mem<ALIGNED, NT>;
     enum { kPlain, kFixed, kFp, kBin0 };
@@ -137,13 +150,14 @@ __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int6
     else if (mode == kBin0) pass(std::integral_constant<int, kBin0>{});
     else pass(std::integral_constant<int, kPlain>{});
     if (HIST) {
+        if (out_part.first && threadIdx.x == 0) *out_part.info = HistInfo{inv, mode == kFixed ? kHistFixed : kHistFp};
         if (mode == kFixed) {
-            rhist_store(hist.fixed, shift, inv, ws, slot);
+            rhist_store(hist.fixed, shift, reinterpret_cast<BinPart*>(out_part.row), out_part.far);
         } else if (mode == kFp) {
             __syncthreads();
-            hist_store(hist.fp, ws, slot);
+            hist_store(hist.fp, out_part.row);
         } else {
-            hist_store_bin0(lane_sum, lane_cnt, ws, slot);
+            hist_store_bin0(lane_sum, lane_cnt, out_part.row);
         }
     }
 }
@@ -160,8 +174,8 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
                       : stats_parts < 0 ? ws->qp.inv_scale
                                         : 1.0f / scale_val;
     __shared__ std::conditional_t<HIST, QuantHist, int> hist_mem;      // no histogram memory without HIST
-    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY, U>(x, n, inv, narrow, zero_point, codes, ws, copies_shift, blockIdx.x, gridDim.x,
-                                                       reinterpret_cast<QuantHist&>(hist_mem));
+    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY, U>(x, n, inv, narrow, zero_point, codes, hist_out_of(HIST ? ws : nullptr, blockIdx.x),
+                                                       copies_shift, blockIdx.x, gridDim.x, reinterpret_cast<QuantHist&>(hist_mem));
 }
 
 // K2 with the scale given and no histogram (quantize_per_tensor_uint8, compression.cpp:9-43), one
@@ -236,47 +250,96 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const flo
         if (a < n_bins) hist_add(hist, a, x[i]);
     }
     __syncthreads();
-    hist_store(hist, ws, blockIdx.x);
+    if (blockIdx.x == 0 && threadIdx.x == 0) ws->hist_info = HistInfo{0.0f, kHistFp};
+    hist_store(hist, ws->hist[blockIdx.x]);
 }
 
 // Second stage of the lookup build.  Workgroup j owns bins 4j .. 4j+3 (64 contiguous bytes
 // of every partial): lane (row, bin) adds partials row, row + 256, ... in order, the 256
 // rows are then added by a tree of fixed shape.  Mean = fp64 sum / count rounded to float
 // once; an empty bin gives 0.0f (compression.cpp:100).  Entries >= 256 of a longer table
-// are 0.0f.
+// are 0.0f.  Fixed-point partials (BinPart) are added as integers, the far elements of the two
+// clip bins beside them, and converted once (fixed_bin_sum).
 __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Workspace* __restrict__ ws, int nparts,
                                                                       float* __restrict__ lut, int64_t n_bins,
                                                                       unsigned long long* __restrict__ counts) {
     constexpr int kRows = kFinalThreads / kLutBinsPerBlock;
-    __shared__ double sh_sum[kFinalThreads];
+    __shared__ double sh_sum[kFinalThreads];                 // fixed-point partials: the upper halves' total, as an integer
+    __shared__ unsigned long long sh_lo[kFinalThreads];
     __shared__ unsigned long long sh_cnt[kFinalThreads];
+    __shared__ double sh_far_s[kRows];
+    __shared__ unsigned long long sh_far_n[kRows];
     const int bl = threadIdx.x % kLutBinsPerBlock;
     const int row = threadIdx.x / kLutBinsPerBlock;
     const int bin = blockIdx.x * kLutBinsPerBlock + bl;
+    const HistInfo info = ws->hist_info;
+    const bool fixed = info.mode == kHistFixed;
+    const bool far_bin = fixed && (bin == 0 || bin == kBins - 1);
     constexpr int kIters = kMaxGrid / kRows;
+    const int side = bin != 0;
     BinAcc part[kIters];
+    double far_s[kIters];
+    unsigned long long far_n[kIters];
 #pragma unroll
     for (int k = 0; k < kIters; ++k) {          // all loads in flight at once
         const int p = row + k * kRows;
         part[k] = p < nparts ? ws->hist[p][bin] : BinAcc{0.0, 0ull};
+        far_s[k] = far_bin && p < nparts ? ws->far[p].sum[side] : 0.0;
+        far_n[k] = far_bin && p < nparts ? ws->far[p].cnt[side] : 0ull;
     }
-    double s = 0.0;
     unsigned long long c = 0;
 #pragma unroll
-    for (int k = 0; k < kIters; ++k) { s += part[k].sum; c += part[k].cnt; }
-    sh_sum[threadIdx.x] = s;
+    for (int k = 0; k < kIters; ++k) c += part[k].cnt;
     sh_cnt[threadIdx.x] = c;
+    if (fixed) {
+        long long hi = 0;
+        unsigned long long lo = 0;
+#pragma unroll
+        for (int k = 0; k < kIters; ++k) {
+            const long long u = __double_as_longlong(part[k].sum);     // BinPart::units
+            hi += units_hi(u);
+            lo += units_lo(u);
+        }
+        sh_sum[threadIdx.x] = __longlong_as_double(hi);
+        sh_lo[threadIdx.x] = lo;
+        if (far_bin) {
+            double fs = 0.0;
+            unsigned long long fn = 0;
+#pragma unroll
+            for (int k = 0; k < kIters; ++k) { fs += far_s[k]; fn += far_n[k]; }
+            sh_far_s[row] = fs;
+            sh_far_n[row] = fn;
+        }
+    } else {
+        double s = 0.0;
+#pragma unroll
+        for (int k = 0; k < kIters; ++k) s += part[k].sum;
+        sh_sum[threadIdx.x] = s;
+    }
     __syncthreads();
     for (int half = kRows / 2; half > 0; half >>= 1) {
         if (row < half) {
-            sh_sum[threadIdx.x] += sh_sum[threadIdx.x + half * kLutBinsPerBlock];
-            sh_cnt[threadIdx.x] += sh_cnt[threadIdx.x + half * kLutBinsPerBlock];
+            const int other = threadIdx.x + half * kLutBinsPerBlock;
+            sh_cnt[threadIdx.x] += sh_cnt[other];
+            if (fixed) {
+                sh_sum[threadIdx.x] = __longlong_as_double(__double_as_longlong(sh_sum[threadIdx.x]) + __double_as_longlong(sh_sum[other]));
+                sh_lo[threadIdx.x] += sh_lo[other];
+                if (far_bin) {
+                    sh_far_s[row] += sh_far_s[row + half];
+                    sh_far_n[row] += sh_far_n[row + half];
+                }
+            } else {
+                sh_sum[threadIdx.x] += sh_sum[other];
+            }
         }
         __syncthreads();
     }
     if (row == 0 && bin < n_bins) {
         const unsigned long long cc = sh_cnt[threadIdx.x];
-        lut[bin] = cc ? static_cast<float>(sh_sum[threadIdx.x] / static_cast<double>(cc)) : 0.0f;
+        const double sum = fixed ? fixed_bin_sum(cc, __double_as_longlong(sh_sum[threadIdx.x]), sh_lo[threadIdx.x], far_bin ? sh_far_n[0] : 0ull,
+                                                 far_bin ? sh_far_s[0] : 0.0, info.inv, bin)
+                                 : sh_sum[threadIdx.x];
+        lut[bin] = mean_entry(sum, cc);
         if (counts) counts[bin] = cc;
     }
     if (blockIdx.x == 0)
@@ -406,8 +469,11 @@ __global__ __launch_bounds__(kBatchThreads) void batched_kernel(const float* __r
         }
         rhist_flush(h, shift);
         for (int bin = threadIdx.x; bin < kBins; bin += kBatchThreads) {
-            const BinAcc e = rhist_bin(h, inv, bin);
-            luts[t * kBins + bin] = e.cnt ? static_cast<float>(e.sum / static_cast<double>(e.cnt)) : 0.0f;
+            unsigned long long far_n = 0;
+            double far_s = 0.0;
+            if (bin == 0 || bin == kBins - 1) rhist_far_side(h, bin != 0, far_n, far_s);
+            const unsigned long long cnt = h.wide_cnt[bin];
+            luts[t * kBins + bin] = mean_entry(fixed_bin_sum(cnt, units_hi(h.wide_sum[bin]), units_lo(h.wide_sum[bin]), far_n, far_s, inv, bin), cnt);
         }
         return;
     }

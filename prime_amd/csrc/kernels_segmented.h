@@ -1,0 +1,175 @@
+// Segmented launches: up to kSegMax tensors (or ring chunks) go through a pass in ONE launch, each
+// with as many workgroups as its size wants, so that a set of mid-size tensors pays three kernel
+// boundaries in all instead of three per tensor (the ring all-reduce of one layer bucket cuts it
+// into 2 W chunks, collectives.cpp:89-90, and the per-layer loop of diloco.py:108-110 visits one
+// bucket after the other).  Results equal the one-tensor entry points' bit for bit:
+//  * statistics: tensor t has `parts[t]` partial slots, the grid the one-tensor entry point would
+//    launch for it, and the workgroup that plays slot v adds exactly what workgroup v of that grid
+//    adds, in the same order (stats_partial / dequant_block are written for "workgroup `slot` of G");
+//    the consuming pass adds the slots as the one-tensor quantize kernel does;
+//  * codes depend on the element and the scale alone;
+//  * the histogram partials are integers (BinPart), so their totals do not depend on how many
+//    workgroups shared a tensor or which of them saw which tile.
+// What may differ in its last bit: the lookup entries of a tensor whose 1 / scale is zero or not
+// finite (fp64 partials, rare), and bins 0 / 255 of a tensor with elements beyond the fixed-point
+// range in more than one workgroup (fp64 sums of those elements, already dependent on arrival order).
+//
+// The tensors' descriptors travel by value in the kernel arguments (no device-side table to fill
+// before the launch); a workgroup finds its tensor by a binary search over the block ranges.
+//
+// Included by prime_hip.hip inside its anonymous namespace; not a translation unit of its own.
+
+struct SegJob {
+    int count;
+    int first[kSegMax + 1];              // workgroups [first[t], first[t + 1]) of this launch belong to tensor t
+    int parts[kSegMax];                  // statistics partials of tensor t: the grid of the one-tensor entry point
+    unsigned long long two_row;          // bit t: the pass of this launch takes tiles of two rows on tensor t
+    int64_t n[kSegMax];
+    float* x[kSegMax];                   // the tensor / the ring chunk (updated in place by a ring step)
+    uint8_t* codes[kSegMax];             // codes out
+    const uint8_t* codes_in[kSegMax];    // the received message of a ring step
+    const float* lut_in[kSegMax];
+};
+static_assert(sizeof(SegJob) <= 4000, "the descriptors must fit the kernel argument segment");
+
+// The tensor whose block range holds `block`: the last t with first[t] <= block.
+__device__ __forceinline__ int seg_tensor_of(const int* first, int count, int block) {
+    int lo = 0, hi = count;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (first[mid] <= block) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+// A tensor with fewer rows than one tile per statistics slot: its slots own single rows, and one
+// workgroup plays several of them at once (stats_partial_short): eight vectors per lane in flight.
+__host__ __device__ constexpr int seg_short_slots(bool two_row) { return two_row ? 4 : 2; }
+__host__ __device__ inline bool seg_short(int64_t n, int parts, bool two_row) {
+    return ((n >> 2) / kThreads) / (static_cast<int64_t>(parts) * (two_row ? 2 : kUnroll)) == 0;
+}
+
+// K1 for every tensor of the job: one workgroup per statistics slot (per group of slots of a short tensor).
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void seg_stats_kernel(const SegJob job, Workspace* ws) {
+    const int t = seg_tensor_of(job.first, job.count, blockIdx.x);
+    const int v = blockIdx.x - job.first[t];
+    const int64_t n = job.n[t];
+    const int G = job.parts[t];
+    const bool two = (job.two_row >> t) & 1;
+    double* ps = ws->seg_part_sum[t];
+    double* pq = ws->seg_part_sq[t];
+    if (seg_short(n, G, two)) {
+        if (two) stats_partial_short<2, seg_short_slots(true)>(job.x[t], n, v * seg_short_slots(true), G, ps, pq);
+        else stats_partial_short<kUnroll, seg_short_slots(false)>(job.x[t], n, v * seg_short_slots(false), G, ps, pq);
+    } else if (two) {
+        stats_partial<true, false, 2>(job.x[t], n, v, G, ps, pq);
+    } else {
+        stats_partial<true, false, kUnroll>(job.x[t], n, v, G, ps, pq);
+    }
+}
+
+// First pass of a ring step for every chunk of the job: chunk (+)= lut_in[codes_in] [/ divisor] with
+// the statistics of the result, one workgroup per statistics slot.
+template <bool ADD, bool DIV, int POLICY>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void seg_dequant_kernel(const SegJob job, float divisor, Workspace* ws) {
+    __shared__ float s_lut[kBins];
+    const int t = seg_tensor_of(job.first, job.count, blockIdx.x);
+    const int v = blockIdx.x - job.first[t];
+    dequant_block<ADD, true, true, false, DIV, POLICY, false, kShotUnroll>(job.x[t], job.lut_in[t], job.codes_in[t], job.n[t], ws->seg_part_sum[t],
+                                                                          ws->seg_part_sq[t], divisor, v, job.parts[t], s_lut);
+}
+
+// K2 + K3 for every tensor of the job: tensor t is shared by the workgroups of its block range, each
+// of which derives the tensor's scale from the statistics slots and leaves one histogram partial in
+// the row of its block index.
+template <int POLICY>
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void seg_quantize_kernel(const SegJob job, prime_qparams* qp_out, Workspace* ws,
+                                                                                int copies_shift) {
+    __shared__ QuantHist hist_mem;
+    const int t = seg_tensor_of(job.first, job.count, blockIdx.x);
+    const int p = blockIdx.x - job.first[t];
+    const int P = job.first[t + 1] - job.first[t];
+    const int64_t n = job.n[t];
+    int narrow = INT_MIN;
+    const float inv = block_scale_from_partials<kThreads>(ws->seg_part_sum[t], ws->seg_part_sq[t], job.parts[t], n, p == 0, &ws->seg[t].qp,
+                                                          qp_out ? qp_out + t : nullptr, &narrow);
+    const HistOut out{ws->hist[blockIdx.x], &ws->far[blockIdx.x], &ws->seg[t].info, p == 0};
+    if ((job.two_row >> t) & 1)
+        quantize_block<true, true, true, true, POLICY, 2>(job.x[t], n, inv, narrow, kZeroPoint, job.codes[t], out, copies_shift, p, P, hist_mem);
+    else
+        quantize_block<true, true, true, true, POLICY, kUnroll>(job.x[t], n, inv, narrow, kZeroPoint, job.codes[t], out, copies_shift, p, P, hist_mem);
+}
+
+// The lookup tables of the job: one workgroup per tensor.  Lane (g, b) adds bin b of every fourth of
+// the tensor's partials (rows first[t] .. first[t + 1] of the quantize launch), several loads in
+// flight; the four groups are joined in LDS and the total converted once.
+constexpr int kSegFinalGroups = kFinalThreads / kBins;
+__global__ __launch_bounds__(kFinalThreads) void seg_lut_finalize_kernel(const SegJob job, const Workspace* __restrict__ ws, float* __restrict__ luts) {
+    __shared__ double sh_sum[kSegFinalGroups][kBins];            // fixed-point partials: the upper halves' total, as an integer
+    __shared__ unsigned long long sh_lo[kSegFinalGroups][kBins];
+    __shared__ unsigned long long sh_cnt[kSegFinalGroups][kBins];
+    __shared__ double sh_far_s[kSegFinalGroups][2];
+    __shared__ unsigned long long sh_far_n[kSegFinalGroups][2];
+    const int t = blockIdx.x;
+    const int b = threadIdx.x & (kBins - 1), g = threadIdx.x / kBins;
+    const int p0 = job.first[t], p1 = job.first[t + 1];
+    const HistInfo info = ws->seg[t].info;
+    const bool fixed = info.mode == kHistFixed;
+    const bool far_bin = fixed && (b == 0 || b == kBins - 1);
+    const int side = b != 0;
+    unsigned long long cnt = 0, lo = 0, far_n = 0;
+    long long hi = 0;
+    double sum = 0.0, far_s = 0.0;
+    constexpr int kInFlight = 8;
+    for (int q0 = p0 + g; q0 < p1; q0 += kSegFinalGroups * kInFlight) {
+        BinAcc e[kInFlight];
+        double fs[kInFlight];
+        unsigned long long fn[kInFlight];
+#pragma unroll
+        for (int k = 0; k < kInFlight; ++k) {
+            const int p = q0 + k * kSegFinalGroups;
+            e[k] = p < p1 ? ws->hist[p][b] : BinAcc{0.0, 0ull};
+            fs[k] = far_bin && p < p1 ? ws->far[p].sum[side] : 0.0;
+            fn[k] = far_bin && p < p1 ? ws->far[p].cnt[side] : 0ull;
+        }
+#pragma unroll
+        for (int k = 0; k < kInFlight; ++k) {
+            cnt += e[k].cnt;
+            if (fixed) {
+                const long long u = __double_as_longlong(e[k].sum);      // BinPart::units
+                hi += units_hi(u);
+                lo += units_lo(u);
+                far_s += fs[k];
+                far_n += fn[k];
+            } else {
+                sum += e[k].sum;
+            }
+        }
+    }
+    sh_cnt[g][b] = cnt;
+    sh_lo[g][b] = lo;
+    sh_sum[g][b] = fixed ? __longlong_as_double(hi) : sum;
+    if (far_bin) {
+        sh_far_s[g][side] = far_s;
+        sh_far_n[g][side] = far_n;
+    }
+    __syncthreads();
+    if (g == 0) {
+#pragma unroll
+        for (int k = 1; k < kSegFinalGroups; ++k) {
+            cnt += sh_cnt[k][b];
+            if (fixed) {
+                hi += __double_as_longlong(sh_sum[k][b]);
+                lo += sh_lo[k][b];
+                if (far_bin) {
+                    far_s += sh_far_s[k][side];
+                    far_n += sh_far_n[k][side];
+                }
+            } else {
+                sum += sh_sum[k][b];
+            }
+        }
+        if (fixed) sum = fixed_bin_sum(cnt, hi, lo, far_n, far_s, info.inv, b);
+        luts[static_cast<int64_t>(t) * kBins + b] = mean_entry(sum, cnt);
+    }
+}

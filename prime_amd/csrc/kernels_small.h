@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kThreads) void uniform_small_kernel(float* __restri
     const bool mine = static_cast<int>(threadIdx.x) < rows;
     const double pa = (0.0 + (mine ? sh_part_s[threadIdx.x & (kSmallSlots - 1)] : 0.0)) + 0.0;
     const double pb = (0.0 + (mine ? sh_part_q[threadIdx.x & (kSmallSlots - 1)] : 0.0)) + 0.0;
-    const float inv = block_scale_reduce<kThreads>(pa, pb, ws, n, qp_out, &narrow);
+    const float inv = block_scale_reduce<kThreads>(pa, pb, n, true, &ws->qp, qp_out, &narrow);
 
     // codes and histogram; the modes are those of quantize_block
     enum { kFixed, kFp, kBin0 };
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kThreads) void uniform_small_kernel(float* __restri
             rhist_add(hists.row[0], kSmallShift, copy, a, far ? 0 : residual_fixed(tail_v, inv, a));
         }
         __syncthreads();
-        // lane -> (row, bin): the bin's entry of that row's partial, left where the bin's slots were
+        // lane -> (row, bin): the bin's integer totals of that row's partial, left where the bin's slots were
         const int bin = threadIdx.x & (kBins - 1);
 #pragma unroll
         for (int pass = 0; pass < kSmallSlots * kBins / kThreads; ++pass) {
@@ -193,24 +193,40 @@ __global__ __launch_bounds__(kThreads) void uniform_small_kernel(float* __restri
                 cnt += s >> 48;
                 sum += s & 0xffffffffffffull;
             }
-            unsigned long long far_n;
-            double far_s;
-            rhist_far_of(h, bin, far_n, far_s);
-            const BinAcc e = rhist_entry(cnt, static_cast<long long>(sum) - static_cast<long long>(cnt << 31), far_n, far_s, inv, bin);
-            static_assert(kSmallShift >= 1, "an entry takes the place of two slots");
-            h.slot[(bin << kSmallShift)] = static_cast<unsigned long long>(__double_as_longlong(e.sum));
-            h.slot[(bin << kSmallShift) + 1] = e.cnt;
+            static_assert(kSmallShift >= 1, "the totals take the place of two slots");
+            h.slot[(bin << kSmallShift)] = static_cast<unsigned long long>(static_cast<long long>(sum) - static_cast<long long>(cnt << 31));
+            h.slot[(bin << kSmallShift) + 1] = cnt;
         }
         __syncthreads();
         if (threadIdx.x < kBins) {
+            // what lut_finalize_kernel makes of these partials: integer totals over the rows, the far
+            // elements' sums added in the order of its tree, one conversion
+            unsigned long long cnt = 0, lo = 0, far_n = 0;
+            long long hi = 0;
+            double leaf[kSmallSlots];
+            const bool far_bin = bin == 0 || bin == kBins - 1;
 #pragma unroll
             for (int r = 0; r < kSmallSlots; ++r) {
+                leaf[r] = 0.0;
                 if (r < rows) {
-                    part[r].sum = __longlong_as_double(static_cast<long long>(hists.row[r].slot[(bin << kSmallShift)]));
-                    part[r].cnt = hists.row[r].slot[(bin << kSmallShift) + 1];
+                    const long long u = static_cast<long long>(hists.row[r].slot[(bin << kSmallShift)]);
+                    hi += units_hi(u);
+                    lo += units_lo(u);
+                    cnt += hists.row[r].slot[(bin << kSmallShift) + 1];
+                    if (far_bin) {
+                        unsigned long long fn;
+                        double fs;
+                        rhist_far_side(hists.row[r], bin != 0, fn, fs);
+                        far_n += fn;
+                        leaf[r] = 0.0 + fs;
+                    }
                 }
             }
+            const double far_s = (leaf[0] + leaf[2]) + (leaf[1] + leaf[3]);
+            lut[threadIdx.x] = mean_entry(fixed_bin_sum(cnt, hi, lo, far_n, far_s, inv, bin), cnt);
         }
+        if (threadIdx.x == 0) ws->hist_info = HistInfo{inv, kHistFixed};
+        return;
     } else {
         // row by row through one histogram (rare: a zero or non-finite 1 / scale)
         auto set_part = [&](int r, BinAcc e) {

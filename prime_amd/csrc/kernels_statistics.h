@@ -13,7 +13,7 @@ __global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace
 // The statistics partial of workgroup `slot` of a grid of G, computed by the calling workgroup and
 // stored in the workspace: fp64 sum and sum of squares of the rows that workgroup owns.
 template <bool ALIGNED, bool NT, int U = kUnroll>
-__device__ __forceinline__ void stats_partial(const float* __restrict__ x, int64_t n, int slot, int G, Workspace* ws) {
+__device__ __forceinline__ void stats_partial(const float* __restrict__ x, int64_t n, int slot, int G, double* part_sum, double* part_sq) {
     using M = Mem<ALIGNED, NT>;
     const int64_t nvec = n >> 2;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
@@ -36,14 +36,73 @@ __device__ __forceinline__ void stats_partial(const float* __restrict__ x, int64
         s0 += v;
         q0 = fma(v, v, q0);
     }
-    block_stats_store(s0 + s1, q0 + q1, ws, slot);
+    block_stats_store(s0 + s1, q0 + q1, part_sum, part_sq, slot);
+}
+
+// The statistics partials of K consecutive slots, first, first + 1, ..., of a grid of G by ONE workgroup,
+// for a tensor so short that no slot has a whole tile (fewer than G * U rows: every slot owns the rows
+// slot, slot + G, ... only).  Each slot's sums are formed exactly as stats_partial forms them - the same
+// additions in the same order - but the K slots' loads are in flight together and their reductions
+// run side by side: a workgroup that plays one such slot has a single 16 KiB row in flight.
+template <int U, int K>
+__device__ __forceinline__ void stats_partial_short(const float* __restrict__ x, int64_t n, int first, int G, double* part_sum,
+                                                    double* part_sq) {
+    using M = Mem<true, false>;
+    __shared__ double sh_s[K][kWaves];
+    __shared__ double sh_q[K][kWaves];
+    const int64_t nvec = n >> 2;
+    const int64_t rows = (nvec + kThreads - 1) / kThreads;
+    f4a v[K][U];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const int64_t row = first + k + static_cast<int64_t>(j) * G;
+            const int64_t i = row * kThreads + threadIdx.x;
+            v[k][j] = (first + k < G && first + k < rows && i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    double s[K], q[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            if (j & 1) stats_add4(v[k][j], s1, q1); else stats_add4(v[k][j], s0, q0);
+        }
+        if (first + k == 0 && threadIdx.x < (n & 3)) {
+            const double t = x[(nvec << 2) + threadIdx.x];
+            s0 += t;
+            q0 = fma(t, t, q0);
+        }
+        s[k] = s0 + s1;
+        q[k] = q0 + q1;
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {                 // independent chains: the compiler overlaps them
+        s[k] = wave_sum(s[k]);
+        q[k] = wave_sum(q[k]);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) { sh_s[k][wave] = s[k]; sh_q[k][wave] = q[k]; }
+    }
+    __syncthreads();
+    if (threadIdx.x < K && first + static_cast<int>(threadIdx.x) < G) {
+        double S = sh_s[threadIdx.x][0], Q = sh_q[threadIdx.x][0];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) { S += sh_s[threadIdx.x][w]; Q += sh_q[threadIdx.x][w]; }
+        part_sum[first + threadIdx.x] = S;
+        part_sq[first + threadIdx.x] = Q;
+    }
 }
 
 // K1: sum and sum of squares in fp64.  4 bytes per element.
 // U = rows per tile: 4 from 2^27 elements up, 2 below (a 51 M-element bucket: 33.3 against 34.4 us).
 template <bool ALIGNED, bool NT, int U = kUnroll>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
-    stats_partial<ALIGNED, NT, U>(x, n, blockIdx.x, gridDim.x, ws);
+    stats_partial<ALIGNED, NT, U>(x, n, blockIdx.x, gridDim.x, ws->part_sum, ws->part_sq);
 }
 
 // The norm as libtorch's CPU kernel accumulates it (the value compression.cpp:113 actually

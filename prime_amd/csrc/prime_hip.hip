@@ -33,6 +33,7 @@ namespace {
 #include "kernels_small.h"
 #include "kernels_codes.h"
 #include "kernels_outer.h"
+#include "kernels_segmented.h"
 
 // ---------------------------------------------------------------------------------------------
 // host side
@@ -73,6 +74,7 @@ struct Options {
     // a 51 M-element bucket 74.5 against 78.4 us for the three launches, 2^26 elements 93.5 against 97.4;
     // from 2^27 up four rows win (2^27: 196 against 207 us, 2^28: 378 against 404)
     int64_t two_row_below_elems = int64_t(1) << 27;
+    int segment_blocks_per_cu = 2;  // workgroups per compute unit the quantize pass of a segmented launch shares out among its tensors
     int64_t set_four_rows_max_elems = int64_t(1) << 25;  // the one-workgroup-per-tile dequantize set takes tiles of four rows up to this many elements (0: never)
 };
 Options g_opt;
@@ -136,13 +138,15 @@ int launch_check(const char* where) {
 // default; when off a launch site pays one branch.
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
-    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouchCodes, kIdCodeCount, kIdCodeTotal, kIdRequantPlan, kIdCodeRemap, kIdNormLiteral, kIdUniformSmall, kIdCount
+    kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouchCodes, kIdCodeCount, kIdCodeTotal, kIdRequantPlan, kIdCodeRemap, kIdNormLiteral, kIdUniformSmall,
+    kIdSegStats, kIdSegDequantAdd, kIdSegDequantSet, kIdSegQuantize, kIdSegLutFinalize, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
     "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
     "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>", "div_kernel",
-    "first_touch_kernel<codes>", "code_count_kernel", "code_total_kernel", "requant_plan_kernel", "code_remap_kernel", "norm_literal_kernel", "uniform_small_kernel"};
+    "first_touch_kernel<codes>", "code_count_kernel", "code_total_kernel", "requant_plan_kernel", "code_remap_kernel", "norm_literal_kernel", "uniform_small_kernel",
+    "seg_stats_kernel", "seg_dequant_kernel<add,stats>", "seg_dequant_kernel<set,stats>", "seg_quantize_kernel+hist", "seg_lut_finalize_kernel"};
 
 struct TimedLaunch {
     int id;
@@ -414,6 +418,7 @@ int prime_hip_set_option(const char* name, int value) {
         if (value < 0) return fail(PRIME_EINVAL, "large_read_min_mi_elems must be >= 0");
         g_opt.large_read_min_elems = static_cast<int64_t>(value) << 20;
     } else if (!strcmp(name, "grid_cap")) {
+        if (value < 0) return fail(PRIME_EINVAL, "grid_cap must be >= 0 (0: none)");
         g_opt.grid_cap = value;
     } else if (!strcmp(name, "one_shot")) {
         g_opt.one_shot = value != 0;
@@ -430,6 +435,9 @@ int prime_hip_set_option(const char* name, int value) {
     } else if (!strcmp(name, "set_four_rows_max_mi_elems")) {
         if (value < 0 || value > 8192) return fail(PRIME_EINVAL, "set_four_rows_max_mi_elems must be in [0, 8192] (0: off)");
         g_opt.set_four_rows_max_elems = static_cast<int64_t>(value) << 20;
+    } else if (!strcmp(name, "segment_blocks_per_cu")) {
+        if (value < 1 || value > 8) return fail(PRIME_EINVAL, "segment_blocks_per_cu must be 1..8");
+        g_opt.segment_blocks_per_cu = value;
     } else if (!strcmp(name, "reverse_second_pass")) {
         g_opt.reverse_second_pass = value != 0;
     } else if (!strcmp(name, "nt_load_min_mib")) {
@@ -450,6 +458,7 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "hist_replicas")) *value = g_opt.hist_replicas;
     else if (!strcmp(name, "code_store_policy")) *value = g_opt.code_store_policy;
     else if (!strcmp(name, "reverse_second_pass")) *value = g_opt.reverse_second_pass;
+    else if (!strcmp(name, "segment_blocks_per_cu")) *value = g_opt.segment_blocks_per_cu;
     else if (!strcmp(name, "large_read_grid_eighths")) *value = g_opt.large_read_grid_eighths;
     else if (!strcmp(name, "large_read_min_mi_elems")) *value = static_cast<int>(g_opt.large_read_min_elems >> 20);
     else if (!strcmp(name, "average_replicas")) *value = g_opt.average_replicas;
@@ -761,6 +770,148 @@ int ring_step(float* chunk, const uint8_t* codes_in, const float* lut_in, int64_
 
 }  // namespace
 
+namespace {
+
+// ---- segmented launches -------------------------------------------------------------------------
+enum SegKind { kSegUniform = 0, kSegReduce = 1, kSegGather = 2, kSegReduceDiv = 3 };
+
+// One group of at most kSegMax tensors, all 16-byte (codes: 4-byte) aligned and non-empty: three
+// launches.  luts / qps point at the group's first entry.
+int run_segment_group(SegKind kind, int count, float* const* xs, const int64_t* ns, uint8_t* const* codes, const uint8_t* const* codes_in,
+                      const float* const* luts_in, float divisor, float* luts, prime_qparams* qps, Workspace* w, hipStream_t st) {
+    SegJob job;
+    memset(&job, 0, sizeof(job));
+    job.count = count;
+    const bool add = kind == kSegReduce || kind == kSegReduceDiv;
+    int64_t total = 0;
+    double bytes_a = 0.0, bytes_q = 0.0;
+    for (int t = 0; t < count; ++t) {
+        job.n[t] = ns[t];
+        job.x[t] = xs[t];
+        job.codes[t] = codes[t];
+        job.codes_in[t] = codes_in ? codes_in[t] : nullptr;
+        job.lut_in[t] = luts_in ? luts_in[t] : nullptr;
+        // the statistics slots: the grid the one-tensor entry point launches for its first pass
+        job.parts[t] = kind == kSegUniform ? grid_for(ns[t], true) : grid_for(ns[t], add);
+        if (kind == kSegUniform && two_row_tiles(ns[t])) job.two_row |= 1ull << t;
+        total += ns[t];
+        bytes_a += (kind == kSegUniform ? 4.0 : add ? 9.0 : 5.0) * ns[t];
+        bytes_q += 5.0 * ns[t];
+    }
+    job.first[0] = 0;
+    for (int t = 0; t < count; ++t) {
+        int blocks = job.parts[t];
+        const bool two = (job.two_row >> t) & 1;
+        if (kind == kSegUniform && seg_short(ns[t], job.parts[t], two)) blocks = (blocks + seg_short_slots(two) - 1) / seg_short_slots(two);
+        job.first[t + 1] = job.first[t] + blocks;
+    }
+    const int grid_a = job.first[count];
+    if (kind == kSegUniform) {
+        launch(kIdSegStats, bytes_a, seg_stats_kernel, grid_a, kThreads, st, job, w);
+    } else {
+        with_policy(g_opt.f32_reread_store_policy, [&](auto P) {
+            constexpr int POL = decltype(P)::value;
+            if (kind == kSegGather) launch(kIdSegDequantSet, bytes_a, seg_dequant_kernel<false, false, POL>, grid_a, kThreads, st, job, divisor, w);
+            else if (kind == kSegReduceDiv && divisor != 1.0f)
+                launch(kIdSegDequantAdd, bytes_a, seg_dequant_kernel<true, true, POL>, grid_a, kThreads, st, job, divisor, w);
+            else launch(kIdSegDequantAdd, bytes_a, seg_dequant_kernel<true, false, POL>, grid_a, kThreads, st, job, divisor, w);
+        });
+    }
+    if (int rc = launch_check("segmented first pass")) return rc;
+    // the quantize pass: segment_blocks_per_cu workgroups per compute unit, shared out by size; a tensor
+    // gets at least one and at most one per tile
+    const int64_t budget = static_cast<int64_t>(cu_count()) * g_opt.segment_blocks_per_cu;
+    job.two_row = 0;
+    int first = 0;
+    for (int t = 0; t < count; ++t) {
+        const bool two = two_row_tiles(ns[t], kind != kSegUniform);
+        if (two) job.two_row |= 1ull << t;
+        const int64_t rows = (ns[t] + kRowElems - 1) / kRowElems;
+        const int64_t tiles = (rows + (two ? 2 : kUnroll) - 1) / (two ? 2 : kUnroll);
+        int64_t share = (budget * ns[t] + total / 2) / total;
+        if (share > tiles) share = tiles;
+        if (share < 1) share = 1;
+        job.first[t] = first;
+        first += static_cast<int>(share);
+    }
+    job.first[count] = first;
+    if (first > kMaxGrid) return fail(PRIME_EINVAL, "segmented launch: more workgroups than histogram rows in the workspace");
+    int shift = 0;
+    while ((1 << (shift + 1)) <= g_opt.hist_replicas) ++shift;
+    launch(kIdSegQuantize, bytes_q, seg_quantize_kernel<kStoreNt>, first, kThreads, st, job, qps, w, shift);
+    if (int rc = launch_check("seg_quantize_kernel")) return rc;
+    launch(kIdSegLutFinalize, 16.0 * kBins * first, seg_lut_finalize_kernel, count, kFinalThreads, st, job, w, luts);
+    return launch_check("seg_lut_finalize_kernel");
+}
+
+int ring_step_one(SegKind kind, float* chunk, const uint8_t* codes_in, const float* lut_in, int64_t n, float divisor, uint8_t* codes_out,
+                  float* lut_out, prime_qparams* qp, void* ws, prime_stream_t stream);
+
+// Every tensor of the call: those a segmented launch can take go in groups of kSegMax, the others
+// (empty, or not aligned for vector access) through the one-tensor entry point, which gives the same results.
+int run_segmented(SegKind kind, const char* who, float* const* xs, const int64_t* ns, int64_t count, uint8_t* const* codes,
+                  const uint8_t* const* codes_in, const float* const* luts_in, float divisor, float* luts, prime_qparams* qps, void* ws,
+                  prime_stream_t stream) {
+    if (count < 0 || (count > 0 && (!xs || !ns || !codes || !luts)) || (count > 0 && kind != kSegUniform && (!codes_in || !luts_in)))
+        return fail(PRIME_EINVAL, who);
+    if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
+    if (kind == kSegReduceDiv && (!(divisor == divisor) || divisor == 0.0f)) return fail(PRIME_EINVAL, "segmented ring step: divisor must be a non-zero number");
+    for (int64_t i = 0; i < count; ++i) {
+        if (bad_n(ns[i]) || (ns[i] > 0 && (!xs[i] || !codes[i])) || (kind != kSegUniform && ((ns[i] > 0 && !codes_in[i]) || !luts_in[i])))
+            return fail(PRIME_EINVAL, who);
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Workspace* w = static_cast<Workspace*>(ws);
+    float* gx[kSegMax];
+    int64_t gn[kSegMax];
+    uint8_t* gc[kSegMax];
+    const uint8_t* gci[kSegMax];
+    const float* gli[kSegMax];
+    int64_t i = 0;
+    while (i < count) {
+        // a group: consecutive tensors that qualify (outputs of a group are contiguous in luts / qps)
+        int g = 0;
+        const int64_t start = i;
+        while (i < count && g < kSegMax) {
+            const bool ok = ns[i] > 0 && aligned_to(xs[i], 16) && aligned_to(codes[i], 4) && (kind == kSegUniform || aligned_to(codes_in[i], 4));
+            if (!ok) break;
+            gx[g] = xs[i];
+            gn[g] = ns[i];
+            gc[g] = codes[i];
+            gci[g] = codes_in ? codes_in[i] : nullptr;
+            gli[g] = luts_in ? luts_in[i] : nullptr;
+            ++g;
+            ++i;
+        }
+        if (g == 1) {                     // a group of one gains nothing over the one-tensor entry point
+            i = start;
+            g = 0;
+        }
+        if (g > 0) {
+            if (int rc = run_segment_group(kind, g, gx, gn, gc, codes_in ? gci : nullptr, luts_in ? gli : nullptr, divisor, luts + start * kBins,
+                                           qps ? qps + start : nullptr, w, st))
+                return rc;
+            continue;
+        }
+        prime_qparams* qp = qps ? qps + i : nullptr;
+        int rc;
+        if (kind == kSegUniform) rc = uniform_checked(xs[i], ns[i], codes[i], luts + i * kBins, qp, ws, stream);
+        else rc = ring_step_one(kind, xs[i], codes_in[i], luts_in[i], ns[i], divisor, codes[i], luts + i * kBins, qp, ws, stream);
+        if (rc) return rc;
+        ++i;
+    }
+    return 0;
+}
+
+int ring_step_one(SegKind kind, float* chunk, const uint8_t* codes_in, const float* lut_in, int64_t n, float divisor, uint8_t* codes_out,
+                  float* lut_out, prime_qparams* qp, void* ws, prime_stream_t stream) {
+    if (kind == kSegGather) return ring_step<false>(chunk, codes_in, lut_in, n, codes_out, lut_out, qp, ws, stream, "segmented ring step: bad argument");
+    return ring_step<true>(chunk, codes_in, lut_in, n, codes_out, lut_out, qp, ws, stream, "segmented ring step: bad argument",
+                           kind == kSegReduceDiv ? divisor : 1.0f);
+}
+
+}  // namespace
+
 extern "C" {
 
 int prime_ring_reduce_step(float* acc, const uint8_t* codes_in, const float* lut_in, int64_t n, uint8_t* codes_out,
@@ -780,6 +931,33 @@ int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* l
                            float* lut_out, prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
     return ring_step<false>(chunk, codes_in, lut_in, n, codes_out, lut_out, qparams_out, ws, stream,
                             "prime_ring_gather_step: bad argument");
+}
+
+int prime_uniform_8bit_quantize_segmented(const float* const* xs, const int64_t* ns, int64_t count, uint8_t* const* codes, float* luts,
+                                          prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
+    return run_segmented(kSegUniform, "prime_uniform_8bit_quantize_segmented: bad argument", const_cast<float* const*>(xs), ns, count, codes, nullptr,
+                         nullptr, 1.0f, luts, qparams_out, ws, stream);
+}
+
+int prime_ring_reduce_step_segmented(float* const* accs, const uint8_t* const* codes_in, const float* const* luts_in, const int64_t* ns,
+                                     int64_t count, uint8_t* const* codes_out, float* luts_out, prime_qparams* qparams_out, void* ws,
+                                     prime_stream_t stream) {
+    return run_segmented(kSegReduce, "prime_ring_reduce_step_segmented: bad argument", accs, ns, count, codes_out, codes_in, luts_in, 1.0f, luts_out,
+                         qparams_out, ws, stream);
+}
+
+int prime_ring_reduce_div_step_segmented(float* const* accs, const uint8_t* const* codes_in, const float* const* luts_in, const int64_t* ns,
+                                         int64_t count, float divisor, uint8_t* const* codes_out, float* luts_out,
+                                         prime_qparams* qparams_out, void* ws, prime_stream_t stream) {
+    return run_segmented(kSegReduceDiv, "prime_ring_reduce_div_step_segmented: bad argument", accs, ns, count, codes_out, codes_in, luts_in, divisor,
+                         luts_out, qparams_out, ws, stream);
+}
+
+int prime_ring_gather_step_segmented(float* const* chunks, const uint8_t* const* codes_in, const float* const* luts_in, const int64_t* ns,
+                                     int64_t count, uint8_t* const* codes_out, float* luts_out, prime_qparams* qparams_out, void* ws,
+                                     prime_stream_t stream) {
+    return run_segmented(kSegGather, "prime_ring_gather_step_segmented: bad argument", chunks, ns, count, codes_out, codes_in, luts_in, 1.0f, luts_out,
+                         qparams_out, ws, stream);
 }
 
 int prime_div_f32(float* x, int64_t n, float divisor, prime_stream_t stream) {

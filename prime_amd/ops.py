@@ -594,3 +594,109 @@ def quantize_buckets(tensors, n_streams: int = PIPELINE_STREAMS):
         qps = torch.empty((len(xs), 4), dtype=torch.float64, device=dev)
     BucketPlan(xs, codes, luts, qps, n_streams).run()
     return codes, luts, qps
+
+
+# --------------------------------------------------------------------------------------------
+# Segmented launches: many mid-size tensors (the 2 * world_size chunks the ring cuts a layer
+# bucket into, collectives.cpp:89-90; the chunks all simulated ranks work on in one step) in
+# three kernel launches in all instead of three per tensor.
+
+SEG_UNIFORM, SEG_REDUCE, SEG_GATHER, SEG_REDUCE_DIV = "uniform", "reduce", "gather", "reduce_div"
+
+
+class SegmentPlan:
+    """Pointer tables of one segmented call, built once and replayed (``run``): ``tensors`` are the
+    fp32 tensors (``uniform``) or the ring chunks that a step updates in place; ``codes_in`` /
+    ``luts_in`` the received messages of a ring step.  Outputs: ``codes`` (one uint8 tensor per
+    input, allocated here unless given), ``luts`` [count, 256] float32 and ``qparams`` [count, 4]
+    float64 words.  Results equal the one-tensor ops' bit for bit."""
+
+    def __init__(self, kind: str, tensors, codes_in=None, luts_in=None, divisor: float = 1.0, codes=None,
+                 luts: Optional[torch.Tensor] = None, qparams: Optional[torch.Tensor] = None):
+        import ctypes
+
+        if kind not in (SEG_UNIFORM, SEG_REDUCE, SEG_GATHER, SEG_REDUCE_DIV):
+            raise ValueError(f"unknown segmented operation {kind!r}")
+        if len(tensors) == 0:
+            raise RuntimeError("segmented call: no tensors")
+        ring = kind != SEG_UNIFORM
+        if ring and (codes_in is None or luts_in is None or len(codes_in) != len(tensors) or len(luts_in) != len(tensors)):
+            raise RuntimeError("segmented ring step: one (codes_in, lut_in) message per chunk is needed")
+        dev = tensors[0].device
+        n = len(tensors)
+        xs = []
+        for t in tensors:
+            _need_f32(t, "segmented call")
+            if t.device != dev or not t.is_cuda:
+                raise RuntimeError("segmented call: all tensors must live on one ROCm device")
+            if ring and not t.is_contiguous():
+                raise RuntimeError("segmented ring step: chunks must be contiguous (they are updated in place)")
+            xs.append(t if t.is_contiguous() else t.contiguous())
+        cin, lin = [], []
+        if ring:
+            for t, c, l in zip(xs, codes_in, luts_in):
+                _need_u8(c, "segmented ring step")
+                if c.numel() != t.numel():
+                    raise RuntimeError("segmented ring step: chunk and codes_in differ in numel")
+                cin.append(c.contiguous())
+                lin.append(_need_lut(l, "segmented ring step"))
+        with _on(dev):
+            if codes is None:
+                codes = [torch.empty(t.shape, dtype=torch.uint8, device=dev) for t in xs]
+            if luts is None:
+                luts = torch.empty((n, N_BINS), dtype=torch.float32, device=dev)
+        for t, c in zip(xs, codes):
+            _need_u8(c, "segmented call")
+            if c.numel() != t.numel() or not c.is_contiguous() or c.device != dev:
+                raise RuntimeError("segmented call: codes must be contiguous uint8 tensors of the inputs' sizes on their device")
+        if luts.shape != (n, N_BINS) or luts.dtype != torch.float32 or not luts.is_contiguous() or luts.device != dev:
+            raise RuntimeError("segmented call: luts must be a contiguous float32 [count, 256] tensor")
+        if qparams is not None and (qparams.shape != (n, 4) or qparams.dtype != torch.float64 or not qparams.is_contiguous()):
+            raise RuntimeError("segmented call: qparams must be a contiguous float64 [count, 4] tensor")
+        self.kind, self.dev, self.count, self.divisor = kind, dev, n, float(divisor)
+        self.codes, self.luts, self.qparams = list(codes), luts, qparams
+        self.keep = (xs, cin, lin)                   # the tables hold raw pointers
+        self.xs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in xs])
+        self.ns = (ctypes.c_int64 * n)(*[t.numel() for t in xs])
+        self.cs = (ctypes.c_void_p * n)(*[c.data_ptr() for c in self.codes])
+        self.ci = (ctypes.c_void_p * n)(*[c.data_ptr() for c in cin]) if ring else None
+        self.li = (ctypes.c_void_p * n)(*[l.data_ptr() for l in lin]) if ring else None
+
+    def run(self) -> None:
+        lib = _lib.load()
+        dev = self.dev
+        with _on(dev):
+            st = _stream(dev)
+            ws = workspace(dev, st).data_ptr()
+            qp = self.qparams.data_ptr() if self.qparams is not None else None
+            lp = self.luts.data_ptr()
+            if self.kind == SEG_UNIFORM:
+                rc = lib.prime_uniform_8bit_quantize_segmented(self.xs, self.ns, self.count, self.cs, lp, qp, ws, st)
+            elif self.kind == SEG_REDUCE:
+                rc = lib.prime_ring_reduce_step_segmented(self.xs, self.ci, self.li, self.ns, self.count, self.cs, lp, qp, ws, st)
+            elif self.kind == SEG_GATHER:
+                rc = lib.prime_ring_gather_step_segmented(self.xs, self.ci, self.li, self.ns, self.count, self.cs, lp, qp, ws, st)
+            else:
+                rc = lib.prime_ring_reduce_div_step_segmented(self.xs, self.ci, self.li, self.ns, self.count, self.divisor, self.cs, lp,
+                                                              qp, ws, st)
+            if rc:
+                _lib.check(rc, f"segmented {self.kind}")
+
+
+def uniform_8bit_quantize_segmented(tensors, want_qparams: bool = False):
+    """uniform_8bit_quantize of every tensor in ``tensors`` in three launches per 64 tensors.
+    Returns (list of codes, luts [count, 256]) and, with ``want_qparams``, qparams [count, 4]."""
+    qps = torch.empty((len(tensors), 4), dtype=torch.float64, device=tensors[0].device) if want_qparams and len(tensors) else None
+    plan = SegmentPlan(SEG_UNIFORM, tensors, qparams=qps)
+    plan.run()
+    codes = [c.view(t.shape) for c, t in zip(plan.codes, tensors)]
+    return (codes, plan.luts, qps) if want_qparams else (codes, plan.luts)
+
+
+def ring_step_segmented(kind: str, chunks, codes_in, luts_in, divisor: float = 1.0):
+    """ring_reduce_step / ring_gather_step / ring_reduce_div_step on every chunk of ``chunks`` (in
+    place) with its received message, in three launches.  Returns (list of codes, luts [count, 256]);
+    row i of luts goes with codes i."""
+    plan = SegmentPlan(kind, chunks, codes_in, luts_in, divisor)
+    plan.run()
+    return plan.codes, plan.luts

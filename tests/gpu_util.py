@@ -114,3 +114,38 @@ class Abi:
 def announce(msg: str) -> None:
     """Name the case before its GPU step, flushed, so a lost box still tells which one ran."""
     print(f"[gpu-case] {msg}", flush=True)
+
+
+def _ptrs(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def segmented_uniform(abi: Abi, xs):
+    """prime_uniform_8bit_quantize_segmented on a list of device tensors."""
+    count = len(xs)
+    codes = [torch.empty(x.numel(), dtype=torch.uint8, device=abi.dev) for x in xs]
+    luts = torch.empty((count, 256), dtype=torch.float32, device=abi.dev)
+    qps = torch.empty((count, 4), dtype=torch.float64, device=abi.dev)
+    ns = (ctypes.c_int64 * count)(*[x.numel() for x in xs])
+    _lib.check(abi.lib.prime_uniform_8bit_quantize_segmented(_ptrs(xs), ns, count, _ptrs(codes), luts.data_ptr(), qps.data_ptr(),
+                                                             abi.ws.data_ptr(), abi.st), "uniform_segmented")
+    return codes, luts, qps
+
+
+def segmented_ring_step(abi: Abi, kind: str, accs, codes_in, luts_in, divisor: float = 1.0):
+    """prime_ring_{reduce,gather,reduce_div}_step_segmented on lists of device tensors (accs in place)."""
+    count = len(accs)
+    codes = [torch.empty(a.numel(), dtype=torch.uint8, device=abi.dev) for a in accs]
+    luts = torch.empty((count, 256), dtype=torch.float32, device=abi.dev)
+    qps = torch.empty((count, 4), dtype=torch.float64, device=abi.dev)
+    ns = (ctypes.c_int64 * count)(*[a.numel() for a in accs])
+    args = (_ptrs(accs), _ptrs(codes_in), _ptrs(luts_in), ns, count)
+    tail = (_ptrs(codes), luts.data_ptr(), qps.data_ptr(), abi.ws.data_ptr(), abi.st)
+    if kind == "reduce":
+        rc = abi.lib.prime_ring_reduce_step_segmented(*args, *tail)
+    elif kind == "gather":
+        rc = abi.lib.prime_ring_gather_step_segmented(*args, *tail)
+    else:
+        rc = abi.lib.prime_ring_reduce_div_step_segmented(*args, ctypes.c_float(divisor), *tail)
+    _lib.check(rc, f"ring_{kind}_step_segmented")
+    return codes, luts, qps
