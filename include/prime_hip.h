@@ -306,6 +306,21 @@ int prime_outer_sgd_nesterov_u8(float* param, float* momentum_buf, const uint8_t
                                 float* inner_out, int64_t n, float lr, float momentum, int first_step,
                                 prime_stream_t stream);
 
+/* The two loops over the parameter list either side of the all-reduce as one launch per 64 tensors:
+ * prime_pseudo_gradient_f32 for every parameter (the loop of diloco.py:93-99) and
+ * prime_outer_sgd_nesterov_f32 for every parameter (the outer optimizer's step over its parameters
+ * and sync_inner_model, diloco.py:212-215, :137-144).  Host arrays of `count` device pointers and
+ * sizes, read before the call returns; inner_outs may be NULL, and so may single entries of it.
+ * Elementwise arithmetic: results are those of the one-tensor calls.  Empty tensors are skipped;
+ * tensors not aligned to 16 bytes take the one-tensor entry point inside the call. */
+int prime_pseudo_gradient_f32_segmented(const float* const* outers, const float* const* inners,
+                                        const int64_t* ns, int64_t count, float world_size,
+                                        float* const* outs, prime_stream_t stream);
+int prime_outer_sgd_nesterov_f32_segmented(float* const* params, float* const* momentum_bufs,
+                                           const float* const* grads, float* const* inner_outs,
+                                           const int64_t* ns, int64_t count, float lr, float momentum,
+                                           int first_step, prime_stream_t stream);
+
 /* A plain device copy of n bytes (16-byte vectors): the yardstick the profiler's byte
  * counters are scaled against.  No counterpart in the reference. */
 int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t stream);

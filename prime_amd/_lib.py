@@ -79,6 +79,8 @@ SIGNATURES = {
     "prime_ring_first_touch": (ctypes.c_int, [_vp, _vp, _i64, _f32, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp, _vp]),
     "prime_outer_sgd_nesterov_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _f32, _f32, ctypes.c_int, _vp]),
     "prime_outer_sgd_nesterov_u8": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _f32, _f32, ctypes.c_int, _vp]),
+    "prime_pseudo_gradient_f32_segmented": (ctypes.c_int, [_vp, _vp, _vp, _i64, _f32, _vp, _vp]),
+    "prime_outer_sgd_nesterov_f32_segmented": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _f32, _f32, ctypes.c_int, _vp]),
     "prime_copy_bytes": (ctypes.c_int, [_vp, _vp, _i64, _vp]),
 }
 

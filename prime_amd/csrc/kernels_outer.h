@@ -45,14 +45,15 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
 // (src/zeroband/diloco.py:93-101): grad = outer_param - inner_param, then the whole flat buffer
 // divided by the world size; an fp32 subtraction and an fp32 division per element.
 // 12 bytes per element.
-template <bool ALIGNED, bool NT, int POLICY, bool ONESHOT = false>
-__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer, const float* __restrict__ inner, int64_t n,
-                                            float world_size, float* __restrict__ out) {
+// pseudo_gradient_block is the pass for the calling workgroup as workgroup `slot` of a grid of G.
+template <bool ALIGNED, bool NT, int POLICY, bool ONESHOT>
+__device__ __forceinline__ void pseudo_gradient_block(const float* __restrict__ outer, const float* __restrict__ inner, int64_t n,
+                                                      float world_size, float* __restrict__ out, int64_t slot, int64_t G) {
     using M = Mem<ALIGNED, NT>;
     const int64_t nvec = n >> 2;
     constexpr int T = ONESHOT ? kShotThreads : kThreads;
     constexpr int U = ONESHOT ? kShotUnroll : kDivUnroll;
-    walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+    walk_tiles_of<T, U, ONESHOT>(nvec, slot, G, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         const Window win(out + base * 4, (nvec - base) * 16);
@@ -74,10 +75,16 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
             }
         }
     });
-    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    if (slot == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
         out[i] = (outer[i] - inner[i]) / world_size;
     }
+}
+
+template <bool ALIGNED, bool NT, int POLICY, bool ONESHOT = false>
+__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer, const float* __restrict__ inner, int64_t n,
+                                            float world_size, float* __restrict__ out) {
+    pseudo_gradient_block<ALIGNED, NT, POLICY, ONESHOT>(outer, inner, n, world_size, out, blockIdx.x, gridDim.x);
 }
 
 // A chunk's first touch in the ring when the pseudo-gradient has not been written yet: every
@@ -170,20 +177,21 @@ __device__ __forceinline__ void outer_sgd_one(float& p, float& buf, float g, flo
 // the inner model (sync_inner_model, :137-144) in the same pass.  The gradient is fp32
 // (24 bytes per element) or, with CODES, uint8 codes and their lookup table (21 bytes per
 // element, and the dequantize pass is saved).
-template <bool CODES, bool ALIGNED, bool NT, int POLICY, bool ONESHOT = false>
-__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom, const float* __restrict__ grad,
-                                       const uint8_t* __restrict__ codes, const float* __restrict__ lut, float* __restrict__ inner,
-                                       int64_t n, float neg_lr, float mu, int first) {
+// outer_step_block is the pass for the calling workgroup as workgroup `slot` of a grid of G (s_lut: 256
+// floats of LDS, used with CODES).
+template <bool CODES, bool ALIGNED, bool NT, int POLICY, bool ONESHOT>
+__device__ __forceinline__ void outer_step_block(float* __restrict__ param, float* __restrict__ mom, const float* __restrict__ grad,
+                                                 const uint8_t* __restrict__ codes, const float* __restrict__ lut, float* __restrict__ inner,
+                                                 int64_t n, float neg_lr, float mu, int first, int64_t slot, int64_t G, float* s_lut) {
     using M = Mem<ALIGNED, NT>;
     constexpr int T = ONESHOT ? kShotThreads : kThreads;
     constexpr int U = ONESHOT ? kShotUnroll : kUnroll;
-    __shared__ float s_lut[kBins];
     if (CODES) {
         for (int b = threadIdx.x; b < kBins; b += T) s_lut[b] = lut[b];
         __syncthreads();
     }
     const int64_t nvec = n >> 2;
-    walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+    walk_tiles_of<T, U, ONESHOT>(nvec, slot, G, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         const Window wp(param + base * 4, (nvec - base) * 16), wm(mom + base * 4, (nvec - base) * 16),
@@ -226,7 +234,7 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
             }
         }
     });
-    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+    if (slot == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
         float p = param[i];
         float m = first ? 0.f : mom[i];
@@ -236,6 +244,14 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
         mom[i] = m;
         if (inner) inner[i] = p;
     }
+}
+
+template <bool CODES, bool ALIGNED, bool NT, int POLICY, bool ONESHOT = false>
+__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom, const float* __restrict__ grad,
+                                       const uint8_t* __restrict__ codes, const float* __restrict__ lut, float* __restrict__ inner,
+                                       int64_t n, float neg_lr, float mu, int first) {
+    __shared__ float s_lut[CODES ? kBins : 1];
+    outer_step_block<CODES, ALIGNED, NT, POLICY, ONESHOT>(param, mom, grad, codes, lut, inner, n, neg_lr, mu, first, blockIdx.x, gridDim.x, s_lut);
 }
 
 template <int POLICY, bool ONESHOT = false>

@@ -173,3 +173,32 @@ __global__ __launch_bounds__(kFinalThreads) void seg_lut_finalize_kernel(const S
         luts[static_cast<int64_t>(t) * kBins + b] = mean_entry(sum, cnt);
     }
 }
+
+// ---- elementwise passes over many tensors ---------------------------------------------------------
+// The per-parameter loops either side of the all-reduce (src/zeroband/diloco.py:93-99 and the outer
+// optimizer's step over its parameter list, :72-74, :212-215) as one launch: one 256-lane workgroup
+// per tile of each tensor.  Elementwise arithmetic: the results are the one-tensor kernels'.
+struct SegPointwiseJob {
+    int count;
+    int first[kSegMax + 1];              // workgroups [first[t], first[t + 1]) belong to tensor t
+    int64_t n[kSegMax];
+    float* a[kSegMax];                   // pseudo-gradient: outer      outer step: param
+    float* b[kSegMax];                   //                  inner                  momentum buffer
+    float* c[kSegMax];                   //                  out                    gradient
+    float* d[kSegMax];                   //                                         inner model (may be null)
+};
+static_assert(sizeof(SegPointwiseJob) <= 4000, "the descriptors must fit the kernel argument segment");
+
+template <int POLICY>
+__global__ __launch_bounds__(kShotThreads, 8) void seg_pseudo_gradient_kernel(const SegPointwiseJob job, float world_size) {
+    const int t = seg_tensor_of(job.first, job.count, blockIdx.x);
+    pseudo_gradient_block<true, true, POLICY, true>(job.a[t], job.b[t], job.n[t], world_size, job.c[t], blockIdx.x - job.first[t],
+                                                   job.first[t + 1] - job.first[t]);
+}
+
+template <int POLICY>
+__global__ __launch_bounds__(kShotThreads, 8) void seg_outer_step_kernel(const SegPointwiseJob job, float neg_lr, float mu, int first) {
+    const int t = seg_tensor_of(job.first, job.count, blockIdx.x);
+    outer_step_block<false, true, true, POLICY, true>(job.a[t], job.b[t], job.c[t], nullptr, nullptr, job.d[t], job.n[t], neg_lr, mu, first,
+                                                     blockIdx.x - job.first[t], job.first[t + 1] - job.first[t], nullptr);
+}

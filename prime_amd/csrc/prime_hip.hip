@@ -139,14 +139,15 @@ int launch_check(const char* where) {
 enum KernelId {
     kIdStats, kIdStatsFinalize, kIdQuantize, kIdQuantizeHist, kIdHist, kIdLutFinalize, kIdDequantSet, kIdDequantAdd,
     kIdDequantAddStats, kIdDequantSetStats, kIdBatched, kIdCopy, kIdFill, kIdPseudoGrad, kIdOuterStep, kIdOuterStepCodes, kIdDiv, kIdFirstTouchCodes, kIdCodeCount, kIdCodeTotal, kIdRequantPlan, kIdCodeRemap, kIdNormLiteral, kIdUniformSmall,
-    kIdSegStats, kIdSegDequantAdd, kIdSegDequantSet, kIdSegQuantize, kIdSegLutFinalize, kIdCount
+    kIdSegStats, kIdSegDequantAdd, kIdSegDequantSet, kIdSegQuantize, kIdSegLutFinalize, kIdSegPseudoGrad, kIdSegOuterStep, kIdCount
 };
 const char* const kKernelNames[kIdCount] = {
     "stats_kernel", "stats_finalize_kernel", "quantize_kernel", "quantize_kernel+hist", "hist_kernel", "lut_finalize_kernel",
     "dequant_kernel<set>", "dequant_kernel<add>", "dequant_kernel<add,stats>", "dequant_kernel<set,stats>",
     "batched_kernel", "copy_kernel", "fill_zero_kernel", "pseudo_gradient_kernel", "outer_step_kernel", "outer_step_kernel<codes>", "div_kernel",
     "first_touch_kernel<codes>", "code_count_kernel", "code_total_kernel", "requant_plan_kernel", "code_remap_kernel", "norm_literal_kernel", "uniform_small_kernel",
-    "seg_stats_kernel", "seg_dequant_kernel<add,stats>", "seg_dequant_kernel<set,stats>", "seg_quantize_kernel+hist", "seg_lut_finalize_kernel"};
+    "seg_stats_kernel", "seg_dequant_kernel<add,stats>", "seg_dequant_kernel<set,stats>", "seg_quantize_kernel+hist", "seg_lut_finalize_kernel",
+    "seg_pseudo_gradient_kernel", "seg_outer_step_kernel"};
 
 struct TimedLaunch {
     int id;
@@ -1101,6 +1102,89 @@ int prime_outer_sgd_nesterov_u8(float* param, float* momentum_buf, const uint8_t
         launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, false, false, kStorePlain>, grid, kThreads, st, param, momentum_buf, no_grad, codes,
                lut, inner_out, n, -lr, momentum, first_step);
     return launch_check("outer_step_kernel");
+}
+
+int prime_pseudo_gradient_f32_segmented(const float* const* outers, const float* const* inners, const int64_t* ns, int64_t count,
+                                        float world_size, float* const* outs, prime_stream_t stream) {
+    if (count < 0 || (count > 0 && (!outers || !inners || !ns || !outs))) return fail(PRIME_EINVAL, "prime_pseudo_gradient_f32_segmented: bad argument");
+    for (int64_t i = 0; i < count; ++i)
+        if (bad_n(ns[i]) || (ns[i] > 0 && (!outers[i] || !inners[i] || !outs[i])))
+            return fail(PRIME_EINVAL, "prime_pseudo_gradient_f32_segmented: bad argument");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    SegPointwiseJob job;
+    auto flush = [&]() -> int {
+        if (job.count == 0) return 0;
+        double bytes = 0.0;
+        for (int t = 0; t < job.count; ++t) bytes += 12.0 * job.n[t];
+        with_policy(g_opt.one_shot_store_policy, [&](auto P) {
+            launch(kIdSegPseudoGrad, bytes, seg_pseudo_gradient_kernel<decltype(P)::value>, job.first[job.count], kShotThreads, st, job, world_size);
+        });
+        job.count = 0;
+        return launch_check("seg_pseudo_gradient_kernel");
+    };
+    memset(&job, 0, sizeof(job));
+    for (int64_t i = 0; i < count; ++i) {
+        if (ns[i] == 0) continue;
+        const bool al = aligned_to(outers[i], 16) && aligned_to(inners[i], 16) && aligned_to(outs[i], 16);
+        if (!al || ns[i] > (int64_t(1) << 34)) {         // the one-tensor entry point takes what a one-workgroup-per-tile launch cannot
+            if (int rc = prime_pseudo_gradient_f32(outers[i], inners[i], ns[i], world_size, outs[i], stream)) return rc;
+            continue;
+        }
+        const int blocks = shot_grid(ns[i] >> 2) > 0 ? shot_grid(ns[i] >> 2) : 1;
+        if (job.count == kSegMax || job.first[job.count] + static_cast<int64_t>(blocks) > 0x7fffffff)
+            if (int rc = flush()) return rc;
+        const int t = job.count++;
+        job.n[t] = ns[i];
+        job.a[t] = const_cast<float*>(outers[i]);
+        job.b[t] = const_cast<float*>(inners[i]);
+        job.c[t] = outs[i];
+        job.first[t + 1] = job.first[t] + blocks;
+    }
+    return flush();
+}
+
+int prime_outer_sgd_nesterov_f32_segmented(float* const* params, float* const* momentum_bufs, const float* const* grads,
+                                           float* const* inner_outs, const int64_t* ns, int64_t count, float lr, float momentum,
+                                           int first_step, prime_stream_t stream) {
+    if (count < 0 || (count > 0 && (!params || !momentum_bufs || !grads || !ns)))
+        return fail(PRIME_EINVAL, "prime_outer_sgd_nesterov_f32_segmented: bad argument");
+    for (int64_t i = 0; i < count; ++i)
+        if (bad_n(ns[i]) || (ns[i] > 0 && (!params[i] || !momentum_bufs[i] || !grads[i])))
+            return fail(PRIME_EINVAL, "prime_outer_sgd_nesterov_f32_segmented: bad argument");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    SegPointwiseJob job;
+    auto flush = [&]() -> int {
+        if (job.count == 0) return 0;
+        double bytes = 0.0;
+        for (int t = 0; t < job.count; ++t) bytes += (job.d[t] ? 24.0 : 20.0) * job.n[t];
+        with_policy(g_opt.one_shot_store_policy, [&](auto P) {
+            launch(kIdSegOuterStep, bytes, seg_outer_step_kernel<decltype(P)::value>, job.first[job.count], kShotThreads, st, job, -lr, momentum,
+                   first_step);
+        });
+        job.count = 0;
+        return launch_check("seg_outer_step_kernel");
+    };
+    memset(&job, 0, sizeof(job));
+    for (int64_t i = 0; i < count; ++i) {
+        if (ns[i] == 0) continue;
+        float* inner = inner_outs ? inner_outs[i] : nullptr;
+        const bool al = aligned_to(params[i], 16) && aligned_to(momentum_bufs[i], 16) && aligned_to(grads[i], 16) && aligned_to(inner, 16);
+        if (!al || ns[i] > (int64_t(1) << 34)) {
+            if (int rc = prime_outer_sgd_nesterov_f32(params[i], momentum_bufs[i], grads[i], inner, ns[i], lr, momentum, first_step, stream)) return rc;
+            continue;
+        }
+        const int blocks = shot_grid(ns[i] >> 2) > 0 ? shot_grid(ns[i] >> 2) : 1;
+        if (job.count == kSegMax || job.first[job.count] + static_cast<int64_t>(blocks) > 0x7fffffff)
+            if (int rc = flush()) return rc;
+        const int t = job.count++;
+        job.n[t] = ns[i];
+        job.a[t] = params[i];
+        job.b[t] = momentum_bufs[i];
+        job.c[t] = const_cast<float*>(grads[i]);
+        job.d[t] = inner;
+        job.first[t + 1] = job.first[t] + blocks;
+    }
+    return flush();
 }
 
 int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t stream) {

@@ -12,7 +12,7 @@ side of the compressed all-reduce:
 
 The reference keeps the outer copy, the gradient and the optimizer state in host memory and
 pays a device-to-host copy of every parameter per outer step; with 288 GB of HBM they stay on
-the device: the pseudo-gradient is one fused kernel per parameter, and the optimizer step
+the device: the pseudo-gradient is one fused launch per 64 parameters, and the optimizer step
 and the copy back to the model are one more.  Elastic membership, retries and the barrier of
 the reference (:84,:92-126) belong to its control plane and are not here.
 
@@ -122,8 +122,10 @@ class Diloco:
         if self._inner_is_flat(model):
             ops.pseudo_gradient_(self.grad_flat, self.outer_data_flat, self.inner_flat, float(world_size))
             return
-        for (outer, grad, _), p in zip(self._views, self._params(model)):
-            ops.pseudo_gradient_(grad, outer, p.data.view(-1), float(world_size))
+        # one launch per 64 parameters instead of one per parameter
+        ps = self._params(model)
+        ops.pseudo_gradient_segmented_([v[1] for v in self._views], [v[0] for v in self._views], [p.data.view(-1) for p in ps],
+                                       float(world_size))
 
     @torch.no_grad()
     def all_reduce_buckets(self, group: Optional[object]) -> None:
@@ -133,15 +135,16 @@ class Diloco:
 
     @torch.no_grad()
     def outer_step(self, model: nn.Module) -> None:
-        """outer_optimizer.step() and sync_inner_model (diloco.py:212-215), one kernel per parameter
+        """outer_optimizer.step() and sync_inner_model (diloco.py:212-215), one launch per 64 parameters
         (one for the whole model when the inner parameters are flat)."""
         if self._inner_is_flat(model):
             ops.outer_sgd_nesterov_(self.outer_data_flat, self.momentum_flat, self.grad_flat, self.inner_flat, self.outer_lr,
                                     OUTER_MOMENTUM, self._first_step)
             self._first_step = False
             return
-        for (outer, grad, mom), p in zip(self._views, self._params(model)):
-            ops.outer_sgd_nesterov_(outer, mom, grad, p.data.view(-1), self.outer_lr, OUTER_MOMENTUM, self._first_step)
+        ps = self._params(model)
+        ops.outer_sgd_nesterov_segmented_([v[0] for v in self._views], [v[2] for v in self._views], [v[1] for v in self._views],
+                                          [p.data.view(-1) for p in ps], self.outer_lr, OUTER_MOMENTUM, self._first_step)
         self._first_step = False
 
     @torch.no_grad()

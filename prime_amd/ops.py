@@ -700,3 +700,51 @@ def ring_step_segmented(kind: str, chunks, codes_in, luts_in, divisor: float = 1
     plan = SegmentPlan(kind, chunks, codes_in, luts_in, divisor)
     plan.run()
     return plan.codes, plan.luts
+
+
+def _ptr_table(tensors):
+    import ctypes
+
+    return (ctypes.c_void_p * len(tensors))(*[None if t is None else t.data_ptr() for t in tensors])
+
+
+def pseudo_gradient_segmented_(outs, outers, inners, world_size: float) -> None:
+    """``pseudo_gradient_`` for every parameter of a list in one launch per 64 tensors: the loop of
+    src/zeroband/diloco.py:93-99 with both copies of the parameters on the device."""
+    import ctypes
+
+    if not (len(outs) == len(outers) == len(inners)):
+        raise RuntimeError("pseudo_gradient_segmented_: the three lists differ in length")
+    if not outs:
+        return
+    for o, a, b in zip(outs, outers, inners):
+        n = o.numel()
+        for t in (o, a, b):
+            _need_flat_f32(t, "pseudo_gradient_segmented_", n)
+    dev = outs[0].device
+    ns = (ctypes.c_int64 * len(outs))(*[o.numel() for o in outs])
+    with _on(dev):
+        _lib.check(_lib.load().prime_pseudo_gradient_f32_segmented(_ptr_table(outers), _ptr_table(inners), ns, len(outs), float(world_size),
+                                                                   _ptr_table(outs), _stream(dev)), "prime_pseudo_gradient_f32_segmented")
+
+
+def outer_sgd_nesterov_segmented_(params, momentum_bufs, grads, inners, lr: float, momentum: float, first_step: bool) -> None:
+    """``outer_sgd_nesterov_`` for every parameter of a list in one launch per 64 tensors
+    (src/zeroband/diloco.py:212-215, :137-144).  ``inners`` may be None or hold None entries."""
+    import ctypes
+
+    if not (len(params) == len(momentum_bufs) == len(grads)) or (inners is not None and len(inners) != len(params)):
+        raise RuntimeError("outer_sgd_nesterov_segmented_: the lists differ in length")
+    if not params:
+        return
+    for i, (p, m, g) in enumerate(zip(params, momentum_bufs, grads)):
+        n = p.numel()
+        for t in (p, m, g) + ((inners[i],) if inners is not None and inners[i] is not None else ()):
+            _need_flat_f32(t, "outer_sgd_nesterov_segmented_", n)
+    dev = params[0].device
+    ns = (ctypes.c_int64 * len(params))(*[p.numel() for p in params])
+    with _on(dev):
+        _lib.check(_lib.load().prime_outer_sgd_nesterov_f32_segmented(_ptr_table(params), _ptr_table(momentum_bufs), _ptr_table(grads),
+                                                                      _ptr_table(inners) if inners is not None else None, ns, len(params),
+                                                                      float(lr), float(momentum), int(first_step), _stream(dev)),
+                   "prime_outer_sgd_nesterov_f32_segmented")

@@ -96,10 +96,14 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
 
     own: dict = {}     # (rank, chunk) -> (codes, lut) of the rank's reduced chunk, not yet written back
     final: List[List] = [[None] * nb for _ in range(W)]
+    div = float(W) if avg else 1.0
     for phase in (1, 2):
         inbox: List[dict] = [dict() for _ in range(W)]
         for step in range(1, nb + 1):
             posted = []
+            # What every rank does in this step.  The W ranks' work of one kind is independent, so it goes to
+            # the device as one segmented call (three launches for all ranks) instead of three launches per rank.
+            batch: dict = {}       # kind -> list of (rank, chunk index, chunk, message)
             for r in range(W):
                 if phase == 1:
                     c = (r * BUFFER_COUNT - step) % nb                      # collectives.cpp:116
@@ -109,7 +113,7 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
                 msg = inbox[r].pop(step - BUFFER_COUNT, None)
                 sending = step <= (W - 1) * BUFFER_COUNT                    # :136 / :212
                 if phase == 1 and sources is not None and (msg is not None or sending):
-                    pair = touch(r, c, msg, float(W) if (avg and not sending) else 1.0)
+                    pair = touch(r, c, msg, div if not sending else 1.0)
                     if sending:
                         posted.append(((r + 1) % W, step, pair[0], pair[1]))
                     else:
@@ -121,25 +125,31 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
                         codes, lut = ops.requantize_codes(pair[0], pair[1])     # :215 without the fp32 chunk
                         posted.append(((r + 1) % W, step, codes, lut))
                 elif msg is not None and sending:
-                    if phase == 1:
-                        codes, lut = ops.ring_reduce_step(ch, msg[0], msg[1])   # :128-138 fused
-                    else:
-                        codes, lut = ops.ring_gather_step(ch, msg[0], msg[1])   # :204-215 fused
-                    posted.append(((r + 1) % W, step, codes, lut))
+                    # :128-138 fused (phase 1) / :204-215 fused (phase 2)
+                    batch.setdefault(ops.SEG_REDUCE if phase == 1 else ops.SEG_GATHER, []).append((r, c, ch, msg))
                 elif msg is not None and phase == 1:
                     # the last accumulation into one of the rank's own chunks, its division for AVG
                     # and its quantization in two passes (:128-133, :155-162)
-                    own[(r, c)] = ops.ring_reduce_div_step(ch, msg[0], msg[1], float(W) if avg else 1.0)
+                    batch.setdefault(ops.SEG_REDUCE_DIV, []).append((r, c, ch, msg))
                 elif msg is not None:
                     ops.dequantize_(ch, msg[0], msg[1], False)              # :204-209, nothing forwarded
                 elif sending and (r, c) in own:
                     # the write-back of the rank's own codes (:167-172) and the quantization that
                     # forwards the chunk (:215), as one gather step
-                    codes, lut = ops.ring_gather_step(ch, *own.pop((r, c)))
-                    posted.append(((r + 1) % W, step, codes, lut))
+                    batch.setdefault(ops.SEG_GATHER, []).append((r, c, ch, own.pop((r, c))))
                 elif sending:
-                    codes, lut = ops.uniform_8bit_quantize(ch, False)       # :138
-                    posted.append(((r + 1) % W, step, codes, lut))
+                    batch.setdefault(ops.SEG_UNIFORM, []).append((r, c, ch, None))     # :138
+            for kind, items in batch.items():
+                chunks_k = [it[2] for it in items]
+                if kind == ops.SEG_UNIFORM:
+                    codes_k, luts_k = ops.uniform_8bit_quantize_segmented(chunks_k)
+                else:
+                    codes_k, luts_k = ops.ring_step_segmented(kind, chunks_k, [it[3][0] for it in items], [it[3][1] for it in items], div)
+                for (r, c, _, _), codes, lut in zip(items, codes_k, luts_k):
+                    if kind == ops.SEG_REDUCE_DIV:
+                        own[(r, c)] = (codes, lut)
+                    else:
+                        posted.append(((r + 1) % W, step, codes, lut))
             for dst, st, codes, lut in posted:
                 inbox[dst][st] = (codes, lut)
         if phase == 1 and W == 1:

@@ -156,3 +156,58 @@ def test_segmented_ops_layer(dev, oracle):
     for a, a1, c_in, l_in, c, l in zip(accs, accs1, codes, luts, codes2, luts2):
         c1, l1 = ops.ring_reduce_step(a1, c_in, l_in)
         assert torch.equal(a, a1) and torch.equal(c, c1) and np.array_equal(bits(l), bits(l1))
+
+
+def test_segmented_pointwise_passes_equal_the_one_tensor_calls(dev, oracle):
+    # the per-parameter loops of diloco.py:93-99 and :212-215 as one launch per 64 tensors: 150 parameter-like
+    # tensors, among them empty ones, one of three elements and views that start at an odd element
+    from prime_amd import ops
+
+    rng = np.random.default_rng(35)
+    g = torch.Generator(device=dev).manual_seed(35)
+    sizes = [int(n) for n in rng.integers(1, 300_000, 146)] + [0, 3, 1 << 21, 0]
+    pool = torch.randn(sum(sizes) + 8, device=dev, generator=g)
+
+    def views(shift):
+        out, off = [], shift
+        for n in sizes:
+            out.append(pool[off:off + n])
+            off += n
+        return out
+
+    for shift in (0, 1):                      # shift 1: most views are not 16-byte aligned
+        outers = views(shift)
+        inners = [o + torch.randn(o.numel(), device=dev, generator=g) * 1e-3 for o in outers]
+        grads = [torch.empty_like(o) for o in outers]
+        announce(f"segmented pseudo-gradient, {len(sizes)} tensors, shift {shift}")
+        ops.pseudo_gradient_segmented_(grads, outers, inners, 4.0)
+        for o, i, gr in zip(outers, inners, grads):
+            want = torch.empty_like(o)
+            if o.numel():
+                ops.pseudo_gradient_(want, o, i, 4.0)
+            assert np.array_equal(bits(gr), bits(want))
+            assert np.array_equal(gr.cpu().numpy(), oracle.pseudo_gradient(o.cpu().numpy(), i.cpu().numpy(), 4.0))
+        for first in (True, False):
+            params = [o.clone() for o in outers]
+            moms = [torch.randn(o.numel(), device=dev, generator=g) for o in outers]
+            models = [torch.empty_like(o) for o in outers]
+            p1 = [p.clone() for p in params]
+            m1 = [m.clone() for m in moms]
+            i1 = [torch.empty_like(o) for o in outers]
+            announce(f"segmented outer step, first_step={first}, shift {shift}")
+            ops.outer_sgd_nesterov_segmented_(params, moms, grads, models, 0.7, 0.9, first)
+            for k in range(len(sizes)):
+                if sizes[k]:
+                    ops.outer_sgd_nesterov_(p1[k], m1[k], grads[k], i1[k], 0.7, 0.9, first)
+                    assert np.array_equal(bits(params[k]), bits(p1[k])) and np.array_equal(bits(moms[k]), bits(m1[k]))
+                    assert np.array_equal(bits(models[k]), bits(i1[k]))
+        # without an inner model
+        params = [o.clone() for o in outers]
+        moms = [torch.zeros_like(o) for o in outers]
+        p1 = [p.clone() for p in params]
+        ops.outer_sgd_nesterov_segmented_(params, moms, grads, None, 0.7, 0.9, True)
+        for k in range(len(sizes)):
+            if sizes[k]:
+                m = torch.zeros_like(p1[k])
+                ops.outer_sgd_nesterov_(p1[k], m, grads[k], None, 0.7, 0.9, True)
+                assert np.array_equal(bits(params[k]), bits(p1[k]))
