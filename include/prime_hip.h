@@ -60,11 +60,13 @@ const char* prime_hip_last_error(void);
  * elements instead of four on tensors below this many Mi elements; 0: never),
  * "set_four_rows_max_mi_elems" (the one-workgroup-per-tile dequantize set takes tiles of four rows of
  * 1024 elements instead of two on tensors of at most this many Mi elements; 0: never),
- * "segment_blocks_per_cu" (workgroups per compute unit that the quantize pass of a segmented launch
- * shares out among its tensors), "grid_cap" (upper bound on the workgroups of a looping kernel, for
+ * "dynamic_tail_percent" / "dynamic_tail_min_mi_elems" (the fused quantize + lookup pass hands out this
+ * share of its tiles, the last ones, on demand instead of round-robin, on tensors of at least that many
+ * Mi elements; 0: never), "segment_blocks_per_cu" (workgroups per compute unit that the quantize pass of
+ * a segmented launch shares out among its tensors), "grid_cap" (upper bound on the workgroups of a looping kernel, for
  * experiments; 0: none).
  * Cache policies, load hints, the one-workgroup-per-tile and one-launch variants, the number of LDS
- * copies and segment_blocks_per_cu never change a result.  The options that change the number of
+ * copies, the dynamic tail and segment_blocks_per_cu never change a result.  The options that change the number of
  * workgroups of the statistics pass or its tile shape (blocks_per_cu, grid_cap, large_read_*,
  * two_row_below_mi_elems) change the order in which the fp64 sums are added: codes and scale have been
  * equal on all tested data, but a sum may move in its last bit and, rarely, a scale with it.

@@ -354,6 +354,50 @@ __device__ __forceinline__ void sweep_tiles_of(int64_t nvec, int64_t slot, int64
     if (!REVERSE && r0 < rows) body(r0 * kThreads, G * kThreads, std::false_type{});
 }
 
+// The same walk with the last part of the whole tiles dealt on demand.  The workgroups of a long
+// launch do not finish together (on a 2^28-element pass the first ends 10 % ahead of the last), and
+// tiles that are handed out one by one near the end fill that gap.  `dyn_percent` of the rounds are
+// taken out of the round-robin deal and handed out through `counter` (device memory that holds 0
+// when the launch starts; null: everything stays round-robin): a workgroup asks for its next tile
+// while it streams the one before, so the trip to the counter is not waited for.  Which workgroup
+// gets which of these tiles differs from run to run: only for passes whose per-workgroup results add
+// up to the same totals in any order (integer histogram partials; codes depend on nothing but the
+// element).  Every workgroup of the launch must call this (it uses barriers while tiles are left).
+template <int U, bool REVERSE, typename Body>
+__device__ __forceinline__ void sweep_tiles_dynamic(int64_t nvec, int64_t slot, int64_t G, unsigned* counter, int dyn_percent, Body&& body) {
+    __shared__ unsigned sh_next[2];
+    const int64_t rows = (nvec + kThreads - 1) / kThreads;
+    const int64_t rounds = (nvec / kThreads) / (G * U);
+    const int64_t dyn_rounds = counter ? rounds * dyn_percent / 100 : 0;
+    const int64_t static_rounds = rounds - dyn_rounds;
+    const int64_t dyn_tiles = dyn_rounds * G;
+    const int64_t r0 = rounds * G * U + slot;
+    // forward: static tiles [0, static_rounds * G), then the dynamic ones, then the ragged rows;
+    // reverse: the ragged rows, static tiles from the end down to dyn_tiles, then the dynamic ones [0, dyn_tiles) downwards
+    if (REVERSE && r0 < rows) body(r0 * kThreads, G * kThreads, std::false_type{});
+    for (int64_t kk = 0; kk < static_rounds; ++kk) {
+        const int64_t k = REVERSE ? rounds - 1 - kk : kk;
+        body(((k * G + slot) * U) * kThreads, static_cast<int64_t>(kThreads), std::true_type{});
+    }
+    if (dyn_tiles > 0) {
+        if (threadIdx.x == 0) sh_next[0] = atomicAdd(counter, 1u);
+        __syncthreads();
+        unsigned cur = sh_next[0];
+        int ph = 0;
+        while (cur < dyn_tiles) {
+            unsigned ahead = 0;
+            if (threadIdx.x == 0) ahead = atomicAdd(counter, 1u);          // the tile after this one, asked for while this one streams
+            const int64_t tile = REVERSE ? dyn_tiles - 1 - cur : static_rounds * G + cur;
+            body((tile * U) * kThreads, static_cast<int64_t>(kThreads), std::true_type{});
+            if (threadIdx.x == 0) sh_next[ph ^ 1] = ahead;
+            __syncthreads();
+            cur = sh_next[ph ^ 1];
+            ph ^= 1;
+        }
+    }
+    if (!REVERSE && r0 < rows) body(r0 * kThreads, G * kThreads, std::false_type{});
+}
+
 template <int U = kUnroll, bool REVERSE = false, typename Body>
 __device__ __forceinline__ void sweep_tiles(int64_t nvec, Body&& body) {
     sweep_tiles_of<U, REVERSE>(nvec, blockIdx.x, gridDim.x, body);

@@ -301,6 +301,7 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
 void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
                     float divisor) {
     __shared__ float s_lut[kBins];
+    if (STATS && blockIdx.x == 0 && threadIdx.x == 0) ws->tile_counter = 0u;      // for the quantize pass that follows (sweep_tiles_dynamic)
     dequant_block<ADD, STATS, ALIGNED, NT, DIV, POLICY, ONESHOT, SHOT_ROWS>(out, lut, codes, n, STATS ? ws->part_sum : nullptr,
                                                                            STATS ? ws->part_sq : nullptr, divisor, blockIdx.x, gridDim.x, s_lut);
 }

@@ -104,6 +104,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
                                                                                float* __restrict__ out, Workspace* ws) {
     using M = Mem<ALIGNED, NT>;
     __shared__ float s_lut[kBins];
+    if (blockIdx.x == 0 && threadIdx.x == 0) ws->tile_counter = 0u;      // for the quantize pass that follows (sweep_tiles_dynamic)
     if (CODES) {
         for (int b = threadIdx.x; b < kBins; b += kThreads) s_lut[b] = lut[b];
         __syncthreads();

@@ -37,9 +37,12 @@ struct HistOut {
     FarPart* far;
     HistInfo* info;
     bool first;
+    unsigned* tile_counter;     // deals the last part of the tiles on demand (sweep_tiles_dynamic); null: all round-robin
+    int dyn_percent;
 };
-__device__ __forceinline__ HistOut hist_out_of(Workspace* ws, int slot) {
-    return HistOut{ws ? ws->hist[slot] : nullptr, ws ? &ws->far[slot] : nullptr, ws ? &ws->hist_info : nullptr, slot == 0};
+__device__ __forceinline__ HistOut hist_out_of(Workspace* ws, int slot, int dyn_percent) {
+    return HistOut{ws ? ws->hist[slot] : nullptr, ws ? &ws->far[slot] : nullptr, ws ? &ws->hist_info : nullptr, slot == 0,
+                   ws && dyn_percent > 0 ? &ws->tile_counter : nullptr, dyn_percent};
 }
 
 // K2 (+K3 when HIST): quantize to uint8, 4 codes packed per 32-bit store, and the 256-bin
@@ -81,7 +84,7 @@ __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int6
         constexpr int kMode = decltype(mode_t)::value;
         int since_flush = 0;
         const int flush_rounds = kMode == kFixed ? ResidualHist::flush_rounds(shift) : 0;
-        sweep_tiles_of<U, REVERSE>(nvec, slot, G, [&](int64_t base, int64_t stride, auto full_t) {
+        auto body = [&](int64_t base, int64_t stride, auto full_t) {
             constexpr bool full = decltype(full_t)::value;
             const int64_t i0 = base + threadIdx.x;
             const Window out(codes + base * 4, (nvec - base) * 4);
@@ -127,7 +130,10 @@ __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int6
                 rhist_flush(hist.fixed, shift);       // every lane of the workgroup runs the same rounds
                 since_flush = 0;
             }
-        });
+        };
+        // the fixed-point histogram's partials are integers: its tiles may go to any workgroup
+        if constexpr (kMode == kFixed) sweep_tiles_dynamic<U, REVERSE>(nvec, slot, G, out_part.tile_counter, out_part.dyn_percent, body);
+        else sweep_tiles_of<U, REVERSE>(nvec, slot, G, body);
         if (slot == 0 && threadIdx.x < (n & 3)) {
             const int64_t i = (nvec << 2) + threadIdx.x;
             const float v = x[i];
@@ -166,7 +172,7 @@ __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int6
 template <bool ALIGNED, bool NT, bool HIST, bool REVERSE, int POLICY, int U = kUnroll>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
                                                             int stats_parts, prime_qparams* qp_out, int zero_point,
-                                                            uint8_t* __restrict__ codes, Workspace* ws, int copies_shift) {
+                                                            uint8_t* __restrict__ codes, Workspace* ws, int copies_shift, int dyn_percent) {
     // the scale: given by value, or derived here from the statistics partials of the pass before
     // (stats_parts < 0: the record a preceding kernel left in the workspace)
     int narrow = INT_MIN;                // set when the statistics show a tensor crowded into a few codes
@@ -174,7 +180,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
                       : stats_parts < 0 ? ws->qp.inv_scale
                                         : 1.0f / scale_val;
     __shared__ std::conditional_t<HIST, QuantHist, int> hist_mem;      // no histogram memory without HIST
-    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY, U>(x, n, inv, narrow, zero_point, codes, hist_out_of(HIST ? ws : nullptr, blockIdx.x),
+    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY, U>(x, n, inv, narrow, zero_point, codes, hist_out_of(HIST ? ws : nullptr, blockIdx.x, dyn_percent),
                                                        copies_shift, blockIdx.x, gridDim.x, reinterpret_cast<QuantHist&>(hist_mem));
 }
 

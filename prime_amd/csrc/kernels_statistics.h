@@ -102,6 +102,7 @@ __device__ __forceinline__ void stats_partial_short(const float* __restrict__ x,
 // U = rows per tile: 4 from 2^27 elements up, 2 below (a 51 M-element bucket: 33.3 against 34.4 us).
 template <bool ALIGNED, bool NT, int U = kUnroll>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) ws->tile_counter = 0u;      // for the quantize pass that follows (sweep_tiles_dynamic)
     stats_partial<ALIGNED, NT, U>(x, n, blockIdx.x, gridDim.x, ws->part_sum, ws->part_sq);
 }
 

@@ -15,7 +15,7 @@ import torch
 from prime_amd import _lib
 from tests.conftest import lut_rel_err, tables_agree
 from tests.golden.make_fixtures import CASES, case_input
-from tests.gpu_util import Abi, announce
+from tests.gpu_util import Abi, announce, segmented_uniform
 
 pytestmark = pytest.mark.gpu
 
@@ -455,7 +455,11 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
                                            ("code_store_policy", (0, 2, 16)), ("f32_reread_store_policy", (0, 2, 16)),
                                            ("reverse_second_pass", (0, 1)), ("one_shot", (0, 1)),
                                            ("one_shot_store_policy", (0, 2, 16)), ("two_row_below_mi_elems", (0, 128)),
-                                           ("set_four_rows_max_mi_elems", (0, 32))])
+                                           ("set_four_rows_max_mi_elems", (0, 32)), ("grid_cap", (0, 7, 64)),
+                                           ("large_read_grid_eighths", (0, 3, 7)), ("large_read_min_mi_elems", (0, 128)),
+                                           ("f32_store_policy", (0, 2, 16)), ("copy_store_policy", (0, 2, 16)),
+                                           ("dynamic_tail_percent", (0, 5, 100)), ("dynamic_tail_min_mi_elems", (0, 128)),
+                                           ("segment_blocks_per_cu", (1, 2, 4))])
 def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle, option, values):
     # the options change scheduling and cache hints only: codes, scale and lookup must not move,
     # on ordinary data, on a tensor crowded into a few codes, and through a ring step
@@ -478,8 +482,65 @@ def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle,
                 assert q2["scale"] == oracle.scale_exact(want)
                 oc2, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q2["scale"]))
                 assert np.array_equal(c2.cpu().numpy(), oc2)
+            # the same tensors through one segmented call, and the plain copy
+            xs = [abi.to_dev(v) for v in inputs.values()]
+            sc, sl, sq = segmented_uniform(abi, xs)
+            for i, xt in enumerate(xs):
+                c1, l1, q1 = abi.uniform(xt)
+                assert torch.equal(sc[i], c1) and torch.equal(sl[i].view(torch.int32), l1.view(torch.int32))
+                assert torch.equal(sq[i].view(torch.int64), q1.view(torch.int64))
+            src = xs[0][:700_000]
+            dst = torch.zeros_like(src)
+            _lib.check(abi.lib.prime_copy_bytes(dst.data_ptr(), src.data_ptr(), src.numel() * 4, abi.st), "copy")
+            assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
     finally:
         _lib.set_option(option, old)
+
+
+def test_tiles_dealt_on_demand_give_the_results_of_the_round_robin_deal_bit_for_bit(abi, oracle):
+    # the fused pass may hand out its last tiles through a counter: which workgroup sees which tile then changes
+    # from run to run, the integer histogram partials add up to the same totals, the codes depend on the element
+    # alone.  Tensors with several rounds of tiles (two- and four-row), ordinary data and values beyond the
+    # fixed-point range, through uniform_8bit_quantize and a ring step.
+    rng = np.random.default_rng(77)
+    saved = {k: _lib.get_option(k) for k in ("dynamic_tail_percent", "dynamic_tail_min_mi_elems", "two_row_below_mi_elems")}
+    try:
+        _lib.set_option("dynamic_tail_min_mi_elems", 0)
+        for two_row in (128, 0):
+            _lib.set_option("two_row_below_mi_elems", two_row)
+            n = 9_000_003 if two_row else 13_000_001
+            x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+            x[rng.integers(0, n, 40)] = np.float32(0.9)                  # beyond 628 bins: fp64 side sums
+            xt = abi.to_dev(x)
+            acc0 = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+            want = None
+            for percent in (0, 5, 50, 100, 100):
+                _lib.set_option("dynamic_tail_percent", percent)
+                announce(f"dynamic tail {percent} % n={n} two_row_below={two_row}")
+                codes, lut, qp = abi.uniform(xt)
+                acc = abi.to_dev(acc0)
+                c2, l2, q2 = abi.ring_step(acc, codes, lut)
+                torch.cuda.synchronize()
+                got = [codes.cpu().numpy(), lut.cpu().numpy().view(np.uint32), qp.cpu().numpy().view(np.uint64),
+                       c2.cpu().numpy(), l2.cpu().numpy().view(np.uint32), q2.cpu().numpy().view(np.uint64), acc.cpu().numpy().view(np.uint32)]
+                if want is None:
+                    want = got
+                    q = abi.qparams(qp)
+                    oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
+                    assert q["scale"] == oracle.scale_exact(x) and np.array_equal(got[0], oc)
+                    mean, _ = oracle.average_buckets_f64(x, oc)
+                    assert lut_rel_err(lut.cpu().numpy(), mean, float(q["scale"])) <= LUT_TOL
+                    continue
+                for k, (a, b) in enumerate(zip(got, want)):
+                    # entries 0 and 255 of a table with far elements are fp64 sums in arrival order: compared by value
+                    if k in (1, 4):
+                        assert np.array_equal(a[1:255], b[1:255]), (percent, k)
+                        assert np.allclose(a.view(np.float32)[[0, 255]], b.view(np.float32)[[0, 255]], rtol=1e-6, atol=0), (percent, k)
+                    else:
+                        assert np.array_equal(a, b), (percent, k)
+    finally:
+        for k, v in saved.items():
+            _lib.set_option(k, v)
 
 
 def _small_inputs(n, rng):
