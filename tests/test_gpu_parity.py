@@ -543,6 +543,66 @@ def test_tiles_dealt_on_demand_give_the_results_of_the_round_robin_deal_bit_for_
             _lib.set_option(k, v)
 
 
+def check_special(abi, oracle, x: np.ndarray, label: str):
+    """check_uniform for tensors whose statistics are not finite numbers: scale bit for bit (NaN equal to NaN),
+    codes bit-exact against the oracle under that scale, counts exact, table against the fp64 bin means with
+    NaN and infinite entries in the same places."""
+    announce(f"{label} n={x.size}")
+    xt = abi.to_dev(x)
+    codes, lut, qp = abi.uniform(xt)
+    torch.cuda.synchronize()
+    q = abi.qparams(qp)
+    gc, gl = codes.cpu().numpy(), lut.cpu().numpy()
+    want_scale = oracle.scale_exact(x)
+    assert np.array_equal(np.array([q["scale"]]), np.array([want_scale]), equal_nan=True), (label, q["scale"], want_scale)
+    oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
+    assert np.array_equal(gc, oc), (label, int((gc != oc).sum()))
+    mean, cnt = oracle.average_buckets_f64(x, gc)
+    floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1e-3
+    assert lut_rel_err(gl, mean, floor) <= LUT_TOL, (label, gl[cnt > 0], mean[cnt > 0])
+    assert not gl[cnt == 0].any(), label
+    _, cnt2 = abi.average_buckets(xt, codes)
+    assert np.array_equal(cnt2.cpu().numpy(), cnt), label
+    return xt, codes, lut, q
+
+
+@pytest.mark.parametrize("n", [65_543, (1 << 20) + 3])
+def test_special_values_on_the_multi_workgroup_path_against_the_oracle(abi, oracle, n):
+    # a NaN, an infinity, squares beyond fp32 and a norm beyond fp32 at sizes that take several workgroups:
+    # the branches of the fused pass for a 1 / scale that is NaN (every code 0, one fp64 sum) or zero (fp64
+    # histogram), through uniform_8bit_quantize and through a ring step whose accumulator holds the tensor
+    from tests.test_oracle_pins import special_tensors
+
+    rng = np.random.default_rng(n)
+    msg_x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+    mc, ml, _ = abi.uniform(abi.to_dev(msg_x))
+    c_in, l_in = mc.cpu().numpy(), ml.cpu().numpy()
+    for label, x in special_tensors(n, rng).items():
+        check_special(abi, oracle, x, label)
+        # the ring step on it: acc += lut[codes], then the same quantization of the result
+        announce(f"ring step on {label} n={n}")
+        acc = abi.to_dev(x)
+        codes, lut, qp = abi.ring_step(acc, mc, ml)
+        torch.cuda.synchronize()
+        want = x.copy()
+        oracle.index_add(want, l_in, c_in)
+        assert np.array_equal(acc.cpu().numpy().view(np.uint32), want.view(np.uint32)), label
+        q = abi.qparams(qp)
+        assert np.array_equal(np.array([q["scale"]]), np.array([oracle.scale_exact(want)]), equal_nan=True), label
+        oc, _, _ = oracle.uniform_8bit_quantize(want, "given", scale=float(q["scale"]))
+        assert np.array_equal(codes.cpu().numpy(), oc), label
+        mean, cnt = oracle.average_buckets_f64(want, oc)
+        floor = float(q["scale"]) if np.isfinite(q["scale"]) and q["scale"] > 0 else 1e-3
+        assert lut_rel_err(lut.cpu().numpy(), mean, floor) <= LUT_TOL, label
+    # the same tensors through one segmented call: equal to the one-tensor results where the header promises it
+    xs = [abi.to_dev(v) for v in special_tensors(n, np.random.default_rng(n + 1)).values()]
+    sc, sl, sq = segmented_uniform(abi, xs)
+    for i, xt in enumerate(xs):
+        c1, l1, q1 = abi.uniform(xt)
+        assert torch.equal(sc[i], c1) and torch.equal(sq[i].view(torch.int64), q1.view(torch.int64))
+        assert tables_agree(sl[i].cpu().numpy(), l1.cpu().numpy(), 1e-3, LUT_TOL)
+
+
 def _small_inputs(n, rng):
     """What the kernel has a branch for: ordinary data, a tensor crowded into a few codes, all zeros
     (every code 0), products beyond the fixed-point range, a not-a-number, a huge scale."""

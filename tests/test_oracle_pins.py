@@ -321,6 +321,52 @@ def test_oracle_against_compiled_reference(oracle):
         assert np.array_equal(q, oracle.quantize_per_tensor_uint8(x, 3e-5, 100))
 
 
+def special_tensors(n, rng):
+    """Tensors that leave the ordinary branch of compression.cpp:113-122: a not-a-number (the norm, the
+    scale and every product are NaN: all codes 0), an infinity (infinite scale, 1 / scale = 0: every
+    finite element gets code 128, the infinity NaN -> code 0), values whose squares overflow fp32 but
+    not fp64 (an ordinary tensor for an fp64 sum of squares), and values whose norm overflows fp32
+    (infinite scale again)."""
+    base = (rng.standard_normal(n) * 1e-3 + 5e-3).astype(np.float32)
+    nan = base.copy()
+    nan[n // 3] = np.nan
+    inf = base.copy()
+    inf[2 * n // 3] = np.inf
+    big = (rng.standard_normal(n) * 1e25).astype(np.float32)
+    huge = np.full(n, 3e38, np.float32)
+    huge[::2] = np.float32(-2.5e38)
+    return {"one NaN": nan, "one +inf": inf, "squares overflow fp32": big, "norm overflows fp32": huge}
+
+
+def test_oracle_against_compiled_reference_on_special_values(oracle):
+    # the branches a NaN, an infinity and an overflowing norm take: codes and scale of the restatement against
+    # the reference's own compression.cpp, the table where the reference's fp32 sums are exact or infinite
+    if not oracle.ref_available():
+        pytest.skip("oracle/_ref not built (the reference checkout is not present)")
+    import torch
+
+    R = oracle.ref()
+    rng = np.random.default_rng(22)
+    for n in (1000, 65543):
+        for label, x in special_tensors(n, rng).items():
+            rc, rl = R.uniform_8bit_quantize(torch.from_numpy(x.copy()), True)
+            if label == "squares overflow fp32":
+                # libtorch's fp32 norm overflows where the formula's value is finite: the reference's scale is
+                # infinite, the exact one is not (a reference artefact, like its drift at large n)
+                oc, ol, sc = oracle.uniform_8bit_quantize(x, "literal")
+                assert np.isinf(sc) and np.isfinite(oracle.scale_exact(x))
+            else:
+                oc, ol, sc = oracle.uniform_8bit_quantize(x, "exact")
+                assert np.array_equal(np.array([sc]), np.array([oracle.scale_literal(x)]), equal_nan=True), label
+            assert np.array_equal(rc.numpy(), oc), label
+            assert np.array_equal(np.isnan(rl.numpy()), np.isnan(ol)), label
+            assert np.array_equal(np.isinf(rl.numpy()), np.isinf(ol)), label
+            if label == "one NaN":
+                assert not oc.any() and np.isnan(ol[0]) and not ol[1:].any()
+            if label == "one +inf":
+                assert (oc == 128).sum() == n - 1 and oc[2 * n // 3] == 0 and np.isposinf(ol[0])
+
+
 # ---------------------------------------------------------------- callers of the path (src/zeroband/diloco.py)
 
 def test_pseudo_gradient_is_torch_sub_then_div(oracle):
