@@ -3,36 +3,38 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--legs a,b,...]
 
-One "step" is one pass of the hot path over the workload of benchmark configuration 2: the 22
-per-layer pseudo-gradient buckets of a 1B Llama-style model (51,380,224 fp32 elements each,
-Student-t(3) * 1e-4), each run through uniform_8bit_quantize (statistics pass, then the
-fused quantize + 256-bin lookup build).  Inputs are generated on the GPU with a seeded torch
-generator (seed = layer index) and are resident in HBM before the timed region.
+One "step" is one pass of the hot path, uniform_8bit_quantize (statistics pass, then the fused
+quantize + 256-bin lookup build), over one 2^28-element fp32 tensor N(0, 1e-3): the size the
+target is quoted on, 1 GiB, four times the last-level cache, so every pass reads from HBM.  Three
+such tensors (torch generator on the GPU, seeds 0..2) and three code buffers are resident before
+the timed region and visited in rotation.
 
 The single JSON line printed at the end carries
-  value          algorithmic GB/s of quantize+lookup (9 bytes per element: x read twice, codes
-                 written once) over the whole step, wall clock between two synchronisations, with
-                 the buckets dealt over two HIP streams (--streams); one_stream is the same work
-                 strictly bucket after bucket
-  roofline       the dominant kernel (quantize + histogram, 5 bytes per element) on a 2^28-element
-                 tensor (1 GiB, four times the last-level cache, so what it reads comes from HBM),
-                 priced against the 8 TB/s HBM peak from per-launch HIP-event times inside
-                 uniform_8bit_quantize calls that rotate over three such tensors; the same kernel on
-                 the 205 MB buckets of the step (partly served by the last-level cache) is listed
-                 beside it, as run and with its input cold
+  value          algorithmic GB/s of uniform_8bit_quantize (9 bytes per element: x read twice, codes
+                 written once): K calls back to back between two synchronisations
+  ring_step_2p28 the ring reduce step (dequantize-add + requantize, 14 bytes per element) at the same size
+  roofline       the dominant kernel (quantize + histogram, 5 bytes per element) inside those calls,
+                 priced against the 8 TB/s HBM peak from per-launch HIP-event times; the same kernel on
+                 the 205 MB buckets of configuration 2 is listed beside it, as run and with its input cold
   tensor_2p28    every operation of the path on 2^28-element tensors, one row each: statistics,
                  quantize (a2), average_buckets (a3), dequantize add / set (a4 / a5), the fused
                  quantize + lookup, uniform_8bit_quantize and the ring reduce step
+  config_2_buckets  benchmark configuration 2: the 22 per-layer buckets of a 1B model (51,380,224 elements each,
+                 Student-t(3) * 1e-4), quantized bucket by bucket on one stream and dealt over two; a
+                 205 MB bucket stays in the 256 MB last-level cache between its two passes: cache-assisted
   ring_step      benchmark configuration 3: W = 8 chunks of 2^26 elements; quantize chunk 0, then 7 hops of
                  dequantize-add + requantize (14 bytes per element per hop)
+  ring_chunks    the sizes the ring really runs at: a layer bucket cut into 2 W = 16 chunks (3,211,264
+                 elements for configuration 2, 1,860,119 for configuration 4) and 64 tensors of 2^20 elements;
+                 one chunk at a time against all W = 8 ranks' chunks of a step in one segmented call
   other_configs  benchmark configurations 1, 4 and 5 (round trip on 2^24 elements; 42 buckets of a 10B model's
                  shard with outliers, quantize + dequantize; 2,000 small tensors in one launch and the
                  edge tensors), each as algorithmic GB/s
   cpu_baseline   the reference's own compression.cpp (compiled into oracle/_ref) on this box's
-                 host cores, on a bounded sample (one bucket, a few repetitions), with the same
-                 operations one by one
+                 host cores, on the same tensor the GPU leg starts with (copied to the host), a few
+                 repetitions, with the same operations one by one
 
---legs runs a subset (buckets, t28, ring, outer, diloco, configs, staging): what a profiler run
+--legs runs a subset (t28, buckets, ring, chunks, outer, diloco, configs, staging): what a profiler run
 of one workload uses, so that every kernel name in its trace belongs to one element count.
 """
 from __future__ import annotations
@@ -54,13 +56,28 @@ N_LAYERS = 22
 RING_W = 8
 RING_CHUNK = 1 << 26
 N28 = 1 << 28
-# HBM bytes one launch of the dominant kernel moves on a 2^28-element tensor, from rocprofv3
-# FETCH_SIZE / WRITE_SIZE scaled by the same counters' readings for the 1 GiB copy that this
-# program runs first: 1074.0 MB read + 269.3 MB written (codes + 0.9 MB of per-workgroup histogram partials)
-# against 1342.2 MB algorithmic (profiles/uniform_2p28_hbm_traffic.txt), and 205.8 + 52.4 MB against 256.9 MB
-# on a 51,380,224-element bucket (profiles/cfg2_buckets_hbm_traffic.txt).
-TRAFFIC_BYTES_PER_LAUNCH_2P28 = 1343.36e6
-TRAFFIC_BYTES_PER_LAUNCH_BUCKET = 258.27e6
+RING_CHUNK_CFG2 = BUCKET_ELEMS // 16     # a layer bucket cut into 2 * W chunks for W = 8 (collectives.cpp:89-90)
+RING_CHUNK_CFG4 = 29_761_904 // 16       # 1,860,119: the same for a 10B model's shard bucket
+
+
+def measured_traffic(profile: str, kernel_prefix: str, min_total_mb: float = 0.0):
+    """HBM bytes one launch of a kernel moves, from the committed summary of the two rocprofv3 --pmc
+    runs (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB copy
+    this program runs first): the total_MB column of the kernel's row in profiles/<profile>.  None
+    when the file or the row is missing."""
+    path = ROOT / "profiles" / profile
+    if not path.exists():
+        return None
+    best = None
+    for line in path.read_text().splitlines():
+        if line.startswith(kernel_prefix):
+            try:
+                total = float(line.split()[-1])
+            except ValueError:
+                continue
+            if total >= min_total_mb and (best is None or total > best):
+                best = total
+    return None if best is None else best * 1e6
 
 
 def student_t3(n, device, seed, scale):
@@ -99,17 +116,17 @@ def _median_time(fn, reps: int) -> float:
     return statistics.median(times)
 
 
-def cpu_baseline(sample_elems: int, ring_elems: int, reps: int) -> dict:
-    """The reference's CPU ops on this host, on a bounded sample: one config-2 bucket for
-    quantize + lookup, one config-3 chunk for the ring hop.  kind "reference" when oracle/_ref
-    is present (the reference's compression.cpp compiled unchanged), else the restatement
-    ("port").  The ring's dequantize loops exist only as a restatement (collectives.cpp does
-    not build without the gloo headers); as shipped they run on one thread."""
-    import numpy as np
+def cpu_baseline(x, acc, ring_codes, ring_lut, what: str, reps: int) -> dict:
+    """The reference's CPU ops on this host on the tensors the GPU leg works on (numpy arrays copied
+    from the device): ``x`` for uniform_8bit_quantize and its parts, ``acc`` with the message
+    (``ring_codes``, ``ring_lut``) for the ring hop.  kind "reference" when oracle/_ref is present
+    (the reference's compression.cpp compiled unchanged), else the restatement ("port").  The ring's
+    dequantize loops exist only as a restatement (collectives.cpp does not build without the gloo
+    headers); as shipped they run on one thread."""
     import torch
     from oracle import oracle as O
 
-    x = (np.random.default_rng(0).standard_t(3, sample_elems) * 1e-4).astype(np.float32)
+    sample_elems, ring_elems = x.size, acc.size
     threads = O.hardware_threads()
     if O.ref_available():
         R = O.ref()
@@ -137,9 +154,7 @@ def cpu_baseline(sample_elems: int, ring_elems: int, reps: int) -> dict:
     t = _median_time(fn, reps)
 
     # ring hop: chunk += lut[codes] on one thread as shipped, then uniform_8bit_quantize(chunk)
-    rng = np.random.default_rng(1)
-    acc = (rng.standard_normal(ring_elems) * 1e-3).astype(np.float32)
-    rc, rl, _ = O.uniform_8bit_quantize((rng.standard_normal(ring_elems) * 1e-3).astype(np.float32), "literal")
+    rc, rl = ring_codes, ring_lut
     t_add = _median_time(lambda: O.index_add(acc, rl, rc, 1), 3)
     t_add_threads = _median_time(lambda: O.index_add(acc, rl, rc, threads), 3)
     t_set = _median_time(lambda: O.index_set(acc, rl, rc, 1), 3)
@@ -154,11 +169,11 @@ def cpu_baseline(sample_elems: int, ring_elems: int, reps: int) -> dict:
         "unit": "GB/s",
         "cores": threads,
         "kind": kind,
-        "sample": f"uniform_8bit_quantize on one {sample_elems}-element Student-t(3)*1e-4 bucket, median of {reps} runs "
+        "sample": f"uniform_8bit_quantize on {what} ({sample_elems} elements, copied from the GPU), median of {reps} runs "
                   f"after one warm-up, {threads} threads (hardware_concurrency, as compression.cpp:7), "
                   f"{os.cpu_count()} logical CPUs visible",
         "elements_per_s": round(sample_elems / t, 1),
-        "ms_per_bucket": round(t * 1e3, 3),
+        "ms_per_call": round(t * 1e3, 3),
         "breakdown_ms": {k: round(v, 3) for k, v in parts.items()},
         # the same operations one by one, as GB/s of their algorithmic bytes (beside tensor_2p28.operations)
         "operations": {
@@ -177,7 +192,7 @@ def cpu_baseline(sample_elems: int, ring_elems: int, reps: int) -> dict:
             "value": round(14.0 * ring_elems / hop / 1e9, 3),
             "unit": "GB/s",
             "kind": kind + " quantize + port index_add (1 thread, as shipped)",
-            "sample": f"one hop on a {ring_elems}-element chunk, median of 3",
+            "sample": f"one hop on a {ring_elems}-element chunk (the first quarter of the GPU leg's accumulator and message), median of 3",
             "ms_per_hop": round(hop * 1e3, 3),
             "index_add_1_thread_ms": round(t_add * 1e3, 3),
             "index_add_unused_thread_variant_ms": round(t_add_threads * 1e3, 3),
@@ -200,9 +215,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--streams", type=int, default=2,
                     help="HIP streams the buckets are spread over in the timed region (1 = strictly one after another)")
-    ap.add_argument("--legs", default="buckets,t28,ring,outer,diloco,configs,staging",
-                    help="comma list of buckets (carries value), t28 (carries roofline and the per-operation rows), ring, "
-                         "outer, diloco, configs, staging")
+    ap.add_argument("--legs", default="buckets,t28,ring,chunks,outer,diloco,configs,staging",
+                    help="comma list of t28 (carries value, roofline and the per-operation rows), buckets (configuration 2), ring, "
+                         "chunks (ring chunks at their real sizes, one by one and segmented), outer, diloco, configs, staging")
     ap.add_argument("--t28-ops", default="",
                     help="comma list of substrings: the t28 leg runs only the operations whose name contains one of them "
                          "(uniform_8bit_quantize always runs: it carries the roofline)")
@@ -287,15 +302,16 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "benchmark configuration 2: 22 per-layer pseudo-gradient buckets x 51,380,224 fp32 elements, "
-                        "Student-t(3)*1e-4 (torch cuda generator, seed = layer), uniform_8bit_quantize bucket by bucket",
-            "elements_per_step": BUCKET_ELEMS * N_LAYERS,
-            "streams": args.streams,
+            "workload": "uniform_8bit_quantize (statistics pass, then fused quantize + 256-bin lookup build) on one 2^28-element fp32 "
+                        "tensor N(0, 1e-3) per step, three tensors and three code buffers (torch cuda generator, seeds 0..2) resident "
+                        "in HBM and visited in rotation: 3 GiB pass through the 256 MB last-level cache between two visits of one tensor",
+            "elements_per_step": N28,
             "algorithmic_bytes_per_element": 9,
             "n_bins": 256,
         },
     }
     bucket_kernel = None
+    cpu_inputs = None
 
     if "buckets" in legs:
         # ---- config 2: 22 layer buckets, quantize + lookup per bucket ---------------------------
@@ -352,18 +368,24 @@ def main() -> int:
             "input_cold": {"what": "quantize + lookup with the scale given, over the 22 buckets in turn: every bucket comes from HBM",
                            "avg_launch_us": round(cold, 2), "achieved": round(dom_bytes / cold / 1e3, 1),
                            "frac": round(dom_bytes / cold / 1e3 / HBM_PEAK_GBS, 4)},
-            "traffic": TRAFFIC_BYTES_PER_LAUNCH_BUCKET,
+            "traffic": measured_traffic("cfg2_buckets_hbm_traffic.txt", "quantize_kernel<true, true, true, true"),
             "kernels": {k: {"avg_us": round(us, 2), "algo_GBps": round(b / us / 1e3, 1), "launches": prof[k]["launches"]}
                         for k, (us, b) in per.items()},
         }
-        out.update({
-            "value": round(value, 1),
-            "ms_per_step": round(sec_pipelined * 1e3, 4),
-            "elements_per_s": round(elems / sec_pipelined, 1),
-            "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-            "one_stream": {"value": round(value_one_stream, 1), "unit": "GB/s", "ms_per_step": round(sec * 1e3, 4),
+        out["config_2_buckets"] = {
+            "workload": "benchmark configuration 2: 22 per-layer pseudo-gradient buckets x 51,380,224 fp32 elements, Student-t(3)*1e-4 "
+                        "(torch cuda generator, seed = layer), uniform_8bit_quantize bucket by bucket; cache-assisted: a 205 MB bucket "
+                        "stays in the 256 MB last-level cache between its statistics pass and its quantize pass",
+            "elements": elems, "algorithmic_bytes_per_element": 9,
+            "one_stream": {"value": round(value_one_stream, 1), "unit": "GB/s", "ms": round(sec * 1e3, 4),
                            "frac_of_hbm_peak": round(value_one_stream / HBM_PEAK_GBS, 4)},
-        })
+            "two_streams": {"value": round(value, 1), "unit": "GB/s", "ms": round(sec_pipelined * 1e3, 4), "streams": args.streams,
+                            "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                            "what": "the buckets dealt over HIP streams: one bucket's statistics pass overlaps its neighbours' quantize pass"},
+        }
+        if "t28" not in legs:            # a profiler run of this leg alone: its figure stands in for the headline
+            out.update({"value": round(value_one_stream, 1), "ms_per_step": round(sec * 1e3, 4)})
+            out["config"]["workload"] = out["config_2_buckets"]["workload"]
         del buckets, codes, plan
         torch.cuda.empty_cache()
 
@@ -450,6 +472,18 @@ def main() -> int:
                                                "frac_of_hbm_peak": round(4 * n28 / fill_us / 1e3 / HBM_PEAK_GBS, 4)}}
         dom_us, dom_bytes = uni_prof["quantize_kernel+hist"]
         uni, ring28 = rows["uniform_8bit_quantize (a1)"], rows.get("ring reduce step (a4 + a1)", {})
+        # the headline: K calls of uniform_8bit_quantize back to back between two synchronisations
+        step_s = uni["us_wall_back_to_back"] * 1e-6
+        out.update({"value": round(9.0 * n28 / step_s / 1e9, 1), "ms_per_step": round(step_s * 1e3, 4),
+                    "elements_per_s": round(n28 / step_s, 1), "frac_of_hbm_peak": round(9.0 * n28 / step_s / 1e9 / HBM_PEAK_GBS, 4)})
+        if ring28:
+            ring_s = ring28["us_wall_back_to_back"] * 1e-6
+            out["ring_step_2p28"] = {
+                "workload": "prime_ring_reduce_step on a 2^28-element accumulator (three in rotation) with a 2^28-code message: "
+                            "acc += lut[codes] with the statistics of the result, then quantize + lookup; 14 bytes per element",
+                "value": round(14.0 * n28 / ring_s / 1e9, 1), "unit": "GB/s", "ms_per_step": round(ring_s * 1e3, 4),
+                "elements_per_s": round(n28 / ring_s, 1), "frac_of_hbm_peak": round(14.0 * n28 / ring_s / 1e9 / HBM_PEAK_GBS, 4),
+                "sum_of_kernel_times": {"us": ring28["us"], "frac_of_hbm_peak": ring28["frac_of_hbm_peak"]}}
         out["tensor_2p28"] = {
             "workload": "2^28-element fp32 tensors N(0,1e-3), inputs and outputs three in rotation (3 GiB between two visits of the same "
                         "buffer); per operation: sum of its kernels' launch times (HIP events per launch), and wall time of "
@@ -463,25 +497,33 @@ def main() -> int:
         }
         out["roofline"] = {
             "bound": "hbm",
-            "kernel": "quantize_kernel<aligned, nt loads, hist, write-through stores> (quantize + 256-bin sum/count histogram)",
+            "kernel": "quantize_kernel<aligned, nt loads, hist, walked from the end, non-temporal code stores, four-row tiles> "
+                      "(quantize + 256-bin count / fixed-point sum histogram, the last 5 % of the tiles dealt on demand)",
             "workload": "inside uniform_8bit_quantize on 2^28-element tensors (1 GiB each; inputs and code buffers three in rotation: "
                         "nothing of either is left in the 256 MB last-level cache when the call starts)",
             "achieved": round(dom_bytes / dom_us / 1e3, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBS, 4),
-            "traffic": TRAFFIC_BYTES_PER_LAUNCH_2P28,
+            "traffic": measured_traffic("uniform_2p28_hbm_traffic.txt", "quantize_kernel<true, true, true, true"),
             "algo_bytes_per_launch": 5 * n28,
             "avg_launch_us": round(dom_us, 2),
             **overhead_note,
             "on_the_buckets_of_the_step": bucket_kernel,
         }
+        if not args.no_cpu_baseline:
+            # what the CPU leg works on: the first tensor of the rotation, and for the ring hop the first quarter
+            # (2^26 elements, configuration 3's chunk) of an accumulator with the message it received
+            uniform(xs28[0], cin28, lin28, qp28)
+            torch.cuda.synchronize()
+            cpu_inputs = (xs28[0].cpu().numpy(), xs28[1][:RING_CHUNK].cpu().numpy().copy(), cin28[:RING_CHUNK].cpu().numpy().copy(),
+                          lin28.cpu().numpy().copy())
         del xs28, c28s, cin28, o28s
         torch.cuda.empty_cache()
     elif bucket_kernel is not None:
         out["roofline"] = {"bound": "hbm", "kernel": "quantize_kernel+hist", "workload": bucket_kernel["workload"],
                            "achieved": bucket_kernel["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": bucket_kernel["frac"],
-                           "traffic": TRAFFIC_BYTES_PER_LAUNCH_BUCKET, "algo_bytes_per_launch": 5 * BUCKET_ELEMS,
+                           "traffic": measured_traffic("cfg2_buckets_hbm_traffic.txt", "quantize_kernel<true, true, true, true"), "algo_bytes_per_launch": 5 * BUCKET_ELEMS,
                            "avg_launch_us": bucket_kernel["avg_launch_us"], **overhead_note, "on_the_buckets_of_the_step": bucket_kernel}
 
     if "ring" in legs:
@@ -533,6 +575,72 @@ def main() -> int:
         }
         del chunks, pristine, cbuf
         torch.cuda.empty_cache()
+
+    if "chunks" in legs:
+        # ---- the sizes the ring really runs at: a layer bucket is cut into 2 W chunks (collectives.cpp:89-90) -----
+        # one ring hop / one uniform_8bit_quantize per chunk, chunk after chunk (three launches each), against all
+        # W = 8 ranks' chunks of one step of the lock-stepped ring in ONE segmented call (three launches in all).
+        # Three sets of tensors in rotation, so that a set is not simply served by the last-level cache.
+        def chunk_rows(label, sizes, rot):
+            res = {}
+            tot = sum(sizes)
+            g = torch.Generator(device=dev).manual_seed(len(sizes) * 1000 + sizes[0] % 997)
+            for kind, bpe in ((ops.SEG_UNIFORM, 9), (ops.SEG_REDUCE, 14)):
+                plans, singles = [], []
+                for _ in range(rot):
+                    xs = [torch.randn(n, device=dev, generator=g) * 1e-3 for n in sizes]
+                    cs = [torch.empty(n, dtype=torch.uint8, device=dev) for n in sizes]
+                    ls = torch.empty((len(sizes), 256), device=dev)
+                    if kind == ops.SEG_UNIFORM:
+                        plans.append(ops.SegmentPlan(kind, xs, codes=cs, luts=ls))
+
+                        def one(xs=xs, cs=cs, ls=ls):
+                            for x, c, l in zip(xs, cs, ls):
+                                _lib.check(lib.prime_uniform_8bit_quantize(x.data_ptr(), x.numel(), c.data_ptr(), l.data_ptr(), None,
+                                                                           ws.data_ptr(), st), "uniform")
+                    else:
+                        cin, lin = ops.uniform_8bit_quantize_segmented([torch.randn(n, device=dev, generator=g) * 1e-3 for n in sizes])
+                        plans.append(ops.SegmentPlan(kind, xs, cin, list(lin), codes=cs, luts=ls))
+
+                        def one(xs=xs, cin=cin, lin=lin, cs=cs, ls=ls):
+                            for a, ci, li, c, l in zip(xs, cin, lin, cs, ls):
+                                ring_step(a, ci, li, c, l)
+                    singles.append(one)
+                k = [0]
+
+                def run_seg():
+                    plans[k[0] % rot].run()
+                    k[0] += 1
+
+                def run_one():
+                    singles[k[0] % rot]()
+                    k[0] += 1
+
+                t_seg = timed(run_seg, args.steps * 2, args.warmup)
+                t_one = timed(run_one, args.steps * 2, args.warmup)
+                _lib.profile_begin()
+                for _ in range(max(3, args.steps // 2)):
+                    run_seg()
+                kern = kernel_table(_lib.profile_end(), event_overhead_us)
+                res["uniform_8bit_quantize" if kind == ops.SEG_UNIFORM else "ring_reduce_step"] = {
+                    "bytes_per_element": bpe,
+                    "segmented": {"us": round(t_seg * 1e6, 2), "GBps": round(bpe * tot / t_seg / 1e9, 1),
+                                  "frac_of_hbm_peak": round(bpe * tot / t_seg / 1e9 / HBM_PEAK_GBS, 4), "kernels": kern},
+                    "one_by_one": {"us": round(t_one * 1e6, 2), "GBps": round(bpe * tot / t_one / 1e9, 1),
+                                   "frac_of_hbm_peak": round(bpe * tot / t_one / 1e9 / HBM_PEAK_GBS, 4),
+                                   "us_per_tensor": round(t_one * 1e6 / len(sizes), 2)},
+                    "speedup": round(t_one / t_seg, 2)}
+                del plans, singles
+                torch.cuda.empty_cache()
+            return {"tensors": len(sizes), "elements_each": sizes[0], "elements": tot, **res}
+
+        out["ring_chunks"] = {
+            "workload": "N(0, 1e-3) chunks, three sets in rotation; one_by_one: the one-tensor entry point per chunk (three launches each); "
+                        "segmented: all chunks in one call (three launches in all), results bit-identical",
+            "config_2_bucket_over_16 x W=8": chunk_rows("cfg2", [RING_CHUNK_CFG2] * RING_W, 3),
+            "config_4_bucket_over_16 x W=8": chunk_rows("cfg4", [RING_CHUNK_CFG4] * RING_W, 3),
+            "64 x 2^20": chunk_rows("2p20", [1 << 20] * 64, 2),
+        }
 
     if "outer" in legs:
         # ---- the callers either side of the path: pseudo-gradient and outer optimizer step -----------
@@ -819,7 +927,15 @@ def main() -> int:
         del accs, stage
 
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(BUCKET_ELEMS, RING_CHUNK, reps=5)
+        if cpu_inputs is None:           # the t28 leg did not run: one configuration-2 bucket, drawn as the GPU leg draws it
+            b0 = student_t3(BUCKET_ELEMS, dev, 0, 1e-4)
+            c0, l0 = ops.uniform_8bit_quantize(b0[:RING_CHUNK // 4])
+            cpu_inputs = (b0.cpu().numpy(), b0[RING_CHUNK // 4: RING_CHUNK // 2].cpu().numpy().copy(), c0.cpu().numpy(), l0.cpu().numpy())
+            what = "one 51,380,224-element Student-t(3)*1e-4 bucket of configuration 2"
+            del b0
+        else:
+            what = "the first 2^28-element N(0, 1e-3) tensor of the GPU leg's rotation"
+        out["cpu_baseline"] = cpu_baseline(*cpu_inputs, what=what, reps=3)
         out["gpu_over_cpu"] = round(out["value"] / out["cpu_baseline"]["value"], 1) if out["value"] and out["cpu_baseline"]["value"] else None
 
     print(json.dumps(out))

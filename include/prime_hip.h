@@ -235,8 +235,10 @@ int prime_ring_gather_step(float* chunk, const uint8_t* codes_in, const float* l
  * qparams_out[i]) equal what the one-tensor entry point returns for it, bit for bit (the lookup
  * entries of a tensor whose 1 / scale is zero or not finite, and bins 0 / 255 of a tensor with
  * values beyond 628 bins in several workgroups, may differ in their last bit: they are sums of
- * fp64 values in an order that depends on the launch).  Tensors that are empty or not aligned for
- * vector access (tensor 16 bytes, codes 4) take the one-tensor path inside the call.  The pointer
+ * fp64 values in an order that depends on the launch).  Tensors that are empty, not aligned for
+ * vector access (tensor 16 bytes, codes 4), or large enough to fill the device on their own (more than
+ * 2^25 elements, 2^24 for the ring steps: options "segment_max_mi_elems", "segment_ring_max_mi_elems")
+ * take the one-tensor path inside the call.  The pointer
  * and size arrays are host memory and are read before the call returns; luts is count x 256 floats
  * and qparams_out (optional) count records on the device.  One workspace, as for the calls above. */
 int prime_uniform_8bit_quantize_segmented(const float* const* xs, const int64_t* ns, int64_t count,

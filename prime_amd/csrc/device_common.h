@@ -58,11 +58,13 @@ struct BinPart {
     long long units;
     unsigned long long cnt;
 };
-// The elements of a workgroup that lie beyond the range of the fixed-point residual (they all have
-// code 0 or 255): their number and the fp64 sum of their values, per side.
-struct FarPart {
-    double sum[2];
-    unsigned long long cnt[2];
+// Where a workgroup leaves its elements beyond the range of the fixed-point residual (they all have
+// code 0 or 255): their number and the fp64 sum of their values, per side (0: code 0, 1: code 255).
+// The workspace keeps them as one array per side and quantity, indexed by workgroup, so that the
+// second stage reads them with coalesced loads; side 1 lies kMaxGrid entries after side 0.
+struct FarSlot {
+    double* sum;
+    unsigned long long* cnt;
 };
 // Which of the two forms the partials of the launch before have, and the 1 / scale their residuals refer to.
 enum { kHistFp = 0, kHistFixed = 1 };
@@ -89,7 +91,8 @@ struct Workspace {
     unsigned pad;
     double part_sum[kMaxGrid];
     double part_sq[kMaxGrid];
-    FarPart far[kMaxGrid];
+    double far_sum[2][kMaxGrid];
+    unsigned long long far_cnt[2][kMaxGrid];
     union alignas(16) {
         BinAcc hist[kMaxGrid][kBins];    // 4 KiB per workgroup
         BinPart hist_fixed[kMaxGrid][kBins];
@@ -638,10 +641,35 @@ __device__ __forceinline__ void rhist_far_side(const H& h, int side, unsigned lo
 
 // The workgroup's partial: 4 KiB of integer bin totals to `row`, the far elements to `far`.
 template <int T = kThreads>
-__device__ __forceinline__ void rhist_store(ResidualHist& h, int shift, BinPart* __restrict__ row, FarPart* __restrict__ far) {
+__device__ __forceinline__ void rhist_store(ResidualHist& h, int shift, BinPart* __restrict__ row, const FarSlot far) {
     rhist_flush<T>(h, shift);
     for (int b = threadIdx.x; b < kBins; b += T) row[b] = BinPart{h.wide_sum[b], h.wide_cnt[b]};
-    if (threadIdx.x < 2) rhist_far_side(h, threadIdx.x, far->cnt[threadIdx.x], far->sum[threadIdx.x]);
+    if (threadIdx.x < 2) rhist_far_side(h, threadIdx.x, far.cnt[threadIdx.x * kMaxGrid], far.sum[threadIdx.x * kMaxGrid]);
+}
+
+// The far elements of side `side` over the partials [p0, p1), by the calling wavefront (all 64 lanes call;
+// the totals are valid in lane 0): lane l adds partials p0 + l, p0 + l + 64, ... (four loads in flight), the
+// lanes are then added by the fixed tree of wave_sum.
+__device__ __forceinline__ void far_totals(const Workspace* __restrict__ ws, int p0, int p1, int side, double& far_s, unsigned long long& far_n) {
+    const int lane = threadIdx.x & 63;
+    double fs = 0.0;
+    unsigned long long fn = 0;
+    for (int q = p0 + lane; q < p1; q += 4 * 64) {
+        double s[4];
+        unsigned long long c[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int p = q + 64 * k;
+            s[k] = p < p1 ? ws->far_sum[side][p] : 0.0;
+            c[k] = p < p1 ? ws->far_cnt[side][p] : 0ull;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { fs += s[k]; fn += c[k]; }
+    }
+    far_s = wave_sum(fs);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) fn += __shfl_down(fn, off, 64);
+    far_n = fn;
 }
 
 // Register-side accumulators for a tensor whose values crowd into a few codes (a constant, or

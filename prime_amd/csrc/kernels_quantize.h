@@ -34,14 +34,14 @@ __device__ __forceinline__ void hist_store_bin0(double s, unsigned long long c, 
 // with `first` set - the form of the partials for the kernel that reads them.
 struct HistOut {
     BinAcc* row;
-    FarPart* far;
+    FarSlot far;
     HistInfo* info;
     bool first;
     unsigned* tile_counter;     // deals the last part of the tiles on demand (sweep_tiles_dynamic); null: all round-robin
     int dyn_percent;
 };
 __device__ __forceinline__ HistOut hist_out_of(Workspace* ws, int slot, int dyn_percent) {
-    return HistOut{ws ? ws->hist[slot] : nullptr, ws ? &ws->far[slot] : nullptr, ws ? &ws->hist_info : nullptr, slot == 0,
+    return HistOut{ws ? ws->hist[slot] : nullptr, FarSlot{ws ? &ws->far_sum[0][slot] : nullptr, ws ? &ws->far_cnt[0][slot] : nullptr}, ws ? &ws->hist_info : nullptr, slot == 0,
                    ws && dyn_percent > 0 ? &ws->tile_counter : nullptr, dyn_percent};
 }
 
@@ -273,26 +273,29 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
     __shared__ double sh_sum[kFinalThreads];                 // fixed-point partials: the upper halves' total, as an integer
     __shared__ unsigned long long sh_lo[kFinalThreads];
     __shared__ unsigned long long sh_cnt[kFinalThreads];
-    __shared__ double sh_far_s[kRows];
-    __shared__ unsigned long long sh_far_n[kRows];
+    __shared__ double sh_far_s;
+    __shared__ unsigned long long sh_far_n;
     const int bl = threadIdx.x % kLutBinsPerBlock;
     const int row = threadIdx.x / kLutBinsPerBlock;
     const int bin = blockIdx.x * kLutBinsPerBlock + bl;
-    const HistInfo info = ws->hist_info;
-    const bool fixed = info.mode == kHistFixed;
-    const bool far_bin = fixed && (bin == 0 || bin == kBins - 1);
     constexpr int kIters = kMaxGrid / kRows;
-    const int side = bin != 0;
+    const HistInfo info = ws->hist_info;        // first of the loads: it is back when the partials are
     BinAcc part[kIters];
-    double far_s[kIters];
-    unsigned long long far_n[kIters];
 #pragma unroll
     for (int k = 0; k < kIters; ++k) {          // all loads in flight at once
         const int p = row + k * kRows;
         part[k] = p < nparts ? ws->hist[p][bin] : BinAcc{0.0, 0ull};
-        far_s[k] = far_bin && p < nparts ? ws->far[p].sum[side] : 0.0;
-        far_n[k] = far_bin && p < nparts ? ws->far[p].cnt[side] : 0ull;
     }
+    // the far elements of bin 0 / 255 (fixed-point partials only; harmless to read otherwise): the last wavefront
+    // of the workgroup that owns the bin adds them up, its loads in flight with everybody's
+    const bool clip_block = blockIdx.x == 0 || blockIdx.x == kBins / kLutBinsPerBlock - 1;
+    if (clip_block && threadIdx.x >= kFinalThreads - 64) {
+        double fs;
+        unsigned long long fn;
+        far_totals(ws, 0, nparts, blockIdx.x != 0, fs, fn);
+        if (threadIdx.x == kFinalThreads - 64) { sh_far_s = fs; sh_far_n = fn; }
+    }
+    const bool fixed = info.mode == kHistFixed;
     unsigned long long c = 0;
 #pragma unroll
     for (int k = 0; k < kIters; ++k) c += part[k].cnt;
@@ -308,14 +311,6 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
         }
         sh_sum[threadIdx.x] = __longlong_as_double(hi);
         sh_lo[threadIdx.x] = lo;
-        if (far_bin) {
-            double fs = 0.0;
-            unsigned long long fn = 0;
-#pragma unroll
-            for (int k = 0; k < kIters; ++k) { fs += far_s[k]; fn += far_n[k]; }
-            sh_far_s[row] = fs;
-            sh_far_n[row] = fn;
-        }
     } else {
         double s = 0.0;
 #pragma unroll
@@ -330,10 +325,6 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
             if (fixed) {
                 sh_sum[threadIdx.x] = __longlong_as_double(__double_as_longlong(sh_sum[threadIdx.x]) + __double_as_longlong(sh_sum[other]));
                 sh_lo[threadIdx.x] += sh_lo[other];
-                if (far_bin) {
-                    sh_far_s[row] += sh_far_s[row + half];
-                    sh_far_n[row] += sh_far_n[row + half];
-                }
             } else {
                 sh_sum[threadIdx.x] += sh_sum[other];
             }
@@ -342,8 +333,9 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
     }
     if (row == 0 && bin < n_bins) {
         const unsigned long long cc = sh_cnt[threadIdx.x];
-        const double sum = fixed ? fixed_bin_sum(cc, __double_as_longlong(sh_sum[threadIdx.x]), sh_lo[threadIdx.x], far_bin ? sh_far_n[0] : 0ull,
-                                                 far_bin ? sh_far_s[0] : 0.0, info.inv, bin)
+        const bool far_bin = bin == 0 || bin == kBins - 1;
+        const double sum = fixed ? fixed_bin_sum(cc, __double_as_longlong(sh_sum[threadIdx.x]), sh_lo[threadIdx.x], far_bin ? sh_far_n : 0ull,
+                                                 far_bin ? sh_far_s : 0.0, info.inv, bin)
                                  : sh_sum[threadIdx.x];
         lut[bin] = mean_entry(sum, cc);
         if (counts) counts[bin] = cc;

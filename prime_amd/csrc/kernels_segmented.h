@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void seg_quantize_kernel(c
     int narrow = INT_MIN;
     const float inv = block_scale_from_partials<kThreads>(ws->seg_part_sum[t], ws->seg_part_sq[t], job.parts[t], n, p == 0, &ws->seg[t].qp,
                                                           qp_out ? qp_out + t : nullptr, &narrow);
-    const HistOut out{ws->hist[blockIdx.x], &ws->far[blockIdx.x], &ws->seg[t].info, p == 0, nullptr, 0};
+    const HistOut out{ws->hist[blockIdx.x], FarSlot{&ws->far_sum[0][blockIdx.x], &ws->far_cnt[0][blockIdx.x]}, &ws->seg[t].info, p == 0, nullptr, 0};
     if ((job.two_row >> t) & 1)
         quantize_block<true, true, true, true, POLICY, 2>(job.x[t], n, inv, narrow, kZeroPoint, job.codes[t], out, copies_shift, p, P, hist_mem);
     else
@@ -108,51 +108,46 @@ __global__ __launch_bounds__(kFinalThreads) void seg_lut_finalize_kernel(const S
     __shared__ double sh_sum[kSegFinalGroups][kBins];            // fixed-point partials: the upper halves' total, as an integer
     __shared__ unsigned long long sh_lo[kSegFinalGroups][kBins];
     __shared__ unsigned long long sh_cnt[kSegFinalGroups][kBins];
-    __shared__ double sh_far_s[kSegFinalGroups][2];
-    __shared__ unsigned long long sh_far_n[kSegFinalGroups][2];
+    __shared__ double sh_far_s[2];
+    __shared__ unsigned long long sh_far_n[2];
     const int t = blockIdx.x;
     const int b = threadIdx.x & (kBins - 1), g = threadIdx.x / kBins;
     const int p0 = job.first[t], p1 = job.first[t + 1];
-    const HistInfo info = ws->seg[t].info;
-    const bool fixed = info.mode == kHistFixed;
-    const bool far_bin = fixed && (b == 0 || b == kBins - 1);
-    const int side = b != 0;
-    unsigned long long cnt = 0, lo = 0, far_n = 0;
+    unsigned long long cnt = 0, lo = 0;
     long long hi = 0;
-    double sum = 0.0, far_s = 0.0;
+    double sum = 0.0;
     constexpr int kInFlight = 8;
+    // both readings of a partial are added up (the integer one and the fp64 one); the record that says which
+    // one holds arrives with the first partials instead of ahead of them
     for (int q0 = p0 + g; q0 < p1; q0 += kSegFinalGroups * kInFlight) {
         BinAcc e[kInFlight];
-        double fs[kInFlight];
-        unsigned long long fn[kInFlight];
 #pragma unroll
         for (int k = 0; k < kInFlight; ++k) {
             const int p = q0 + k * kSegFinalGroups;
             e[k] = p < p1 ? ws->hist[p][b] : BinAcc{0.0, 0ull};
-            fs[k] = far_bin && p < p1 ? ws->far[p].sum[side] : 0.0;
-            fn[k] = far_bin && p < p1 ? ws->far[p].cnt[side] : 0ull;
         }
 #pragma unroll
         for (int k = 0; k < kInFlight; ++k) {
             cnt += e[k].cnt;
-            if (fixed) {
-                const long long u = __double_as_longlong(e[k].sum);      // BinPart::units
-                hi += units_hi(u);
-                lo += units_lo(u);
-                far_s += fs[k];
-                far_n += fn[k];
-            } else {
-                sum += e[k].sum;
-            }
+            const long long u = __double_as_longlong(e[k].sum);      // BinPart::units
+            hi += units_hi(u);
+            lo += units_lo(u);
+            sum += e[k].sum;
         }
     }
+    // the far elements of bins 0 and 255: the last two wavefronts, one side each
+    if (threadIdx.x >= kFinalThreads - 128) {
+        const int side = threadIdx.x >= kFinalThreads - 64;
+        double fs;
+        unsigned long long fn;
+        far_totals(ws, p0, p1, side, fs, fn);
+        if ((threadIdx.x & 63) == 0) { sh_far_s[side] = fs; sh_far_n[side] = fn; }
+    }
+    const HistInfo info = ws->seg[t].info;
+    const bool fixed = info.mode == kHistFixed;
     sh_cnt[g][b] = cnt;
     sh_lo[g][b] = lo;
     sh_sum[g][b] = fixed ? __longlong_as_double(hi) : sum;
-    if (far_bin) {
-        sh_far_s[g][side] = far_s;
-        sh_far_n[g][side] = far_n;
-    }
     __syncthreads();
     if (g == 0) {
 #pragma unroll
@@ -161,15 +156,12 @@ __global__ __launch_bounds__(kFinalThreads) void seg_lut_finalize_kernel(const S
             if (fixed) {
                 hi += __double_as_longlong(sh_sum[k][b]);
                 lo += sh_lo[k][b];
-                if (far_bin) {
-                    far_s += sh_far_s[k][side];
-                    far_n += sh_far_n[k][side];
-                }
             } else {
                 sum += sh_sum[k][b];
             }
         }
-        if (fixed) sum = fixed_bin_sum(cnt, hi, lo, far_n, far_s, info.inv, b);
+        const bool far_bin = b == 0 || b == kBins - 1;
+        if (fixed) sum = fixed_bin_sum(cnt, hi, lo, far_bin ? sh_far_n[b != 0] : 0ull, far_bin ? sh_far_s[b != 0] : 0.0, info.inv, b);
         luts[static_cast<int64_t>(t) * kBins + b] = mean_entry(sum, cnt);
     }
 }

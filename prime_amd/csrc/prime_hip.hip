@@ -80,7 +80,12 @@ struct Options {
     // 25 % to 224; on a 51 M-element bucket (two-row tiles, 1 us each) any share costs: 37.5 us against 39.8 at 5 %
     int dynamic_tail_percent = 5;
     int64_t dynamic_tail_min_elems = int64_t(1) << 27;
-    int segment_blocks_per_cu = 2;  // workgroups per compute unit the quantize pass of a segmented launch shares out among its tensors
+    int segment_blocks_per_cu = 2;
+    // a tensor of more elements than this fills the device on its own and takes the one-tensor path inside a segmented call:
+    // eight tensors of 2^24 elements 201 us segmented against 283 us one by one (ring step 333 against 385), of 2^25
+    // 396 against 453 (ring step 683 against 643), of 2^26 812 against 804 (ring step 1407 against 1207)
+    int64_t segment_max_elems = int64_t(1) << 25;
+    int64_t segment_ring_max_elems = int64_t(1) << 24;  // workgroups per compute unit the quantize pass of a segmented launch shares out among its tensors
     int64_t set_four_rows_max_elems = int64_t(1) << 25;  // the one-workgroup-per-tile dequantize set takes tiles of four rows up to this many elements (0: never)
 };
 Options g_opt;
@@ -454,6 +459,9 @@ int prime_hip_set_option(const char* name, int value) {
     } else if (!strcmp(name, "segment_blocks_per_cu")) {
         if (value < 1 || value > 8) return fail(PRIME_EINVAL, "segment_blocks_per_cu must be 1..8");
         g_opt.segment_blocks_per_cu = value;
+    } else if (!strcmp(name, "segment_max_mi_elems") || !strcmp(name, "segment_ring_max_mi_elems")) {
+        if (value < 0 || value > 8192) return fail(PRIME_EINVAL, "segment_max_mi_elems / segment_ring_max_mi_elems must be in [0, 8192]");
+        (name[8] == 'r' ? g_opt.segment_ring_max_elems : g_opt.segment_max_elems) = static_cast<int64_t>(value) << 20;
     } else if (!strcmp(name, "reverse_second_pass")) {
         g_opt.reverse_second_pass = value != 0;
     } else if (!strcmp(name, "nt_load_min_mib")) {
@@ -475,6 +483,8 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "code_store_policy")) *value = g_opt.code_store_policy;
     else if (!strcmp(name, "reverse_second_pass")) *value = g_opt.reverse_second_pass;
     else if (!strcmp(name, "segment_blocks_per_cu")) *value = g_opt.segment_blocks_per_cu;
+    else if (!strcmp(name, "segment_max_mi_elems")) *value = static_cast<int>(g_opt.segment_max_elems >> 20);
+    else if (!strcmp(name, "segment_ring_max_mi_elems")) *value = static_cast<int>(g_opt.segment_ring_max_elems >> 20);
     else if (!strcmp(name, "dynamic_tail_percent")) *value = g_opt.dynamic_tail_percent;
     else if (!strcmp(name, "dynamic_tail_min_mi_elems")) *value = static_cast<int>(g_opt.dynamic_tail_min_elems >> 20);
     else if (!strcmp(name, "large_read_grid_eighths")) *value = g_opt.large_read_grid_eighths;
@@ -891,7 +901,8 @@ int run_segmented(SegKind kind, const char* who, float* const* xs, const int64_t
         int g = 0;
         const int64_t start = i;
         while (i < count && g < kSegMax) {
-            const bool ok = ns[i] > 0 && aligned_to(xs[i], 16) && aligned_to(codes[i], 4) && (kind == kSegUniform || aligned_to(codes_in[i], 4));
+            const bool ok = ns[i] > 0 && ns[i] <= (kind == kSegUniform ? g_opt.segment_max_elems : g_opt.segment_ring_max_elems) &&
+                            aligned_to(xs[i], 16) && aligned_to(codes[i], 4) && (kind == kSegUniform || aligned_to(codes_in[i], 4));
             if (!ok) break;
             gx[g] = xs[i];
             gn[g] = ns[i];
