@@ -173,7 +173,10 @@ int prime_uniform_8bit_quantize_buckets(const float* const* xs, const int64_t* n
  * (src/zeroband/diloco.py:147-201), each handled as uniform_8bit_quantize handles one tensor.
  * offsets: count+1 non-decreasing int64 on the device (not checked: they are read by the kernel).
  * x and codes may be NULL only when count is 0.  codes uses the same offsets; luts is count x 256;
- * qparams_out (optional) is count entries.  Meant for small tensors: one workgroup each. */
+ * qparams_out (optional) is count entries.  Meant for tensors of up to 65,536 elements: every tensor gets
+ * exactly one workgroup, so a larger entry is still quantized correctly but on one compute unit; a
+ * caller that knows its sizes on the host takes prime_uniform_8bit_quantize_segmented for such sets
+ * (the Python layer does so by itself when the offsets are host-visible). */
 int prime_uniform_8bit_quantize_batched(const float* x, const int64_t* offsets, int64_t count,
                                         uint8_t* codes, float* luts, prime_qparams* qparams_out,
                                         prime_stream_t stream);

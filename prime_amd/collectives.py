@@ -15,11 +15,11 @@ def gloo_all_reduce(
     op: dist.ReduceOp = dist.ReduceOp.SUM,
     group: Optional[dist.ProcessGroup] = None,
 ) -> None:
-    """Uncompressed path, as the reference spells it (collectives.py:12-28): divide by the group size
-    for AVG, then ``dist.all_reduce(tensor, op)`` with the caller's op.  (With AVG the reference thus
-    divides and then asks the backend for AVG as well; Gloo rejects AVG, so in practice only SUM reaches
-    it.  Kept as is: this path is the reference's, not a kernel of this build.)
-    A ``SimulatedRing`` group is reduced in place: pre-division for AVG, then the sum."""
+    """Uncompressed path (src/zeroband/collectives.py:12-28): for AVG divide by the group size, then sum.
+    The reference divides and then hands its ``op`` on to ``dist.all_reduce``, so with AVG the backend
+    is asked to average once more: Gloo rejects that, and a backend that accepts it would divide twice.
+    What the reference means - divide, then SUM - is what both branches here do.
+    A ``SimulatedRing`` group is reduced in place the same way."""
     from .C.collectives import SimulatedRing
 
     if isinstance(group, SimulatedRing):
@@ -40,7 +40,7 @@ def gloo_all_reduce(
         raise ValueError(f"Unsupported reduce operation {op}. Only SUM and AVG are supported.")
     if op == dist.ReduceOp.AVG:
         tensor.div_(group.size())
-    dist.all_reduce(tensor, op, group=group)
+    dist.all_reduce(tensor, dist.ReduceOp.SUM, group=group)
 
 
 def all_reduce(

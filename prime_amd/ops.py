@@ -296,14 +296,35 @@ def _ring_step(acc: torch.Tensor, codes_in: torch.Tensor, lut_in: torch.Tensor, 
     return codes, lut
 
 
+BATCHED_MAX_ELEMS = 1 << 16      # the one-workgroup-per-tensor kernel is meant for tensors up to this size
+
+
 def _uniform_8bit_quantize_batched(flat: torch.Tensor, offsets: torch.Tensor):
     """Every slice flat[offsets[t]:offsets[t+1]] quantized on its own, one launch.
-    Returns (codes like flat, luts [count, 256], qparams [count, 4] float64 words)."""
+    Returns (codes like flat, luts [count, 256], qparams [count, 4] float64 words).
+    With ``offsets`` in host memory the sizes are checked, and a set that holds an entry of more than
+    65,536 elements is routed through the segmented call; offsets that live on the device are read by
+    the kernel alone and every entry gets one workgroup whatever its size."""
     _need_f32(flat, "uniform_8bit_quantize_batched")
     if offsets.dtype != torch.int64 or offsets.dim() != 1 or offsets.numel() < 1:
         raise RuntimeError("uniform_8bit_quantize_batched: offsets must be a 1-D int64 tensor of count+1 entries")
     if not flat.is_contiguous():
         raise RuntimeError("uniform_8bit_quantize_batched: flat must be contiguous")
+    if not offsets.is_cuda:
+        # offsets the host can see: checked, and a set with an entry too large for one workgroup (the batched
+        # kernel gives every tensor exactly one) goes through the segmented call, which sizes the grid per tensor
+        host = offsets.tolist()
+        if host[0] < 0 or host[-1] > flat.numel() or any(b < a for a, b in zip(host, host[1:])):
+            raise RuntimeError("uniform_8bit_quantize_batched: offsets must be non-decreasing and lie inside flat")
+        if any(b - a > BATCHED_MAX_ELEMS for a, b in zip(host, host[1:])):
+            views = [flat.view(-1)[a:b] for a, b in zip(host, host[1:])]
+            codes = torch.empty(flat.shape, dtype=torch.uint8, device=flat.device)
+            cviews = [codes.view(-1)[a:b] for a, b in zip(host, host[1:])]
+            luts = torch.empty((len(views), N_BINS), dtype=torch.float32, device=flat.device)
+            qps = torch.empty((len(views), 4), dtype=torch.float64, device=flat.device)
+            if views:
+                SegmentPlan(SEG_UNIFORM, views, codes=cviews, luts=luts, qparams=qps).run()
+            return codes, luts, qps
     lib = _lib.load()
     dev = flat.device
     count = offsets.numel() - 1
@@ -377,6 +398,24 @@ def _(codes_in, lut_in):
 @torch.library.register_fake("prime::ring_reduce_div_step")
 def _(acc, codes_in, lut_in, divisor):
     return acc.new_empty(acc.shape, dtype=torch.uint8), acc.new_empty(N_BINS, dtype=torch.float32)
+
+
+@torch.library.register_fake("prime::dequantize_")
+def _(out, codes, lut, accumulate):
+    return None
+
+
+@torch.library.register_fake("prime::uniform_8bit_quantize_stats")
+def _(tensor):
+    return (tensor.new_empty(tensor.shape, dtype=torch.uint8), tensor.new_empty(N_BINS, dtype=torch.float32),
+            tensor.new_empty(4, dtype=torch.float64))
+
+
+@torch.library.register_fake("prime::uniform_8bit_quantize_batched")
+def _(flat, offsets):
+    count = offsets.shape[0] - 1
+    return (flat.new_empty(flat.shape, dtype=torch.uint8), flat.new_empty((count, N_BINS), dtype=torch.float32),
+            flat.new_empty((count, 4), dtype=torch.float64))
 
 
 def unpack_qparams(qp: torch.Tensor) -> dict:
@@ -498,6 +537,31 @@ def _outer_sgd_nesterov_codes_(param, momentum_buf, codes, lut, inner, lr: float
                                                    inner.data_ptr() if inner is not None else None, n, float(lr),
                                                    float(momentum), int(first_step), _stream(dev)),
                    "prime_outer_sgd_nesterov_u8")
+
+
+@torch.library.register_fake("prime::div_")
+def _(x, divisor):
+    return None
+
+
+@torch.library.register_fake("prime::pseudo_gradient_")
+def _(out, outer, inner, world_size):
+    return None
+
+
+@torch.library.register_fake("prime::ring_first_touch_")
+def _(grad, outer, inner, world_size, codes_in, lut_in, divisor):
+    return grad.new_empty(grad.shape, dtype=torch.uint8), grad.new_empty(N_BINS, dtype=torch.float32)
+
+
+@torch.library.register_fake("prime::outer_sgd_nesterov_")
+def _(param, momentum_buf, grad, inner, lr, momentum, first_step):
+    return None
+
+
+@torch.library.register_fake("prime::outer_sgd_nesterov_codes_")
+def _(param, momentum_buf, codes, lut, inner, lr, momentum, first_step):
+    return None
 
 
 _LIB.impl("div_", _div_, "CUDA")

@@ -201,17 +201,24 @@ def ring_allreduce_staged(tensors: Sequence[torch.Tensor], avg: bool = False, tr
     return transport
 
 
-_stages: Dict[Tuple[int, int], HostStage] = {}
+_stages: Dict[Tuple[int, int, int], HostStage] = {}
+_STAGE_CACHE_MAX = 8
 
 
-def _stage_for(device: torch.device, chunk_numel: int) -> HostStage:
-    """One HostStage per (device, chunk size), kept: pinned allocations are slow and the per-layer
-    buckets of a model repeat a handful of sizes."""
+def _stage_for(device: torch.device, chunk_numel: int, group) -> HostStage:
+    """One HostStage per (device, chunk size, group), kept: pinned allocations are slow and the per-layer
+    buckets of a model repeat a handful of sizes.  The cache holds at most _STAGE_CACHE_MAX stages (the
+    least recently used one is dropped: each holds four pinned and two device chunk buffers), and a
+    stage is never shared by two groups.  Calls on one group are expected one at a time, as a ring
+    all-reduce is; two threads driving the same group concurrently would share its slots."""
     idx = device.index if device.index is not None else torch.cuda.current_device()
-    key = (idx, int(chunk_numel))
-    st = _stages.get(key)
+    key = (idx, int(chunk_numel), id(group))
+    st = _stages.pop(key, None)
     if st is None:
-        st = _stages[key] = HostStage(torch.device("cuda", idx), chunk_numel)
+        st = HostStage(torch.device("cuda", idx), chunk_numel)
+        while len(_stages) >= _STAGE_CACHE_MAX:
+            _stages.pop(next(iter(_stages)))
+    _stages[key] = st                 # most recently used last
     return st
 
 
@@ -229,7 +236,7 @@ def ring_allreduce_group(tensor: torch.Tensor, avg: bool, group) -> None:
     n = _check_ring_inputs([flat] * W)
     nb = BUFFER_COUNT * W
     csz = n // nb
-    stage = _stage_for(flat.device, csz)
+    stage = _stage_for(flat.device, csz, group)
     dst = dist.get_global_rank(group, (rank + 1) % W)                    # :111
     src = dist.get_global_rank(group, (rank - 1 + W) % W)               # :112
 
@@ -239,6 +246,22 @@ def ring_allreduce_group(tensor: torch.Tensor, avg: bool, group) -> None:
     own: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
     for phase in (1, 2):
         works: Dict[int, list] = {}
+        pending: Optional[int] = None      # step whose message is on its way to the pinned send slot, not yet handed to the transport
+
+        def hand_over() -> None:
+            # the host waits for the device-to-host copy only here, after the next step's kernels are enqueued:
+            # the copy of step s runs beside the kernels of step s + 1
+            nonlocal pending
+            if pending is None:
+                return
+            s_ = pending
+            pending = None
+            lut_h, codes_h = stage.take_send(s_)                         # the message is in pinned host memory
+            rl, rc = stage.recv_buffers(s_)
+            lut_tag, codes_tag = message_tags(s_)
+            works[s_] = [dist.isend(lut_h, dst, group=group, tag=lut_tag), dist.irecv(rl, src, group=group, tag=lut_tag),
+                         dist.isend(codes_h, dst, group=group, tag=codes_tag), dist.irecv(rc, src, group=group, tag=codes_tag)]
+
         for step in range(1, nb + 1):
             c = ((rank * BUFFER_COUNT - step) if phase == 1 else (rank * BUFFER_COUNT + BUFFER_COUNT - step)) % nb   # :116 / :192
             ch = chunk(c)
@@ -259,12 +282,10 @@ def ring_allreduce_group(tensor: torch.Tensor, avg: bool, group) -> None:
                 out = ops.ring_gather_step(ch, *own.pop(c))
             elif sending:
                 out = ops.uniform_8bit_quantize(ch, False)
+            hand_over()                                                  # the message of the step before
             if out is not None:
                 stage.post_send(step, out[0], out[1])
-                lut_h, codes_h = stage.take_send(step)                   # the message is in pinned host memory
-                rl, rc = stage.recv_buffers(step)
-                lut_tag, codes_tag = message_tags(step)
-                works[step] = [dist.isend(lut_h, dst, group=group, tag=lut_tag), dist.irecv(rl, src, group=group, tag=lut_tag),
-                               dist.isend(codes_h, dst, group=group, tag=codes_tag), dist.irecv(rc, src, group=group, tag=codes_tag)]
+                pending = step
+        hand_over()
         assert not works
     assert not own

@@ -211,3 +211,31 @@ def test_segmented_pointwise_passes_equal_the_one_tensor_calls(dev, oracle):
                 m = torch.zeros_like(p1[k])
                 ops.outer_sgd_nesterov_(p1[k], m, grads[k], None, 0.7, 0.9, True)
                 assert np.array_equal(bits(params[k]), bits(p1[k]))
+
+
+def test_batched_op_routes_a_set_with_a_large_entry_through_the_segmented_call(dev):
+    # prime::uniform_8bit_quantize_batched gives every tensor one workgroup; with host-visible offsets a set that
+    # holds an entry of more than 65,536 elements takes the segmented path instead: same results as tensor by tensor
+    from prime_amd import _lib, ops
+
+    g = torch.Generator(device=dev).manual_seed(36)
+    sizes = [5_000, 300_000, 0, 12, 70_000]
+    flat = torch.randn(sum(sizes), device=dev, generator=g) * 1e-3
+    off = torch.tensor(np.concatenate([[0], np.cumsum(sizes)]), dtype=torch.int64)        # on the host
+    _lib.profile_begin()
+    codes, luts, qps = ops.uniform_8bit_quantize_batched(flat, off)
+    kernels = _lib.profile_end()
+    assert "batched_kernel" not in kernels and "seg_quantize_kernel+hist" in kernels
+    bounds = off.tolist()
+    for t, (a, b) in enumerate(zip(bounds, bounds[1:])):
+        c1, l1, q1 = ops.uniform_8bit_quantize_stats(flat[a:b])
+        assert torch.equal(codes[a:b], c1) and np.array_equal(bits(luts[t]), bits(l1))
+        if b > a:
+            assert np.array_equal(bits(qps[t]), bits(q1))
+    with pytest.raises(RuntimeError, match="non-decreasing"):
+        ops.uniform_8bit_quantize_batched(flat, torch.tensor([0, 10, 5], dtype=torch.int64))
+    # small entries only: the one-launch kernel, as before
+    off2 = torch.tensor([0, 100, 4000, 4000, 60_000], dtype=torch.int64)
+    _lib.profile_begin()
+    ops.uniform_8bit_quantize_batched(flat, off2)
+    assert list(_lib.profile_end()) == ["batched_kernel"]

@@ -67,6 +67,50 @@ def test_fake_tensors_give_shapes():
         assert codes.shape == (3, 5) and codes.dtype == torch.uint8 and lut.shape == (256,) and lut.dtype == torch.float32
 
 
+def test_every_prime_op_traces_on_fake_tensors():
+    # every op of the library has a shape-only implementation: a traced program can carry any of them
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    import prime_amd.ops  # noqa: F401
+
+    P = torch.ops.prime
+    with FakeTensorMode():
+        x = torch.empty(3, 5)
+        flat = torch.empty(40)
+        codes = torch.empty(40, dtype=torch.uint8)
+        lut = torch.empty(256)
+        u8 = (torch.uint8, torch.float32)
+
+        def pair(out, shape):
+            assert out[0].shape == shape and (out[0].dtype, out[1].dtype) == u8 and out[1].shape == (256,)
+
+        calls = {
+            "uniform_8bit_quantize": lambda: pair(P.uniform_8bit_quantize(x), (3, 5)),
+            "uniform_8bit_quantize_literal": lambda: pair(P.uniform_8bit_quantize_literal(x), (3, 5)),
+            "average_buckets": lambda: P.average_buckets(flat, codes, 300).shape == (300,) or pytest.fail("shape"),
+            "quantize_per_tensor_uint8": lambda: P.quantize_per_tensor_uint8(x, 0.1, 128).dtype == torch.uint8 or pytest.fail("dtype"),
+            "dequantize": lambda: P.dequantize(codes, lut).dtype == torch.float32 or pytest.fail("dtype"),
+            "dequantize_": lambda: P.dequantize_(flat, codes, lut, True),
+            "ring_reduce_step": lambda: pair(P.ring_reduce_step(flat, codes, lut), (40,)),
+            "ring_gather_step": lambda: pair(P.ring_gather_step(flat, codes, lut), (40,)),
+            "ring_reduce_div_step": lambda: pair(P.ring_reduce_div_step(flat, codes, lut, 4.0), (40,)),
+            "requantize_codes": lambda: pair(P.requantize_codes(codes, lut), (40,)),
+            "uniform_8bit_quantize_stats": lambda: P.uniform_8bit_quantize_stats(x)[2].shape == (4,) or pytest.fail("qparams"),
+            "uniform_8bit_quantize_batched": lambda: P.uniform_8bit_quantize_batched(flat, torch.empty(6, dtype=torch.int64))[1].shape == (5, 256)
+                                                     or pytest.fail("luts"),
+            "div_": lambda: P.div_(flat, 2.0),
+            "pseudo_gradient_": lambda: P.pseudo_gradient_(flat, flat.clone(), flat.clone(), 4.0),
+            "ring_first_touch_": lambda: (pair(P.ring_first_touch_(flat, flat.clone(), flat.clone(), 4.0, codes, lut, 1.0), (40,)),
+                                          pair(P.ring_first_touch_(flat, flat.clone(), flat.clone(), 4.0, None, None, 1.0), (40,))),
+            "outer_sgd_nesterov_": lambda: (P.outer_sgd_nesterov_(flat, flat.clone(), flat.clone(), flat.clone(), 0.7, 0.9, True),
+                                            P.outer_sgd_nesterov_(flat, flat.clone(), flat.clone(), None, 0.7, 0.9, False)),
+            "outer_sgd_nesterov_codes_": lambda: P.outer_sgd_nesterov_codes_(flat, flat.clone(), codes, lut, flat.clone(), 0.7, 0.9, False),
+        }
+        for name, call in calls.items():
+            call()
+    defined = {s.name.split("::")[1] for s in torch._C._jit_get_all_schemas() if s.name.startswith("prime::")}
+    assert defined == set(calls), defined ^ set(calls)
+
+
 def test_ring_allreduce_rejects_other_reduce_ops():
     # collectives.cpp:83
     from prime_amd.C.collectives import ring_allreduce
@@ -204,3 +248,43 @@ def test_all_reduce_timing_script_without_compression_on_two_host_ranks():
     line = _run_ranks(["--size_model", "100001", "--n_iters", "2", "--compression", "no", "--check"], world=2)
     assert line["ranks"] == 2 and line["size_model"] == 100001 and line["compression"] == "no"
     assert line["MBps"] > 0 and line["rms_error"] < 1e-6
+
+
+def _gloo_avg_worker(rank: int, world: int, port: int, q) -> None:
+    import os
+
+    os.environ.update(MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port))
+    dist.init_process_group("gloo", rank=rank, world_size=world)
+    try:
+        from prime_amd.collectives import gloo_all_reduce
+
+        x = torch.arange(8, dtype=torch.float32) * (rank + 1)
+        gloo_all_reduce(x, dist.ReduceOp.AVG)
+        y = torch.ones(4) * (rank + 1)
+        gloo_all_reduce(y, dist.ReduceOp.SUM)
+        q.put((rank, x.tolist(), y.tolist()))
+    finally:
+        dist.destroy_process_group()
+
+
+def test_uncompressed_all_reduce_averages_over_a_real_gloo_group():
+    # src/zeroband/collectives.py:12-28 with op = AVG on host tensors: divide by the group size, then SUM
+    # (Gloo has no AVG of its own); two ranks, CPU only
+    import socket
+    import torch.multiprocessing as mp
+
+    with socket.socket() as s:
+        s.bind(("127.0.0.1", 0))
+        port = s.getsockname()[1]
+    ctx = mp.get_context("spawn")
+    q = ctx.Queue()
+    procs = [ctx.Process(target=_gloo_avg_worker, args=(r, 2, port, q)) for r in range(2)]
+    for p in procs:
+        p.start()
+    got = [q.get(timeout=120) for _ in procs]
+    for p in procs:
+        p.join(timeout=60)
+        assert p.exitcode == 0
+    for _, x, y in got:
+        assert x == [1.5 * k for k in range(8)]       # (k + 2 k) / 2
+        assert y == [3.0] * 4
