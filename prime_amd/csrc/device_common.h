@@ -30,11 +30,29 @@ constexpr int kZeroPoint = 128;          // compression.cpp:107
 constexpr int kMaxGrid = 2048;           // per-workgroup partial slots in the workspace
 constexpr int kUnroll = PRIME_UNROLL;
 constexpr int kDivUnroll = PRIME_UNROLL > 2 ? 2 : PRIME_UNROLL;   // vectors per step in the kernels that divide
-constexpr int kShotThreads = 256;        // workgroup of a one-tile-per-workgroup launch
+#ifndef PRIME_SHOT_THREADS
+#define PRIME_SHOT_THREADS 256
+#endif
+constexpr int kShotThreads = PRIME_SHOT_THREADS;   // workgroup of a one-tile-per-workgroup launch
 #ifndef PRIME_SHOT_UNROLL
 #define PRIME_SHOT_UNROLL 2
 #endif
 constexpr int kShotUnroll = PRIME_SHOT_UNROLL;   // rows of its tile
+// The tile of a one-workgroup-per-tile launch, by kind of kernel (lanes, rows of that many 16-byte vectors).  Kernels that
+// only stream (copy, divide, pseudo-gradient, outer step) do best with the smallest tile there is, one wavefront and one
+// vector per lane: at 2^28 elements the pseudo-gradient takes 482 us instead of 552 (256 lanes, two rows), the outer step
+// 1060 instead of 1160, a copy 321 instead of 347.  Kernels that first bring the lookup table into LDS want that cost spread
+// over more lanes: accumulate 128 lanes x 2 rows (373 against 380 us), outer step from codes 128 x 1 (915 against 1005),
+// set 256 x 2 (211; 64 x 1: 389); the plain quantizer (16 bytes in, 4 out) 256 x 2 (208; 64 x 1: 257).
+#ifndef PRIME_STREAM_SHOT_THREADS
+#define PRIME_STREAM_SHOT_THREADS 64
+#endif
+#ifndef PRIME_STREAM_SHOT_ROWS
+#define PRIME_STREAM_SHOT_ROWS 1
+#endif
+constexpr int kStreamShotThreads = PRIME_STREAM_SHOT_THREADS, kStreamShotRows = PRIME_STREAM_SHOT_ROWS;
+constexpr int kCodesStepShotThreads = 128, kCodesStepShotRows = 1;
+constexpr int kAddShotThreads = 128, kAddShotRows = 2;
 // wavefronts per SIMD the streaming kernels are compiled for (4 SIMDs per compute unit, at
 // most 8 wavefronts each): bounds their register use so that PRIME_BLOCKS_PER_CU workgroups fit
 constexpr int kWavesPerSimd = (PRIME_THREADS / 64) * PRIME_BLOCKS_PER_CU / 4 > 8 ? 8

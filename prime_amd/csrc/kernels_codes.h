@@ -229,12 +229,12 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_remap_kernel(con
 // against 7.5 us, 2^24: 13.1 against 15.4 us) and with two beyond (2^26: 54 against 58 us, 2^28: 211 against 242 us).
 // dequant_block is the pass for the calling workgroup as workgroup `slot` of a grid of G would run it
 // (s_lut: 256 floats of LDS; the statistics partial goes to part_sum[slot] / part_sq[slot]).
-template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT, int SHOT_ROWS>
+template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT, int SHOT_ROWS, int SHOT_THREADS = kShotThreads>
 __device__ __forceinline__ void dequant_block(float* __restrict__ out, const float* __restrict__ lut, const uint8_t* __restrict__ codes,
                                               int64_t n, double* part_sum, double* part_sq, float divisor, int slot, int G, float* s_lut) {
     static_assert(!(ONESHOT && STATS), "statistics partials need the small grid of the looping sweep");
     using M = Mem<ALIGNED, NT>;
-    constexpr int T = ONESHOT ? kShotThreads : kThreads;
+    constexpr int T = ONESHOT ? SHOT_THREADS : kThreads;
     // The table goes to LDS once per workgroup, first thing.  A workgroup of the plain set that lives
     // for one tile issues the tile's loads before that, so that the table's trip to L2 runs beside the
     // codes' trip to memory instead of in front of it (2^28 elements: 210 instead of 233 us; with the
@@ -258,7 +258,7 @@ __device__ __forceinline__ void dequant_block(float* __restrict__ out, const flo
         for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
             const bool ok = full || i < nvec;
-            c[j] = ok ? M::ldu32(codes, i) : 0u;
+            c[j] = ok ? Mem<ALIGNED, true>::ldu32(codes, i) : 0u;      // a message is read once: never kept in cache
             if (ADD) a[j] = ok ? M::ldf4(out, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
         if (kLateFill) fill_lut();        // every workgroup of such a launch has a tile: the barrier is uniform
@@ -296,12 +296,13 @@ __device__ __forceinline__ void dequant_block(float* __restrict__ out, const flo
     if (STATS) block_stats_store(s0 + s1, q0 + q1, part_sum, part_sq, slot);
 }
 
-template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT = false, int SHOT_ROWS = kShotUnroll>
-__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd)
+template <bool ADD, bool STATS, bool ALIGNED, bool NT, bool DIV, int POLICY, bool ONESHOT = false, int SHOT_ROWS = kShotUnroll,
+          int SHOT_THREADS = kShotThreads>
+__global__ __launch_bounds__(ONESHOT ? SHOT_THREADS : kThreads, ONESHOT ? 8 : kWavesPerSimd)
 void dequant_kernel(float* __restrict__ out, const float* __restrict__ lut, const uint8_t* __restrict__ codes, int64_t n, Workspace* ws,
                     float divisor) {
     __shared__ float s_lut[kBins];
     if (STATS && blockIdx.x == 0 && threadIdx.x == 0) ws->tile_counter = 0u;      // for the quantize pass that follows (sweep_tiles_dynamic)
-    dequant_block<ADD, STATS, ALIGNED, NT, DIV, POLICY, ONESHOT, SHOT_ROWS>(out, lut, codes, n, STATS ? ws->part_sum : nullptr,
+    dequant_block<ADD, STATS, ALIGNED, NT, DIV, POLICY, ONESHOT, SHOT_ROWS, SHOT_THREADS>(out, lut, codes, n, STATS ? ws->part_sum : nullptr,
                                                                            STATS ? ws->part_sq : nullptr, divisor, blockIdx.x, gridDim.x, s_lut);
 }

@@ -10,12 +10,12 @@ __global__ void fill_zero_kernel(uint32_t* p, int64_t nwords) {
 }
 
 // chunk /= world_size for ReduceOp::AVG (collectives.cpp:155-159): an fp32 division in place.
-template <bool ALIGNED, int POLICY, bool ONESHOT = false>
-__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void div_kernel(float* __restrict__ x, int64_t n, float d) {
+template <bool ALIGNED, int POLICY, bool ONESHOT = false, int ST = kStreamShotThreads, int SU = kStreamShotRows>
+__global__ __launch_bounds__(ONESHOT ? ST : kThreads, ONESHOT ? 8 : kWavesPerSimd) void div_kernel(float* __restrict__ x, int64_t n, float d) {
     using M = Mem<ALIGNED, false>;
     const int64_t nvec = n >> 2;
-    constexpr int T = ONESHOT ? kShotThreads : kThreads;
-    constexpr int U = ONESHOT ? kShotUnroll : kDivUnroll;
+    constexpr int T = ONESHOT ? ST : kThreads;
+    constexpr int U = ONESHOT ? SU : kDivUnroll;
     walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
@@ -46,13 +46,13 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
 // divided by the world size; an fp32 subtraction and an fp32 division per element.
 // 12 bytes per element.
 // pseudo_gradient_block is the pass for the calling workgroup as workgroup `slot` of a grid of G.
-template <bool ALIGNED, bool NT, int POLICY, bool ONESHOT>
+template <bool ALIGNED, bool NT, int POLICY, bool ONESHOT, int ST = kStreamShotThreads, int SU = kStreamShotRows>
 __device__ __forceinline__ void pseudo_gradient_block(const float* __restrict__ outer, const float* __restrict__ inner, int64_t n,
                                                       float world_size, float* __restrict__ out, int64_t slot, int64_t G) {
     using M = Mem<ALIGNED, NT>;
     const int64_t nvec = n >> 2;
-    constexpr int T = ONESHOT ? kShotThreads : kThreads;
-    constexpr int U = ONESHOT ? kShotUnroll : kDivUnroll;
+    constexpr int T = ONESHOT ? ST : kThreads;
+    constexpr int U = ONESHOT ? SU : kDivUnroll;
     walk_tiles_of<T, U, ONESHOT>(nvec, slot, G, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
@@ -82,7 +82,7 @@ __device__ __forceinline__ void pseudo_gradient_block(const float* __restrict__ 
 }
 
 template <bool ALIGNED, bool NT, int POLICY, bool ONESHOT = false>
-__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer, const float* __restrict__ inner, int64_t n,
+__global__ __launch_bounds__(ONESHOT ? kStreamShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void pseudo_gradient_kernel(const float* __restrict__ outer, const float* __restrict__ inner, int64_t n,
                                             float world_size, float* __restrict__ out) {
     pseudo_gradient_block<ALIGNED, NT, POLICY, ONESHOT>(outer, inner, n, world_size, out, blockIdx.x, gridDim.x);
 }
@@ -96,7 +96,9 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
 // statistics of the quantization that follows.  12 bytes per element, 13 with codes.  (Only the
 // variant with CODES is launched: without a message the pseudo-gradient as one workgroup per tile
 // followed by the statistics kernel is faster than this loop.)
-template <bool CODES, bool ALIGNED, bool NT, int POLICY>
+// RECIP: world_size and divisor are powers of two and arrive as their reciprocals; x * 2^-k is x / 2^k bit for
+// bit, and the pass then takes tiles of four rows instead of two (no division sequences to hold registers for).
+template <bool CODES, bool ALIGNED, bool NT, int POLICY, bool RECIP = false>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(const float* __restrict__ outer,
                                                                                const float* __restrict__ inner, int64_t n,
                                                                                float world_size, const uint8_t* __restrict__ codes,
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
     }
     const bool div = divisor != 1.0f;
     const int64_t nvec = n >> 2;
-    constexpr int U = kDivUnroll;
+    constexpr int U = RECIP ? kUnroll : kDivUnroll;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
     sweep_tiles<U>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
@@ -130,7 +132,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
-            f4a v = (a[j] - b[j]) / world_size;
+            f4a v = RECIP ? (a[j] - b[j]) * world_size : (a[j] - b[j]) / world_size;
             if (CODES) {
                 f4a l;
                 l.x = s_lut[c[j] & 255];
@@ -138,7 +140,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
                 l.z = s_lut[(c[j] >> 16) & 255];
                 l.w = s_lut[c[j] >> 24];
                 v += l;
-                if (div) v = v / divisor;
+                if (div) v = RECIP ? v * divisor : v / divisor;
             }
             if (full || i < nvec) {
                 if (ALIGNED) win.template st128<POLICY>(static_cast<uint32_t>(threadIdx.x + j * stride) * 16u, v);
@@ -149,10 +151,10 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void first_touch_kernel(co
     });
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
-        float v = (outer[i] - inner[i]) / world_size;
+        float v = RECIP ? (outer[i] - inner[i]) * world_size : (outer[i] - inner[i]) / world_size;
         if (CODES) {
             v += s_lut[codes[i]];
-            if (div) v = v / divisor;
+            if (div) v = RECIP ? v * divisor : v / divisor;
         }
         out[i] = v;
         const double d = v;
@@ -180,13 +182,14 @@ __device__ __forceinline__ void outer_sgd_one(float& p, float& buf, float g, flo
 // element, and the dequantize pass is saved).
 // outer_step_block is the pass for the calling workgroup as workgroup `slot` of a grid of G (s_lut: 256
 // floats of LDS, used with CODES).
-template <bool CODES, bool ALIGNED, bool NT, int POLICY, bool ONESHOT>
+template <bool CODES, bool ALIGNED, bool NT, int POLICY, bool ONESHOT, int ST = CODES ? kCodesStepShotThreads : kStreamShotThreads,
+          int SU = CODES ? kCodesStepShotRows : kStreamShotRows>
 __device__ __forceinline__ void outer_step_block(float* __restrict__ param, float* __restrict__ mom, const float* __restrict__ grad,
                                                  const uint8_t* __restrict__ codes, const float* __restrict__ lut, float* __restrict__ inner,
                                                  int64_t n, float neg_lr, float mu, int first, int64_t slot, int64_t G, float* s_lut) {
     using M = Mem<ALIGNED, NT>;
-    constexpr int T = ONESHOT ? kShotThreads : kThreads;
-    constexpr int U = ONESHOT ? kShotUnroll : kUnroll;
+    constexpr int T = ONESHOT ? ST : kThreads;
+    constexpr int U = ONESHOT ? SU : kUnroll;
     if (CODES) {
         for (int b = threadIdx.x; b < kBins; b += T) s_lut[b] = lut[b];
         __syncthreads();
@@ -248,7 +251,7 @@ __device__ __forceinline__ void outer_step_block(float* __restrict__ param, floa
 }
 
 template <bool CODES, bool ALIGNED, bool NT, int POLICY, bool ONESHOT = false>
-__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom, const float* __restrict__ grad,
+__global__ __launch_bounds__(ONESHOT ? (CODES ? kCodesStepShotThreads : kStreamShotThreads) : kThreads, ONESHOT ? 8 : kWavesPerSimd) void outer_step_kernel(float* __restrict__ param, float* __restrict__ mom, const float* __restrict__ grad,
                                        const uint8_t* __restrict__ codes, const float* __restrict__ lut, float* __restrict__ inner,
                                        int64_t n, float neg_lr, float mu, int first) {
     __shared__ float s_lut[CODES ? kBins : 1];
@@ -256,10 +259,10 @@ __global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kW
 }
 
 template <int POLICY, bool ONESHOT = false>
-__global__ __launch_bounds__(ONESHOT ? kShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
+__global__ __launch_bounds__(ONESHOT ? kStreamShotThreads : kThreads, ONESHOT ? 8 : kWavesPerSimd) void copy_kernel(f4a* __restrict__ dst, const f4a* __restrict__ src, int64_t nvec) {
     using M = Mem<true, true>;
-    constexpr int T = ONESHOT ? kShotThreads : kThreads;
-    constexpr int U = ONESHOT ? kShotUnroll : kUnroll;
+    constexpr int T = ONESHOT ? kStreamShotThreads : kThreads;
+    constexpr int U = ONESHOT ? kStreamShotRows : kUnroll;
     walk_tiles<T, U, ONESHOT>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;

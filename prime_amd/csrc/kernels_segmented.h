@@ -182,14 +182,14 @@ struct SegPointwiseJob {
 static_assert(sizeof(SegPointwiseJob) <= 4000, "the descriptors must fit the kernel argument segment");
 
 template <int POLICY>
-__global__ __launch_bounds__(kShotThreads, 8) void seg_pseudo_gradient_kernel(const SegPointwiseJob job, float world_size) {
+__global__ __launch_bounds__(kStreamShotThreads, 8) void seg_pseudo_gradient_kernel(const SegPointwiseJob job, float world_size) {
     const int t = seg_tensor_of(job.first, job.count, blockIdx.x);
     pseudo_gradient_block<true, true, POLICY, true>(job.a[t], job.b[t], job.n[t], world_size, job.c[t], blockIdx.x - job.first[t],
                                                    job.first[t + 1] - job.first[t]);
 }
 
 template <int POLICY>
-__global__ __launch_bounds__(kShotThreads, 8) void seg_outer_step_kernel(const SegPointwiseJob job, float neg_lr, float mu, int first) {
+__global__ __launch_bounds__(kStreamShotThreads, 8) void seg_outer_step_kernel(const SegPointwiseJob job, float neg_lr, float mu, int first) {
     const int t = seg_tensor_of(job.first, job.count, blockIdx.x);
     outer_step_block<false, true, true, POLICY, true>(job.a[t], job.b[t], job.c[t], nullptr, nullptr, job.d[t], job.n[t], neg_lr, mu, first,
                                                      blockIdx.x - job.first[t], job.first[t + 1] - job.first[t], nullptr);

@@ -125,12 +125,14 @@ int grid_for(int64_t n, bool reads = false) {
 }
 
 // One workgroup per tile for a kernel launched ONESHOT.
-int shot_grid(int64_t nvec, int rows = kShotUnroll) {
-    const int64_t tile = static_cast<int64_t>(kShotThreads) * rows;
+int shot_grid(int64_t nvec, int rows = kShotUnroll, int threads = kShotThreads) {
+    const int64_t tile = static_cast<int64_t>(threads) * rows;
     return static_cast<int>((nvec + tile - 1) / tile);
 }
-// (a dispatch counts its work-items in 32 bits: beyond 2^34 elements the looping kernels take over)
-inline bool one_shot(int64_t n) { return g_opt.one_shot && n >= g_opt.one_shot_min_elems && n <= (int64_t(1) << 34); }
+int stream_shot_grid(int64_t nvec) { return shot_grid(nvec, kStreamShotRows, kStreamShotThreads); }
+// (a dispatch counts its work-items in 32 bits, and a launch of one vector per lane has one work-item per vector: beyond
+// 2^33 elements the looping kernels take over)
+inline bool one_shot(int64_t n) { return g_opt.one_shot && n >= g_opt.one_shot_min_elems && n <= (int64_t(1) << 33); }
 
 // after_writer: the kernel before wrote the tensor (ring step, pseudo-gradient) instead of reading it: half the limit
 // (ring step of 2^26 elements: the quantize pass 51 us with four rows, 62 with two; of 2^25: 27.4 and 26.4)
@@ -309,6 +311,9 @@ void launch_dequant(int id, double bytes, int grid, hipStream_t st, float* out, 
                 if (!ADD && n <= g_opt.set_four_rows_max_elems)
                     launch(id, bytes, dequant_kernel<ADD, false, true, true, DIV, decltype(P)::value, true, 4>, shot_grid(n >> 2, 4), kShotThreads, st,
                            out, lut, codes, n, ws, divisor);
+                else if (ADD)
+                    launch(id, bytes, dequant_kernel<ADD, false, true, true, DIV, decltype(P)::value, true, kAddShotRows, kAddShotThreads>,
+                           shot_grid(n >> 2, kAddShotRows, kAddShotThreads), kAddShotThreads, st, out, lut, codes, n, ws, divisor);
                 else
                     launch(id, bytes, dequant_kernel<ADD, false, true, true, DIV, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, out, lut,
                            codes, n, ws, divisor);
@@ -995,7 +1000,7 @@ int prime_div_f32(float* x, int64_t n, float divisor, prime_stream_t stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (aligned_to(x, 16) && one_shot(n))
         with_policy(g_opt.one_shot_store_policy, [&](auto P) {
-            launch(kIdDiv, 8.0 * n, div_kernel<true, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, x, n, divisor);
+            launch(kIdDiv, 8.0 * n, div_kernel<true, decltype(P)::value, true>, stream_shot_grid(n >> 2), kStreamShotThreads, st, x, n, divisor);
         });
     else if (aligned_to(x, 16))
         with_policy(g_opt.f32_store_policy, [&](auto P) {
@@ -1015,7 +1020,7 @@ int prime_pseudo_gradient_f32(const float* outer, const float* inner, int64_t n,
     const bool pg_aligned = aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(out, 16);
     if (pg_aligned && one_shot(n))
         with_policy(g_opt.one_shot_store_policy, [&](auto P) {
-            launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<true, true, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, outer,
+            launch(kIdPseudoGrad, 12.0 * n, pseudo_gradient_kernel<true, true, decltype(P)::value, true>, stream_shot_grid(n >> 2), kStreamShotThreads, st, outer,
                    inner, n, world_size, out);
         });
     else if (pg_aligned)
@@ -1054,14 +1059,24 @@ int prime_ring_first_touch(const float* outer, const float* inner, int64_t n, fl
     }
     int grid = grid_for(n, true);
     const bool al = aligned_to(outer, 16) && aligned_to(inner, 16) && aligned_to(grad_out, 16) && aligned_to(codes_in, 4);
-    if (al)
+    // a power of two divides exactly as its reciprocal multiplies: x / 2^k == x * 2^-k bit for bit
+    auto pow2 = [](float f) {
+        uint32_t b;
+        memcpy(&b, &f, 4);
+        const uint32_t e = b >> 23;                  // sign 0, exponent field
+        return (b & 0x7fffffu) == 0 && e >= 2 && e <= 252;
+    };
+    // outer, inner and the message are read once: always with the non-temporal hint, so that what the last-level cache
+    // keeps is the gradient this pass writes and the quantize pass reads back (2^26 elements: that pass 52 instead of 66 us)
+    if (al && pow2(world_size) && pow2(divisor))
         with_policy(g_opt.f32_reread_store_policy, [&](auto P) {
-            if (use_nt(n))
-                launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, true, true, decltype(P)::value>, grid, kThreads, st, outer,
-                       inner, n, world_size, codes_in, lut_in, divisor, grad_out, w);
-            else
-                launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, true, false, decltype(P)::value>, grid, kThreads, st, outer,
-                       inner, n, world_size, codes_in, lut_in, divisor, grad_out, w);
+            launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, true, true, decltype(P)::value, true>, grid, kThreads, st, outer,
+                   inner, n, 1.0f / world_size, codes_in, lut_in, 1.0f / divisor, grad_out, w);
+        });
+    else if (al)
+        with_policy(g_opt.f32_reread_store_policy, [&](auto P) {
+            launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, true, true, decltype(P)::value>, grid, kThreads, st, outer,
+                   inner, n, world_size, codes_in, lut_in, divisor, grad_out, w);
         });
     else
         launch(kIdFirstTouchCodes, 13.0 * n, first_touch_kernel<true, false, false, kStorePlain>, grid, kThreads, st, outer, inner, n, world_size,
@@ -1084,7 +1099,7 @@ int prime_outer_sgd_nesterov_f32(float* param, float* momentum_buf, const float*
     const float* no_lut = nullptr;
     if (al && one_shot(n))
         with_policy(g_opt.one_shot_store_policy, [&](auto P) {
-            launch(kIdOuterStep, bytes, outer_step_kernel<false, true, true, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, param,
+            launch(kIdOuterStep, bytes, outer_step_kernel<false, true, true, decltype(P)::value, true>, stream_shot_grid(n >> 2), kStreamShotThreads, st, param,
                    momentum_buf, grad, no_codes, no_lut, inner_out, n, -lr, momentum, first_step);
         });
     else if (al)
@@ -1114,7 +1129,7 @@ int prime_outer_sgd_nesterov_u8(float* param, float* momentum_buf, const uint8_t
     const float* no_grad = nullptr;
     if (al && one_shot(n))
         with_policy(g_opt.one_shot_store_policy, [&](auto P) {
-            launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, true, true, decltype(P)::value, true>, shot_grid(n >> 2), kShotThreads, st, param,
+            launch(kIdOuterStepCodes, bytes, outer_step_kernel<true, true, true, decltype(P)::value, true>, shot_grid(n >> 2, kCodesStepShotRows, kCodesStepShotThreads), kCodesStepShotThreads, st, param,
                    momentum_buf, no_grad, codes, lut, inner_out, n, -lr, momentum, first_step);
         });
     else if (al)
@@ -1145,7 +1160,7 @@ int prime_pseudo_gradient_f32_segmented(const float* const* outers, const float*
         double bytes = 0.0;
         for (int t = 0; t < job.count; ++t) bytes += 12.0 * job.n[t];
         with_policy(g_opt.one_shot_store_policy, [&](auto P) {
-            launch(kIdSegPseudoGrad, bytes, seg_pseudo_gradient_kernel<decltype(P)::value>, job.first[job.count], kShotThreads, st, job, world_size);
+            launch(kIdSegPseudoGrad, bytes, seg_pseudo_gradient_kernel<decltype(P)::value>, job.first[job.count], kStreamShotThreads, st, job, world_size);
         });
         job.count = 0;
         return launch_check("seg_pseudo_gradient_kernel");
@@ -1154,11 +1169,11 @@ int prime_pseudo_gradient_f32_segmented(const float* const* outers, const float*
     for (int64_t i = 0; i < count; ++i) {
         if (ns[i] == 0) continue;
         const bool al = aligned_to(outers[i], 16) && aligned_to(inners[i], 16) && aligned_to(outs[i], 16);
-        if (!al || ns[i] > (int64_t(1) << 34)) {         // the one-tensor entry point takes what a one-workgroup-per-tile launch cannot
+        if (!al || ns[i] > (int64_t(1) << 33)) {         // the one-tensor entry point takes what a one-workgroup-per-tile launch cannot
             if (int rc = prime_pseudo_gradient_f32(outers[i], inners[i], ns[i], world_size, outs[i], stream)) return rc;
             continue;
         }
-        const int blocks = shot_grid(ns[i] >> 2) > 0 ? shot_grid(ns[i] >> 2) : 1;
+        const int blocks = stream_shot_grid(ns[i] >> 2) > 0 ? stream_shot_grid(ns[i] >> 2) : 1;
         if (job.count == kSegMax || job.first[job.count] + static_cast<int64_t>(blocks) > 0x7fffffff)
             if (int rc = flush()) return rc;
         const int t = job.count++;
@@ -1186,7 +1201,7 @@ int prime_outer_sgd_nesterov_f32_segmented(float* const* params, float* const* m
         double bytes = 0.0;
         for (int t = 0; t < job.count; ++t) bytes += (job.d[t] ? 24.0 : 20.0) * job.n[t];
         with_policy(g_opt.one_shot_store_policy, [&](auto P) {
-            launch(kIdSegOuterStep, bytes, seg_outer_step_kernel<decltype(P)::value>, job.first[job.count], kShotThreads, st, job, -lr, momentum,
+            launch(kIdSegOuterStep, bytes, seg_outer_step_kernel<decltype(P)::value>, job.first[job.count], kStreamShotThreads, st, job, -lr, momentum,
                    first_step);
         });
         job.count = 0;
@@ -1197,11 +1212,11 @@ int prime_outer_sgd_nesterov_f32_segmented(float* const* params, float* const* m
         if (ns[i] == 0) continue;
         float* inner = inner_outs ? inner_outs[i] : nullptr;
         const bool al = aligned_to(params[i], 16) && aligned_to(momentum_bufs[i], 16) && aligned_to(grads[i], 16) && aligned_to(inner, 16);
-        if (!al || ns[i] > (int64_t(1) << 34)) {
+        if (!al || ns[i] > (int64_t(1) << 33)) {
             if (int rc = prime_outer_sgd_nesterov_f32(params[i], momentum_bufs[i], grads[i], inner, ns[i], lr, momentum, first_step, stream)) return rc;
             continue;
         }
-        const int blocks = shot_grid(ns[i] >> 2) > 0 ? shot_grid(ns[i] >> 2) : 1;
+        const int blocks = stream_shot_grid(ns[i] >> 2) > 0 ? stream_shot_grid(ns[i] >> 2) : 1;
         if (job.count == kSegMax || job.first[job.count] + static_cast<int64_t>(blocks) > 0x7fffffff)
             if (int rc = flush()) return rc;
         const int t = job.count++;
@@ -1224,7 +1239,7 @@ int prime_copy_bytes(void* dst, const void* src, int64_t n_bytes, prime_stream_t
     const int grid = grid_for(nvec * 4);
     with_policy(g_opt.copy_store_policy, [&](auto P) {
         if (one_shot(nvec * 4))
-            launch(kIdCopy, 2.0 * n_bytes, copy_kernel<decltype(P)::value, true>, shot_grid(nvec), kShotThreads, static_cast<hipStream_t>(stream),
+            launch(kIdCopy, 2.0 * n_bytes, copy_kernel<decltype(P)::value, true>, stream_shot_grid(nvec), kStreamShotThreads, static_cast<hipStream_t>(stream),
                    static_cast<f4a*>(dst), static_cast<const f4a*>(src), nvec);
         else
             launch(kIdCopy, 2.0 * n_bytes, copy_kernel<decltype(P)::value>, grid, kThreads, static_cast<hipStream_t>(stream),
