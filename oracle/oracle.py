@@ -224,17 +224,18 @@ def ring_allreduce_sim(tensors: List[np.ndarray], avg: bool = False, norm: str =
 
     Messages are kept in per-(receiver, step) slots; ranks are stepped in lock step, which
     is equivalent to the reference's asynchronous send/recv with waits at step + 2
-    (BUFFER_COUNT = 2).  Requires numel divisible by 2 W, as the Python twin asserts
-    (src/zeroband/collectives.py:83)."""
+    (BUFFER_COUNT = 2).  Chunks are those of ``flat.chunk(2 W)`` (:90): the last one is shorter
+    when 2 W does not divide numel (the Python twin asserts divisibility,
+    src/zeroband/collectives.py:83; the C++ does not); numel must yield all 2 W chunks."""
     W = len(tensors)
     nb = BUFFER_COUNT * W
     n = tensors[0].size
-    assert n % nb == 0, "Tensor size must be divisible by world size"
-    csz = n // nb
+    bounds = torch_chunk_bounds(n, nb)
+    assert len(bounds) == nb, "torch.chunk gives fewer than 2 W chunks"
     flats = [t.reshape(-1) for t in tensors]
 
     def chunk(r, c):
-        return flats[r][c * csz:(c + 1) * csz]
+        return flats[r][bounds[c][0]:bounds[c][1]]
 
     for phase in (1, 2):
         inbox = [dict() for _ in range(W)]   # inbox[rank][step] = (codes, lut)

@@ -44,10 +44,23 @@ def _check_ring_inputs(tensors: Sequence[torch.Tensor]) -> int:
             raise ValueError("all simulated ranks must hold tensors of one size on one device")
         if not t.is_contiguous():
             raise RuntimeError("ring all-reduce works in place and needs contiguous tensors")
-    if n % (BUFFER_COUNT * len(tensors)) != 0:
-        # the Python twin asserts this (src/zeroband/collectives.py:83)
-        raise ValueError("Tensor size must be divisible by world size")
+    chunk_bounds(n, len(tensors))
     return n
+
+
+def chunk_bounds(n: int, world_size: int) -> List[Tuple[int, int]]:
+    """[lo, hi) of the 2 * world_size chunks ``flat.chunk(2 * world_size)`` cuts a tensor of n elements
+    into (collectives.cpp:89-90): pieces of ceil(n / 2W) elements, the last one shorter when 2W does
+    not divide n.  The reference's C++ takes any n that yields all 2W chunks (its Python twin asserts
+    divisibility, src/zeroband/collectives.py:83); when ``torch.chunk`` returns fewer pieces the C++
+    would index past its chunk list, and this raises instead."""
+    nb = BUFFER_COUNT * world_size
+    size = -(-n // nb) if n else 0
+    bounds = [(lo, min(n, lo + size)) for lo in range(0, n, size)] if size else []
+    if len(bounds) != nb:
+        raise ValueError(f"Tensor size must split into {nb} chunks: torch.chunk cuts {n} elements into {len(bounds)} pieces of "
+                         f"{size} (pad the tensor to a multiple of {nb} elements)")
+    return bounds
 
 
 def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
@@ -81,16 +94,16 @@ def ring_allreduce_simulated(tensors: Sequence[torch.Tensor], avg: bool = False,
         if world_size is None:
             world_size = float(W)
     nb = BUFFER_COUNT * W
-    csz = n // nb
+    bounds = chunk_bounds(n, W)
     flats = [t.view(-1) for t in tensors]
 
     def chunk(r: int, c: int) -> torch.Tensor:
-        return flats[r][c * csz:(c + 1) * csz]
+        return flats[r][bounds[c][0]:bounds[c][1]]
 
     def touch(r: int, c: int, msg, divisor: float):
         # first and only visit of chunk c by rank r in the reduce-scatter, pseudo-gradient included
         o, i = sources[r]
-        sl = slice(c * csz, (c + 1) * csz)
+        sl = slice(*bounds[c])
         return ops.ring_first_touch_(chunk(r, c), o.view(-1)[sl], i.view(-1)[sl], float(world_size),
                                      None if msg is None else msg[0], None if msg is None else msg[1], divisor)
 

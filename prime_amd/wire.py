@@ -34,7 +34,7 @@ import torch
 import torch.distributed as dist
 
 from . import ops
-from .ring import BUFFER_COUNT, _check_ring_inputs
+from .ring import BUFFER_COUNT, _check_ring_inputs, chunk_bounds
 
 LOOKUP_TAG_OFFSET = 1000      # collectives.cpp:141,144
 N_BINS = ops.N_BINS
@@ -68,22 +68,24 @@ class HostStage:
         self._h2d_done: List[Optional[torch.cuda.Event]] = [None] * self.depth
         self._consumed: List[Optional[torch.cuda.Event]] = [None] * self.depth
         self._keep: List[tuple] = [()] * self.depth       # device tensors a copy in flight still reads
+        self._sent_numel: List[int] = [self.chunk_numel] * self.depth
 
     # ---- sending -------------------------------------------------------------------------------
     def post_send(self, step: int, codes: torch.Tensor, lut: torch.Tensor) -> None:
         """Start the device-to-host copy of one message; the kernels that produced it are on the
         current stream.  The slot must have been taken by the transport (``take_send``) before it is
         reused, BUFFER_COUNT steps later."""
-        if codes.numel() != self.chunk_numel or codes.dtype != torch.uint8 or lut.numel() != N_BINS or lut.dtype != torch.float32:
-            raise RuntimeError("post_send: a message is uint8 codes of the chunk size and 256 float32 lookup entries")
+        if codes.numel() > self.chunk_numel or codes.dtype != torch.uint8 or lut.numel() != N_BINS or lut.dtype != torch.float32:
+            raise RuntimeError("post_send: a message is uint8 codes of at most the chunk size and 256 float32 lookup entries")
         slot = step % self.depth
         ready = torch.cuda.current_stream(self.device).record_event()
         self.copy_stream.wait_event(ready)
         with torch.cuda.stream(self.copy_stream):
             self.send_lut[slot].copy_(lut.view(-1), non_blocking=True)
-            self.send_codes[slot].copy_(codes.view(-1), non_blocking=True)
+            self.send_codes[slot][:codes.numel()].copy_(codes.view(-1), non_blocking=True)
             self._d2h_done[slot] = self.copy_stream.record_event()
         self._keep[slot] = (codes, lut)
+        self._sent_numel[slot] = codes.numel()
 
     def take_send(self, step: int) -> Tuple[torch.Tensor, torch.Tensor]:
         """Block until the message of ``step`` is in host memory; returns (lookup, codes), the two
@@ -94,29 +96,32 @@ class HostStage:
             raise RuntimeError(f"no message was posted for step {step}")
         ev.synchronize()
         self._keep[slot] = ()
-        return self.send_lut[slot], self.send_codes[slot]
+        return self.send_lut[slot], self.send_codes[slot][:self._sent_numel[slot]]
 
     # ---- receiving -----------------------------------------------------------------------------
-    def recv_buffers(self, step: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        """(lookup, codes) host tensors for ``recv`` with ``message_tags(step)``.  Blocks until the
+    def recv_buffers(self, step: int, numel: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(lookup, codes) host tensors for ``recv`` with ``message_tags(step)``; ``numel`` codes (the
+        chunk size unless the message is the shorter last chunk of a tensor).  Blocks until the
         host-to-device copy that last read this slot has finished."""
         slot = step % self.depth
         if self._h2d_done[slot] is not None:
             self._h2d_done[slot].synchronize()
-        return self.recv_lut[slot], self.recv_codes[slot]
+        k = self.chunk_numel if numel is None else int(numel)
+        return self.recv_lut[slot], self.recv_codes[slot][:k]
 
-    def to_device(self, step: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        """Start the host-to-device copy of the received message of ``step`` and order the current
-        stream after it; returns (codes, lookup) on the device."""
+    def to_device(self, step: int, numel: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Start the host-to-device copy of the received message of ``step`` (``numel`` codes) and order
+        the current stream after it; returns (codes, lookup) on the device."""
         slot = step % self.depth
+        k = self.chunk_numel if numel is None else int(numel)
         if self._consumed[slot] is not None:
             self.copy_stream.wait_event(self._consumed[slot])      # the kernels that read this device slot last
         with torch.cuda.stream(self.copy_stream):
             self.dev_lut[slot].copy_(self.recv_lut[slot], non_blocking=True)
-            self.dev_codes[slot].copy_(self.recv_codes[slot], non_blocking=True)
+            self.dev_codes[slot][:k].copy_(self.recv_codes[slot][:k], non_blocking=True)
             self._h2d_done[slot] = self.copy_stream.record_event()
         torch.cuda.current_stream(self.device).wait_event(self._h2d_done[slot])
-        return self.dev_codes[slot], self.dev_lut[slot]
+        return self.dev_codes[slot][:k], self.dev_lut[slot]
 
     def release(self, step: int) -> None:
         """The kernels reading the device slot of ``step`` have been enqueued on the current stream."""
@@ -133,7 +138,7 @@ class Loopback:
 
     def deliver(self, src: HostStage, dst: HostStage, step: int) -> None:
         lut, codes = src.take_send(step)
-        rl, rc = dst.recv_buffers(step)
+        rl, rc = dst.recv_buffers(step, codes.numel())
         rl.copy_(lut)
         rc.copy_(codes)
         self.bytes_moved += lut.numel() * 4 + codes.numel()
@@ -149,7 +154,8 @@ def ring_allreduce_staged(tensors: Sequence[torch.Tensor], avg: bool = False, tr
     W = len(tensors)
     n = _check_ring_inputs(tensors)
     nb = BUFFER_COUNT * W
-    csz = n // nb
+    bounds = chunk_bounds(n, W)
+    csz = bounds[0][1] - bounds[0][0]              # the largest chunk: what the buffers are sized for (collectives.cpp:104)
     flats = [t.view(-1) for t in tensors]
     dev = flats[0].device
     transport = transport or Loopback()
@@ -159,7 +165,7 @@ def ring_allreduce_staged(tensors: Sequence[torch.Tensor], avg: bool = False, tr
         raise ValueError("one HostStage per rank, sized for the chunk, is needed")
 
     def chunk(r: int, c: int) -> torch.Tensor:
-        return flats[r][c * csz:(c + 1) * csz]
+        return flats[r][bounds[c][0]:bounds[c][1]]
 
     own: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
     for phase in (1, 2):
@@ -174,7 +180,7 @@ def ring_allreduce_staged(tensors: Sequence[torch.Tensor], avg: bool = False, tr
                 out = None
                 if got:
                     arrived[r].discard(step - BUFFER_COUNT)
-                    codes_in, lut_in = stages[r].to_device(step - BUFFER_COUNT)
+                    codes_in, lut_in = stages[r].to_device(step - BUFFER_COUNT, ch.numel())
                     if sending:
                         out = (ops.ring_reduce_step if phase == 1 else ops.ring_gather_step)(ch, codes_in, lut_in)
                     elif phase == 1:
@@ -235,13 +241,17 @@ def ring_allreduce_group(tensor: torch.Tensor, avg: bool, group) -> None:
     flat = tensor.view(-1)
     n = _check_ring_inputs([flat] * W)
     nb = BUFFER_COUNT * W
-    csz = n // nb
+    bounds = chunk_bounds(n, W)
+    csz = bounds[0][1] - bounds[0][0]              # the largest chunk (collectives.cpp:104)
     stage = _stage_for(flat.device, csz, group)
     dst = dist.get_global_rank(group, (rank + 1) % W)                    # :111
     src = dist.get_global_rank(group, (rank - 1 + W) % W)               # :112
 
     def chunk(c: int) -> torch.Tensor:
-        return flat[c * csz:(c + 1) * csz]
+        return flat[bounds[c][0]:bounds[c][1]]
+
+    def chunk_of(r: int, phase: int, step: int) -> int:
+        return ((r * BUFFER_COUNT - step) if phase == 1 else (r * BUFFER_COUNT + BUFFER_COUNT - step)) % nb     # :116 / :192
 
     own: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
     for phase in (1, 2):
@@ -257,7 +267,9 @@ def ring_allreduce_group(tensor: torch.Tensor, avg: bool, group) -> None:
             s_ = pending
             pending = None
             lut_h, codes_h = stage.take_send(s_)                         # the message is in pinned host memory
-            rl, rc = stage.recv_buffers(s_)
+            # what arrives is the previous rank's chunk of the same step: its size is known here without being sent
+            prev_c = chunk_of((rank - 1 + W) % W, phase, s_)
+            rl, rc = stage.recv_buffers(s_, bounds[prev_c][1] - bounds[prev_c][0])
             lut_tag, codes_tag = message_tags(s_)
             works[s_] = [dist.isend(lut_h, dst, group=group, tag=lut_tag), dist.irecv(rl, src, group=group, tag=lut_tag),
                          dist.isend(codes_h, dst, group=group, tag=codes_tag), dist.irecv(rc, src, group=group, tag=codes_tag)]
@@ -270,7 +282,7 @@ def ring_allreduce_group(tensor: torch.Tensor, avg: bool, group) -> None:
             if (step - BUFFER_COUNT) in works:
                 for w in works.pop(step - BUFFER_COUNT):                 # :118-122
                     w.wait()
-                codes_in, lut_in = stage.to_device(step - BUFFER_COUNT)
+                codes_in, lut_in = stage.to_device(step - BUFFER_COUNT, ch.numel())
                 if sending:
                     out = (ops.ring_reduce_step if phase == 1 else ops.ring_gather_step)(ch, codes_in, lut_in)
                 elif phase == 1:

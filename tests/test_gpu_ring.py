@@ -121,6 +121,55 @@ def test_whole_schedule_tracks_the_cpu_ring_element_by_element(dev, oracle, W, a
         assert np.abs(gpu[r].cpu().numpy() - ref_t).max() < 2.5 * bin_width
 
 
+@pytest.mark.parametrize("W,avg,n", [(2, False, 100_003), (3, True, 100_001), (4, False, 1_000_001), (8, True, 262_147), (4, True, 29)])
+def test_a_tensor_that_2w_does_not_divide_is_cut_as_torch_chunk_cuts_it(dev, oracle, W, avg, n):
+    # collectives.cpp:89-90 cuts with flat.chunk(2 W): pieces of ceil(n / 2W), the last one shorter.  The whole
+    # schedule on such a tensor against the oracle ring (same cut), element by element as above, through the
+    # lock-stepped ring, the staged ring (messages of two sizes through the pinned slots) and with the
+    # closed form: inputs constant on every chunk come back as the exact sums
+    from prime_amd import ring, wire
+    from prime_amd.ring import chunk_bounds
+
+    bounds = chunk_bounds(n, W)
+    assert len(bounds) == 2 * W and bounds[-1][1] == n and bounds[-1][1] - bounds[-1][0] < bounds[0][1] - bounds[0][0]
+    assert bounds == oracle.torch_chunk_bounds(n, 2 * W)
+    assert [b - a for a, b in bounds] == [c.numel() for c in torch.empty(n).chunk(2 * W)]
+    xs = _inputs(W, n, 300 + W)
+    cpu = [x.copy() for x in xs]
+    oracle.ring_allreduce_sim(cpu, avg=avg)
+    announce(f"ring with a shorter last chunk W={W} avg={avg} n={n}")
+    gpu = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    ring.ring_allreduce_simulated(gpu, avg=avg)
+    staged = [torch.from_numpy(x.copy()).to(dev) for x in xs]
+    wire.ring_allreduce_staged(staged, avg=avg)
+    torch.cuda.synchronize()
+    bin_width = 6 * 10 * math.sqrt(W) / 256 / (W if avg else 1)
+    for r in range(W):
+        assert torch.equal(staged[r], gpu[r])
+        d = np.abs(gpu[r].cpu().numpy() - cpu[r])
+        assert d.max() < 2.5 * bin_width
+        if n > 1000:
+            assert (d > 1e-2 * bin_width).mean() < 2e-3
+    # closed form: rank r holds v[r, c] on chunk c; a constant quantizes without loss, so every rank ends with the
+    # exact sum over the ranks on every chunk (a wrong boundary would mix two constants)
+    if bounds[-1][1] - bounds[-1][0] > 1:
+        vals = np.arange(1, W * 2 * W + 1, dtype=np.float32).reshape(W, 2 * W)
+        flat = []
+        for r in range(W):
+            t = np.empty(n, np.float32)
+            for c, (a, b) in enumerate(bounds):
+                t[a:b] = vals[r, c]
+            flat.append(torch.from_numpy(t).to(dev))
+        ring.ring_allreduce_simulated(flat, avg=False)
+        want = np.empty(n, np.float32)
+        for c, (a, b) in enumerate(bounds):
+            want[a:b] = vals[:, c].sum()
+        for r in range(W):
+            assert np.array_equal(flat[r].cpu().numpy(), want), r
+    with pytest.raises(ValueError, match="split into"):
+        ring.ring_allreduce_simulated([torch.zeros(2 * W + 1, device=dev) for _ in range(W)] if W > 1 else [torch.zeros(1, device=dev)])
+
+
 @pytest.mark.parametrize("W,avg", [(1, False), (2, True), (4, False), (8, True)])
 def test_all_gather_in_the_code_domain_gives_the_same_tensors(dev, W, avg):
     # keep_codes: what is forwarded is requantized from the received codes alone and the fp32 chunk is

@@ -42,7 +42,13 @@ def test_message_tags_and_slot_contents(dev):
     with pytest.raises(RuntimeError, match="posted"):
         wire.HostStage(dev, n).take_send(1)
     with pytest.raises(RuntimeError, match="uint8 codes"):
-        stage.post_send(4, codes[:10], lut)
+        stage.post_send(4, torch.cat([codes, codes[:1]]), lut)          # longer than the slot
+    # a shorter message (the last chunk of a tensor that 2 W does not divide) travels in a prefix of the slot
+    stage.post_send(4, codes[:10], lut)
+    lut_h, codes_h = stage.take_send(4)
+    assert codes_h.numel() == 10 and torch.equal(codes_h, codes[:10].cpu())
+    rl, rc = stage.recv_buffers(4, 10)
+    assert rc.numel() == 10
 
 
 @pytest.mark.parametrize("W,avg", [(1, False), (2, False), (3, True), (4, True), (8, False)])
@@ -91,8 +97,9 @@ def _free_port() -> int:
         return sock.getsockname()[1]
 
 
-@pytest.mark.parametrize("W,op,pg", [(2, "sum", "default"), (4, "sum", "default"), (2, "avg", "newgroup"), (4, "avg", "default")])
-def test_ring_over_a_real_gloo_group_one_process_per_rank(dev, oracle, tmp_path, W, op, pg):
+@pytest.mark.parametrize("W,op,pg,n", [(2, "sum", "default", 1_000_000), (4, "sum", "default", 1_000_000), (2, "avg", "newgroup", 1_000_000),
+                                       (4, "avg", "default", 1_000_000), (4, "sum", "default", 1_000_001), (2, "avg", "default", 999_999)])
+def test_ring_over_a_real_gloo_group_one_process_per_rank(dev, oracle, tmp_path, W, op, pg, n):
     # the reference's own acceptance test (tests/test_c/test_collectives.py:14-68): W processes on
     # localhost, a Gloo group, each rank randn(N) * 10; here every rank's kernels run on the one GPU and
     # only codes + lookup travel (pinned host memory, dist.isend / irecv with the reference's tags).
@@ -106,7 +113,8 @@ def test_ring_over_a_real_gloo_group_one_process_per_rank(dev, oracle, tmp_path,
 
     from prime_amd import ring
 
-    n = 1_000_000 - 1_000_000 % (2 * W)          # N of the reference test, made divisible (collectives.py:83)
+    # N of the reference test (divisible by 2 W, collectives.py:83), and sizes 2 W does not divide: the last chunk is
+    # shorter (collectives.cpp:90) and so are the messages that carry it
     seed = 4000 + W
     root = Path(__file__).resolve().parents[1]
     port = _free_port()

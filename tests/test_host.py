@@ -133,9 +133,9 @@ def test_fake_process_group_is_a_no_op():
 def test_simulated_ring_input_checks():
     from prime_amd.C.collectives import SimulatedRing, ring_allreduce
 
-    a, b = torch.zeros(10), torch.zeros(10)
-    with pytest.raises(ValueError, match="divisible"):
-        ring_allreduce(a, dist.ReduceOp.SUM, SimulatedRing([a, b]))      # 10 % (2*2) != 0
+    a, b = torch.zeros(9), torch.zeros(9)
+    with pytest.raises(ValueError, match="split into 4 chunks"):
+        ring_allreduce(a, dist.ReduceOp.SUM, SimulatedRing([a, b]))      # torch.chunk(4) of 9 elements gives 3 pieces
     with pytest.raises(ValueError, match="not one of"):
         ring_allreduce(torch.zeros(8), dist.ReduceOp.SUM, SimulatedRing([torch.zeros(8), torch.zeros(8)]))
     d = a.double()
