@@ -92,7 +92,7 @@ typedef struct prime_kernel_time {
 int prime_hip_profile_begin(void);
 int prime_hip_profile_end(prime_kernel_time* out, int capacity, int* count);
 
-/* Workspace: a fixed-size block of device memory (about 8 MiB) that holds every workgroup's
+/* Workspace: a fixed-size block of device memory (about 10 MiB) that holds every workgroup's
  * partial sums and partial 256-bin histogram between a kernel and its second stage.  It
  * carries no state from one call to the next; prime_workspace_init only validates it and
  * clears the scale record (a fill kernel, safe under stream capture).  Two calls that share a
@@ -131,7 +131,7 @@ int prime_uniform_8bit_quantize(const float* x, int64_t n, uint8_t* codes, float
 /* prime_uniform_8bit_quantize for callers that cannot allocate device memory or carry a
  * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc): no counterpart in the reference.  The per-workgroup partials live in a scratch
- * array inside the library's own device image (8 MiB + 35 KiB per GPU, held until the process
+ * array inside the library's own device image (10.1 MiB per GPU, held until the process
  * ends; its address is looked up once per device on the first call there).  Calls no hipMalloc,
  * hipFree or other allocating routine.  Same results as prime_uniform_8bit_quantize, bit for
  * bit.  n above 2^40 is rejected with PRIME_EINVAL.  All calls on one GPU share that GPU's

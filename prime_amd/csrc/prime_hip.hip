@@ -372,7 +372,7 @@ bool bad_n(int64_t n) { return n < 0 || n > kMaxElems; }
 }  // namespace
 
 // Scratch of the entry point that allocates nothing: one Workspace per GPU in the code object's
-// own device memory (8 MiB + 35 KiB, held by every device the library runs on until the process
+// own device memory (10.1 MiB, held by every device the library runs on until the process
 // ends).  In host code the array's name is only a stand-in for the symbol, not a device address:
 // the address is looked up once per device with hipGetSymbolAddress, kept, and every launch and
 // every other use of the memory gets that pointer.

@@ -288,3 +288,26 @@ def test_uncompressed_all_reduce_averages_over_a_real_gloo_group():
     for _, x, y in got:
         assert x == [1.5 * k for k in range(8)]       # (k + 2 k) / 2
         assert y == [3.0] * 4
+
+
+def test_bench_takes_its_traffic_figure_from_the_committed_counter_summaries():
+    # roofline.traffic is read from profiles/*_hbm_traffic.txt (the scaled FETCH_SIZE + WRITE_SIZE of the dominant
+    # kernel), not typed into bench.py: the figure exists, belongs to that kernel and is the algorithmic 5 B per
+    # element plus the histogram partials, with no wasted re-reads
+    import re
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    sys.path.insert(0, str(root))
+    import bench
+
+    for profile, elems in (("uniform_2p28_hbm_traffic.txt", 1 << 28), ("cfg2_buckets_hbm_traffic.txt", bench.BUCKET_ELEMS)):
+        got = bench.measured_traffic(profile, "quantize_kernel<true, true, true, true")
+        assert got is not None, profile
+        rows = [l for l in (root / "profiles" / profile).read_text().splitlines() if l.startswith("quantize_kernel<true, true, true, true")]
+        assert rows and any(abs(float(r.split()[-1]) * 1e6 - got) < 1 for r in rows)
+        assert 5 * elems <= got <= 1.01 * 5 * elems, (profile, got, 5 * elems)
+        text = (root / "profiles" / profile).read_text()
+        assert re.search(r"rocprofv3 --pmc FETCH_SIZE", text) and re.search(r"rocprofv3 --pmc WRITE_SIZE", text)
+    assert bench.measured_traffic("no_such_file.txt", "quantize_kernel") is None
