@@ -248,7 +248,18 @@ def main() -> int:
         _lib.check(lib.prime_ring_reduce_step(acc.data_ptr(), codes_in.data_ptr(), lut_in.data_ptr(), acc.numel(),
                                               codes_out.data_ptr(), lut_out.data_ptr(), None, ws.data_ptr(), st), "ring_step")
 
+    # The device reaches its full clocks only after some milliseconds of continuous work (the first dozen
+    # launches after an idle spell run up to a third slower): every timed region is preceded by about 20 ms
+    # of untimed copies on the same stream, then by the warm-up steps, with no host synchronisation between.
+    warm_src = torch.empty(1 << 26, dtype=torch.float32, device=dev).normal_()
+    warm_dst = torch.empty_like(warm_src)
+
+    def warm_device(n_copies=250):
+        for _ in range(n_copies):
+            lib.prime_copy_bytes(warm_dst.data_ptr(), warm_src.data_ptr(), warm_src.numel() * 4, st)
+
     def timed(step_fn, steps, warmup):
+        warm_device()
         for _ in range(warmup):
             step_fn()
         torch.cuda.synchronize()
@@ -429,6 +440,7 @@ def main() -> int:
         for name, (bpe, fn) in calls.items():
             if only and name != "uniform_8bit_quantize (a1)" and not any(w in name for w in only):
                 continue
+            warm_device()
             for r in range(args.warmup):
                 _lib.check(fn(r), name)
             torch.cuda.synchronize()
@@ -453,6 +465,7 @@ def main() -> int:
         # only (the statistics pass above), a plain copy, writing only (torch's fill).  HBM moves reads and
         # writes over one bus in turn, so a kernel that does both is bounded by the sum of the two times.
         def event_timed(fn):
+            warm_device()
             for r in range(args.warmup):
                 fn(r)
             evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]

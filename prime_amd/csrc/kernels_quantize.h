@@ -219,10 +219,11 @@ __global__ __launch_bounds__(kShotThreads, 8) void quantize_shot_kernel(const fl
 }
 
 // K3 alone: histogram of x under caller-supplied codes (average_buckets).  5 bytes per element.
-template <bool ALIGNED, int R>
+// ALLBINS: the table has all 256 bins, so no code is left out and the additions need no predicate.
+template <bool ALIGNED, int R, bool NT, bool ALLBINS>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const float* __restrict__ x, const uint8_t* __restrict__ codes,
                                                         int64_t n, int n_bins, Workspace* ws) {
-    using M = Mem<ALIGNED, false>;
+    using M = Mem<ALIGNED, NT>;
     __shared__ LdsHist<R> hist;
     hist_zero(hist);
     __syncthreads();
@@ -243,10 +244,10 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const flo
             const int64_t i = i0 + j * stride;
             if (full || i < nvec) {
                 const int a = c[j] & 255, b = (c[j] >> 8) & 255, cc = (c[j] >> 16) & 255, d = c[j] >> 24;
-                if (a < n_bins) hist_add(hist, a, v[j].x);     // compression.cpp:70
-                if (b < n_bins) hist_add(hist, b, v[j].y);
-                if (cc < n_bins) hist_add(hist, cc, v[j].z);
-                if (d < n_bins) hist_add(hist, d, v[j].w);
+                if (ALLBINS || a < n_bins) hist_add(hist, a, v[j].x);     // compression.cpp:70
+                if (ALLBINS || b < n_bins) hist_add(hist, b, v[j].y);
+                if (ALLBINS || cc < n_bins) hist_add(hist, cc, v[j].z);
+                if (ALLBINS || d < n_bins) hist_add(hist, d, v[j].w);
             }
         }
     });

@@ -591,8 +591,10 @@ int prime_average_buckets(const float* x, const uint8_t* codes, int64_t n, int64
         const bool al = aligned_to(x, 16) && aligned_to(codes, 4);
         auto go = [&](auto copies) {
             constexpr int R = decltype(copies)::value;
-            if (al) launch(kIdHist, 5.0 * n, hist_kernel<true, R>, grid, kThreads, st, x, codes, n, nb, w);
-            else launch(kIdHist, 5.0 * n, hist_kernel<false, R>, grid, kThreads, st, x, codes, n, nb, w);
+            if (al && nb == kBins && use_nt(n)) launch(kIdHist, 5.0 * n, hist_kernel<true, R, true, true>, grid, kThreads, st, x, codes, n, nb, w);
+            else if (al && nb == kBins) launch(kIdHist, 5.0 * n, hist_kernel<true, R, false, true>, grid, kThreads, st, x, codes, n, nb, w);
+            else if (al) launch(kIdHist, 5.0 * n, hist_kernel<true, R, false, false>, grid, kThreads, st, x, codes, n, nb, w);
+            else launch(kIdHist, 5.0 * n, hist_kernel<false, R, false, false>, grid, kThreads, st, x, codes, n, nb, w);
         };
         switch (g_opt.average_replicas) {
             case 1: go(std::integral_constant<int, 1>{}); break;
