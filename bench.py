@@ -883,61 +883,66 @@ def main() -> int:
         # ---- the PCIe side of a host transport: codes + lookup through pinned host double buffers ---------
         from prime_amd import wire
 
-        n_s = RING_CHUNK
-        stage = wire.HostStage(dev, n_s)
-        g = torch.Generator(device=dev).manual_seed(21)
-        accs = [torch.randn(n_s, device=dev, generator=g) * 1e-3 for _ in range(4)]
-        c_s, l_s = ops.uniform_8bit_quantize(accs[0])
-        hops_s = 6
+        def staging_at(n_s):
+            stage = wire.HostStage(dev, n_s)
+            g = torch.Generator(device=dev).manual_seed(21)
+            accs = [torch.randn(n_s, device=dev, generator=g) * 1e-3 for _ in range(4)]
+            c_s, l_s = ops.uniform_8bit_quantize(accs[0])
+            hops_s = 6
 
-        def d2h_only():
-            for k in range(hops_s):
-                stage.post_send(k, c_s, l_s)
-                stage.take_send(k)
+            def d2h_only():
+                for k in range(hops_s):
+                    stage.post_send(k, c_s, l_s)
+                    stage.take_send(k)
 
-        def h2d_only():
-            for k in range(hops_s):
-                stage.recv_buffers(k)
-                stage.to_device(k)
-                stage.release(k)
+            def h2d_only():
+                for k in range(hops_s):
+                    stage.recv_buffers(k)
+                    stage.to_device(k)
+                    stage.release(k)
 
-        def kernels_only():
-            cc, ll = c_s, l_s
-            for k in range(hops_s):
-                cc, ll = ops.ring_reduce_step(accs[k % 4], cc, ll)
+            def kernels_only():
+                cc, ll = c_s, l_s
+                for k in range(hops_s):
+                    cc, ll = ops.ring_reduce_step(accs[k % 4], cc, ll)
 
-        def staged_hops():
-            # hop k: received message (host) -> device, ring step, result -> host; the transport hands the
-            # sender's slot straight to the receiver (no copy), so what is timed is PCIe and kernels
-            cc, ll = c_s, l_s
-            stage.post_send(0, cc, ll)
-            for k in range(hops_s):
-                lut_h, codes_h = stage.take_send(k)
-                rl, rc = stage.recv_buffers(k)
-                rl.copy_(lut_h)
-                stage.recv_codes[k % stage.depth], stage.send_codes[k % stage.depth] = codes_h, rc     # swap the slots
-                dc, dl = stage.to_device(k)
-                cc, ll = ops.ring_reduce_step(accs[k % 4], dc, dl)
-                stage.release(k)
-                stage.post_send(k + 1, cc, ll)
-            stage.take_send(hops_s)
+            def staged_hops():
+                # hop k: received message (host) -> device, ring step, result -> host; the transport hands the
+                # sender's slot straight to the receiver (no copy), so what is timed is PCIe and kernels
+                cc, ll = c_s, l_s
+                stage.post_send(0, cc, ll)
+                for k in range(hops_s):
+                    lut_h, codes_h = stage.take_send(k)
+                    rl, rc = stage.recv_buffers(k)
+                    rl.copy_(lut_h)
+                    stage.recv_codes[k % stage.depth], stage.send_codes[k % stage.depth] = codes_h, rc     # swap the slots
+                    dc, dl = stage.to_device(k)
+                    cc, ll = ops.ring_reduce_step(accs[k % 4], dc, dl)
+                    stage.release(k)
+                    stage.post_send(k + 1, cc, ll)
+                stage.take_send(hops_s)
 
-        t_d2h = timed(d2h_only, 3, 1) / hops_s
-        t_h2d = timed(h2d_only, 3, 1) / hops_s
-        t_k = timed(kernels_only, 3, 1) / hops_s
-        t_st = timed(staged_hops, 3, 1) / hops_s
-        msg_bytes = n_s + 1024
+            reps_s = 3 if n_s >= (1 << 24) else 10
+            t_d2h = timed(d2h_only, reps_s, 1) / hops_s
+            t_h2d = timed(h2d_only, reps_s, 1) / hops_s
+            t_k = timed(kernels_only, reps_s, 1) / hops_s
+            t_st = timed(staged_hops, reps_s, 1) / hops_s
+            msg_bytes = n_s + 1024
+            return {
+                "message_bytes": msg_bytes, "fp32_chunk_bytes": 4 * n_s,
+                "device_to_host": {"ms": round(t_d2h * 1e3, 3), "GBps": round(msg_bytes / t_d2h / 1e9, 1)},
+                "host_to_device": {"ms": round(t_h2d * 1e3, 3), "GBps": round(msg_bytes / t_h2d / 1e9, 1)},
+                "ring_step_kernels_ms": round(t_k * 1e3, 3),
+                "staged_hop_ms": round(t_st * 1e3, 3),
+            }
+
         out["host_staging"] = {
             "workload": "ring hops on 2^26-element chunks with every message through pinned host buffers "
                         "(device -> host, host -> device on a copy stream); the host-to-host transport itself is not timed",
-            "message_bytes": msg_bytes, "fp32_chunk_bytes": 4 * n_s,
-            "device_to_host": {"ms": round(t_d2h * 1e3, 3), "GBps": round(msg_bytes / t_d2h / 1e9, 1)},
-            "host_to_device": {"ms": round(t_h2d * 1e3, 3), "GBps": round(msg_bytes / t_h2d / 1e9, 1)},
-            "ring_step_kernels_ms": round(t_k * 1e3, 3),
-            "staged_hop_ms": round(t_st * 1e3, 3),
+            **staging_at(RING_CHUNK),
             "note": "a hop is bound by the two PCIe copies of the uint8 codes; staging fp32 would move four times as much",
+            "chunk_of_a_config_2_bucket_at_W8": {"elements": BUCKET_ELEMS // 16, **staging_at(BUCKET_ELEMS // 16)},
         }
-        del accs, stage
 
     if not args.no_cpu_baseline:
         if cpu_inputs is None:           # the t28 leg did not run: one configuration-2 bucket, drawn as the GPU leg draws it
