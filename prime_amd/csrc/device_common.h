@@ -245,8 +245,12 @@ __device__ __forceinline__ void finalize_qparams(double sum, double sumsq, int64
     finalize_from_norm(static_cast<float>(sqrt(sumsq)), sum, sumsq, n, qp);
 }
 
-__device__ __forceinline__ void finalize_from_norm(float norm, double sum, double sumsq, int64_t n, prime_qparams* qp) {
-    const double std_unbiased = static_cast<double>(norm) / sqrt(static_cast<double>(n - 1));
+// sqrt(n - 1) of the scale formula, for a caller that computes it ahead of the sums (the root of an
+// integer-valued double is the same correctly rounded value wherever it is taken).
+__device__ __forceinline__ double root_of_n_minus_1(int64_t n) { return sqrt(static_cast<double>(n - 1)); }
+
+__device__ __forceinline__ void finalize_from_norm_root(float norm, double root_nm1, double sum, double sumsq, int64_t n, prime_qparams* qp) {
+    const double std_unbiased = static_cast<double>(norm) / root_nm1;
     const double scale = 6.0 * std_unbiased / 256.0;
     const float sf = static_cast<float>(scale);
     qp->scale = sf;
@@ -254,6 +258,10 @@ __device__ __forceinline__ void finalize_from_norm(float norm, double sum, doubl
     qp->sum = sum;
     qp->sumsq = sumsq;
     qp->n = n;
+}
+
+__device__ __forceinline__ void finalize_from_norm(float norm, double sum, double sumsq, int64_t n, prime_qparams* qp) {
+    finalize_from_norm_root(norm, root_of_n_minus_1(n), sum, sumsq, n, qp);
 }
 
 // Workgroup reduction of (sum, sumsq) in a fixed order; the workgroup's partial goes to the
@@ -299,34 +307,52 @@ __device__ __forceinline__ float block_scale_reduce(double a, double b, int64_t 
     __shared__ double sh_s[THREADS / 64];
     __shared__ double sh_q[THREADS / 64];
     __shared__ float sh_inv;
-    __shared__ int sh_hot;
+    __shared__ float sh_mean;
+    __shared__ int sh_narrow;
+    // sqrt(n - 1) does not wait for the sums: taken here, ahead of the barrier (the empty statement keeps it here)
+    double root_nm1 = root_of_n_minus_1(n);
+    asm volatile("" : "+v"(root_nm1));
     a = wave_sum(a);
     b = wave_sum(b);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (lane == 0) { sh_s[wave] = a; sh_q[wave] = b; }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    // two chains of fp64 divisions and roots hang on the sums: the scale, and whether the tensor crowds into a few
+    // codes (and which).  The first lanes of two wavefronts take one each, side by side; both add the wavefronts'
+    // sums in the same order.
+    constexpr int kSecond = THREADS > 64 ? 64 : 0;
+    if (threadIdx.x == 0 || threadIdx.x == kSecond) {
         double S = sh_s[0], Q = sh_q[0];
 #pragma unroll
         for (int w = 1; w < THREADS / 64; ++w) { S += sh_s[w]; Q += sh_q[w]; }
-        prime_qparams qp;
-        finalize_qparams(S, Q, n, &qp);
-        sh_inv = qp.inv_scale;
-        sh_hot = narrow_distribution(S, Q, n) ? quantize_code(static_cast<float>(S / static_cast<double>(n)), qp.inv_scale, kZeroPoint) - 1
-                                              : INT_MIN;
-        if (publish) {
-            *rec = qp;
-            if (out) *out = qp;
+        if (threadIdx.x == 0) {
+            prime_qparams qp;
+            finalize_from_norm_root(static_cast<float>(sqrt(Q)), root_nm1, S, Q, n, &qp);
+            sh_inv = qp.inv_scale;
+            if (publish) {
+                *rec = qp;
+                if (out) *out = qp;
+            }
+        }
+        if (threadIdx.x == kSecond) {
+            sh_narrow = narrow_distribution(S, Q, n);
+            sh_mean = static_cast<float>(S / static_cast<double>(n));
         }
     }
     __syncthreads();
-    if (hot_base) *hot_base = sh_hot;
-    return sh_inv;
+    const float inv = sh_inv;
+    if (hot_base) *hot_base = sh_narrow ? quantize_code(sh_mean, inv, kZeroPoint) - 1 : INT_MIN;
+    return inv;
 }
 
-template <int THREADS>
+// `meanwhile()` runs between the issue of the partials' loads and their first use: work of the calling kernel
+// that does not depend on the scale (zeroing its LDS tables) goes there, under the loads' trip to memory.
+struct NothingMeanwhile { __device__ __forceinline__ void operator()() const {} };
+
+template <int THREADS, typename Meanwhile = NothingMeanwhile>
 __device__ __forceinline__ float block_scale_from_partials(const double* part_sum, const double* part_sq, int nparts, int64_t n,
-                                                           bool publish, prime_qparams* rec, prime_qparams* out, int* hot_base = nullptr) {
+                                                           bool publish, prime_qparams* rec, prime_qparams* out, int* hot_base = nullptr,
+                                                           Meanwhile&& meanwhile = Meanwhile{}) {
     constexpr int kIters = (kMaxGrid + THREADS - 1) / THREADS;
     double ps[kIters], pq[kIters];
 #pragma unroll
@@ -335,16 +361,18 @@ __device__ __forceinline__ float block_scale_from_partials(const double* part_su
         ps[k] = i < nparts ? part_sum[i] : 0.0;
         pq[k] = i < nparts ? part_sq[i] : 0.0;
     }
+    meanwhile();
     double a = 0.0, b = 0.0;
 #pragma unroll
     for (int k = 0; k < kIters; ++k) { a += ps[k]; b += pq[k]; }
     return block_scale_reduce<THREADS>(a, b, n, publish, rec, out, hot_base);
 }
 
-template <int THREADS>
+template <int THREADS, typename Meanwhile = NothingMeanwhile>
 __device__ __forceinline__ float block_scale_from_partials(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
-                                                           int* hot_base = nullptr) {
-    return block_scale_from_partials<THREADS>(ws->part_sum, ws->part_sq, nparts, n, blockIdx.x == 0, &ws->qp, out, hot_base);
+                                                           int* hot_base = nullptr, Meanwhile&& meanwhile = Meanwhile{}) {
+    return block_scale_from_partials<THREADS>(ws->part_sum, ws->part_sq, nparts, n, blockIdx.x == 0, &ws->qp, out, hot_base,
+                                              static_cast<Meanwhile&&>(meanwhile));
 }
 
 // Work distribution of the streaming kernels.  The tensor is cut into rows of kThreads
@@ -654,15 +682,55 @@ __device__ __forceinline__ void rhist_far_side(const H& h, int side, unsigned lo
     far_n = 0;
     far_s = 0.0;
 #pragma unroll
-    for (int c = 0; c < kFarCopies; ++c) { far_n += h.far_cnt[side][c]; far_s += h.far_sum[side][c]; }
+    for (int c = 0; c < kFarCopies; ++c) far_n += h.far_cnt[side][c];
+    if (far_n == 0) return;              // the usual case; the sums are all 0.0 then, and so is their total
+#pragma unroll
+    for (int c = 0; c < kFarCopies; ++c) far_s += h.far_sum[side][c];
+}
+
+// The value of the lane D (1 or 2) away within the lane's group of four, by a data-parallel move (no trip
+// through the LDS crossbar).
+template <int D>
+__device__ __forceinline__ unsigned long long quad_xor(unsigned long long v) {
+    static_assert(D == 1 || D == 2, "a neighbour within the quad");
+    constexpr int kCtrl = D == 1 ? 0xB1 : 0x4E;          // quad_perm [1, 0, 3, 2] / [2, 3, 0, 1]
+    const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(v), kCtrl, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(v >> 32), kCtrl, 0xf, 0xf, false);
+    return (static_cast<unsigned long long>(static_cast<unsigned>(hi)) << 32) | static_cast<unsigned>(lo);
 }
 
 // The workgroup's partial: 4 KiB of integer bin totals to `row`, the far elements to `far`.
+// T / kBins neighbouring lanes share a bin: each adds its part of the bin's copies, the lanes are joined by
+// exchanges and the first of them adds what earlier flushes left in the 64-bit accumulators (integers: any
+// order gives the same totals).  One barrier; the slots are left as they are.
 template <int T = kThreads>
 __device__ __forceinline__ void rhist_store(ResidualHist& h, int shift, BinPart* __restrict__ row, const FarSlot far) {
-    rhist_flush<T>(h, shift);
-    for (int b = threadIdx.x; b < kBins; b += T) row[b] = BinPart{h.wide_sum[b], h.wide_cnt[b]};
-    if (threadIdx.x < 2) rhist_far_side(h, threadIdx.x, far.cnt[threadIdx.x * kMaxGrid], far.sum[threadIdx.x * kMaxGrid]);
+    constexpr int kPer = T / kBins;
+    static_assert(kPer == 1 || kPer == 2 || kPer == 4, "one, two or four lanes per bin");
+    __syncthreads();
+    const int b = threadIdx.x / kPer, q = threadIdx.x % kPer;
+    unsigned long long cnt = 0, sum = 0;
+    for (int r = q; r < (1 << shift); r += kPer) {
+        const unsigned long long v = h.slot[(b << shift) + r];
+        cnt += v >> 48;
+        sum += v & 0xffffffffffffull;
+    }
+    if constexpr (kPer >= 4) {
+        cnt += quad_xor<2>(cnt);
+        sum += quad_xor<2>(sum);
+    }
+    if constexpr (kPer >= 2) {
+        cnt += quad_xor<1>(cnt);
+        sum += quad_xor<1>(sum);
+    }
+    if (q == 0) row[b] = BinPart{h.wide_sum[b] + static_cast<long long>(sum) - static_cast<long long>(cnt << 31), h.wide_cnt[b] + cnt};
+    if (threadIdx.x < 2) {
+        unsigned long long far_n;
+        double far_s;
+        rhist_far_side(h, threadIdx.x, far_n, far_s);
+        far.cnt[threadIdx.x * kMaxGrid] = far_n;
+        far.sum[threadIdx.x * kMaxGrid] = far_s;
+    }
 }
 
 // The far elements of side `side` over the partials [p0, p1), by the calling wavefront (all 64 lanes call;

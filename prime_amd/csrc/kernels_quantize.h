@@ -39,6 +39,7 @@ struct HistOut {
     bool first;
     unsigned* tile_counter;     // deals the last part of the tiles on demand (sweep_tiles_dynamic); null: all round-robin
     int dyn_percent;
+    bool cleared = false;       // the caller has zeroed the fixed-point histogram (all copies) ahead of a barrier
 };
 __device__ __forceinline__ HistOut hist_out_of(Workspace* ws, int slot, int dyn_percent) {
     return HistOut{ws ? ws->hist[slot] : nullptr, FarSlot{ws ? &ws->far_sum[0][slot] : nullptr, ws ? &ws->far_cnt[0][slot] : nullptr}, ws ? &ws->hist_info : nullptr, slot == 0,
@@ -72,7 +73,7 @@ __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int6
     const int mode = !HIST ? kPlain : !(__builtin_fabsf(inv) < __builtin_inff()) ? kBin0 : inv != 0.0f ? kFixed : kFp;
     const int shift = narrow != INT_MIN ? 3 : copies_shift;        // 8 = kMaxCopies
     const int copy = threadIdx.x & ((1 << shift) - 1);
-    if (HIST) {
+    if (HIST && !(out_part.cleared && mode == kFixed)) {      // cleared: by the caller, ahead of a barrier
         if (mode == kFixed) rhist_zero(hist.fixed, shift);
         else if (mode == kFp) hist_zero(hist.fp);
         __syncthreads();
@@ -176,12 +177,19 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
     // the scale: given by value, or derived here from the statistics partials of the pass before
     // (stats_parts < 0: the record a preceding kernel left in the workspace)
     int narrow = INT_MIN;                // set when the statistics show a tensor crowded into a few codes
-    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &narrow)
+    __shared__ std::conditional_t<HIST, QuantHist, int> hist_mem;      // no histogram memory without HIST
+    // the histogram is cleared while the statistics partials are on their way (all copies: how many the pass
+    // uses depends on the statistics)
+    auto clear = [&]() {
+        if constexpr (HIST) rhist_zero(reinterpret_cast<QuantHist&>(hist_mem).fixed, 3);
+    };
+    const float inv = stats_parts > 0   ? block_scale_from_partials<kThreads>(ws, stats_parts, n, qp_out, &narrow, clear)
                       : stats_parts < 0 ? ws->qp.inv_scale
                                         : 1.0f / scale_val;
-    __shared__ std::conditional_t<HIST, QuantHist, int> hist_mem;      // no histogram memory without HIST
-    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY, U>(x, n, inv, narrow, zero_point, codes, hist_out_of(HIST ? ws : nullptr, blockIdx.x, dyn_percent),
-                                                       copies_shift, blockIdx.x, gridDim.x, reinterpret_cast<QuantHist&>(hist_mem));
+    HistOut out = hist_out_of(HIST ? ws : nullptr, blockIdx.x, dyn_percent);
+    out.cleared = HIST && stats_parts > 0;
+    quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY, U>(x, n, inv, narrow, zero_point, codes, out, copies_shift, blockIdx.x, gridDim.x,
+                                                       reinterpret_cast<QuantHist&>(hist_mem));
 }
 
 // K2 with the scale given and no histogram (quantize_per_tensor_uint8, compression.cpp:9-43), one
@@ -319,27 +327,44 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
         sh_sum[threadIdx.x] = s;
     }
     __syncthreads();
-    for (int half = kRows / 2; half > 0; half >>= 1) {
-        if (row < half) {
-            const int other = threadIdx.x + half * kLutBinsPerBlock;
-            sh_cnt[threadIdx.x] += sh_cnt[other];
-            if (fixed) {
-                sh_sum[threadIdx.x] = __longlong_as_double(__double_as_longlong(sh_sum[threadIdx.x]) + __double_as_longlong(sh_sum[other]));
-                sh_lo[threadIdx.x] += sh_lo[other];
-            } else {
-                sh_sum[threadIdx.x] += sh_sum[other];
+    // The 256 rows of a bin are added as a binary tree that pairs rows 128 apart first and neighbours last
+    // (row r += row r + h for h = 128, 64, ..., 1).  One barrier: the first wavefront, whose lane (r, bin) holds
+    // row r < 16, adds rows r + 16 w of the other wavefronts from LDS (the steps h = 128 .. 16), then the lanes
+    // are joined by exchanges at distances 32, 16, 8 and 4 (h = 8 .. 1); the operands of every addition are the
+    // ones the step-by-step tree would add, so fp64 partials give the same bits.
+    if (threadIdx.x < 64) {
+        unsigned long long cw[16], lw[16];
+        double sw[16];
+#pragma unroll
+        for (int w = 0; w < 16; ++w) {
+            cw[w] = sh_cnt[threadIdx.x + 64 * w];
+            sw[w] = sh_sum[threadIdx.x + 64 * w];
+            lw[w] = fixed ? sh_lo[threadIdx.x + 64 * w] : 0ull;
+        }
+#pragma unroll
+        for (int h = 8; h > 0; h >>= 1) {
+#pragma unroll
+            for (int i = 0; i < h; ++i) {
+                cw[i] += cw[i + h];
+                lw[i] += lw[i + h];
+                sw[i] = fixed ? __longlong_as_double(__double_as_longlong(sw[i]) + __double_as_longlong(sw[i + h])) : sw[i] + sw[i + h];
             }
         }
-        __syncthreads();
-    }
-    if (row == 0 && bin < n_bins) {
-        const unsigned long long cc = sh_cnt[threadIdx.x];
-        const bool far_bin = bin == 0 || bin == kBins - 1;
-        const double sum = fixed ? fixed_bin_sum(cc, __double_as_longlong(sh_sum[threadIdx.x]), sh_lo[threadIdx.x], far_bin ? sh_far_n : 0ull,
-                                                 far_bin ? sh_far_s : 0.0, info.inv, bin)
-                                 : sh_sum[threadIdx.x];
-        lut[bin] = mean_entry(sum, cc);
-        if (counts) counts[bin] = cc;
+        unsigned long long cc = cw[0], lo = lw[0];
+        double sum = sw[0];
+#pragma unroll
+        for (int d = 32; d >= kLutBinsPerBlock; d >>= 1) {
+            cc += __shfl_xor(cc, d, 64);
+            lo += __shfl_xor(lo, d, 64);
+            const double other = __shfl_xor(sum, d, 64);
+            sum = fixed ? __longlong_as_double(__double_as_longlong(sum) + __double_as_longlong(other)) : sum + other;
+        }
+        if (row == 0 && bin < n_bins) {
+            const bool far_bin = bin == 0 || bin == kBins - 1;
+            if (fixed) sum = fixed_bin_sum(cc, __double_as_longlong(sum), lo, far_bin ? sh_far_n : 0ull, far_bin ? sh_far_s : 0.0, info.inv, bin);
+            lut[bin] = mean_entry(sum, cc);
+            if (counts) counts[bin] = cc;
+        }
     }
     if (blockIdx.x == 0)
         for (int64_t b = kBins + threadIdx.x; b < n_bins; b += kFinalThreads) lut[b] = 0.0f;

@@ -92,8 +92,8 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void seg_quantize_kernel(c
     const int64_t n = job.n[t];
     int narrow = INT_MIN;
     const float inv = block_scale_from_partials<kThreads>(ws->seg_part_sum[t], ws->seg_part_sq[t], job.parts[t], n, p == 0, &ws->seg[t].qp,
-                                                          qp_out ? qp_out + t : nullptr, &narrow);
-    const HistOut out{ws->hist[blockIdx.x], FarSlot{&ws->far_sum[0][blockIdx.x], &ws->far_cnt[0][blockIdx.x]}, &ws->seg[t].info, p == 0, nullptr, 0};
+                                                          qp_out ? qp_out + t : nullptr, &narrow, [&]() { rhist_zero(hist_mem.fixed, 3); });
+    const HistOut out{ws->hist[blockIdx.x], FarSlot{&ws->far_sum[0][blockIdx.x], &ws->far_cnt[0][blockIdx.x]}, &ws->seg[t].info, p == 0, nullptr, 0, true};
     if ((job.two_row >> t) & 1)
         quantize_block<true, true, true, true, POLICY, 2>(job.x[t], n, inv, narrow, kZeroPoint, job.codes[t], out, copies_shift, p, P, hist_mem);
     else
