@@ -688,6 +688,22 @@ __device__ __forceinline__ void rhist_far_side(const H& h, int side, unsigned lo
     for (int c = 0; c < kFarCopies; ++c) far_s += h.far_sum[side][c];
 }
 
+// The sum of v over the sixteen lanes of the wavefront that share the lane's index modulo 4, in every lane:
+// two rotations within the rows of sixteen lanes (data-parallel moves), two exchanges between the rows.
+__device__ __forceinline__ unsigned long long sum_lanes_mod4(unsigned long long v) {
+    auto rotated = [](unsigned long long x, auto ctrl_t) {
+        constexpr int kCtrl = decltype(ctrl_t)::value;
+        const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(x), kCtrl, 0xf, 0xf, false);
+        const int hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(x >> 32), kCtrl, 0xf, 0xf, false);
+        return (static_cast<unsigned long long>(static_cast<unsigned>(hi)) << 32) | static_cast<unsigned>(lo);
+    };
+    v += rotated(v, std::integral_constant<int, 0x128>{});      // row_ror:8
+    v += rotated(v, std::integral_constant<int, 0x124>{});      // row_ror:4
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
 // The value of the lane D (1 or 2) away within the lane's group of four, by a data-parallel move (no trip
 // through the LDS crossbar).
 template <int D>
@@ -751,6 +767,11 @@ __device__ __forceinline__ void far_totals(const Workspace* __restrict__ ws, int
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) { fs += s[k]; fn += c[k]; }
+    }
+    if (__ballot(fn != 0) == 0) {        // the usual case: no far element anywhere; the sums are all 0.0 then
+        far_s = 0.0;
+        far_n = 0;
+        return;
     }
     far_s = wave_sum(fs);
 #pragma unroll

@@ -308,8 +308,10 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
     unsigned long long c = 0;
 #pragma unroll
     for (int k = 0; k < kIters; ++k) c += part[k].cnt;
-    sh_cnt[threadIdx.x] = c;
     if (fixed) {
+        // Integer partials: any order of addition gives the same totals.  Every wavefront adds its 16 rows of
+        // each bin by exchanges between lanes, the 16 wavefronts' totals meet in LDS (one barrier) and the
+        // first wavefront adds them the same way.
         long long hi = 0;
         unsigned long long lo = 0;
 #pragma unroll
@@ -318,52 +320,65 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
             hi += units_hi(u);
             lo += units_lo(u);
         }
-        sh_sum[threadIdx.x] = __longlong_as_double(hi);
-        sh_lo[threadIdx.x] = lo;
+        c = sum_lanes_mod4(c);
+        lo = sum_lanes_mod4(lo);
+        hi = static_cast<long long>(sum_lanes_mod4(static_cast<unsigned long long>(hi)));
+        if ((threadIdx.x & 63) < kLutBinsPerBlock) {
+            const int slot = (threadIdx.x >> 6) * kLutBinsPerBlock + bl;
+            sh_cnt[slot] = c;
+            sh_lo[slot] = lo;
+            sh_sum[slot] = __longlong_as_double(hi);
+        }
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            const unsigned long long cc = sum_lanes_mod4(sh_cnt[threadIdx.x]);
+            const unsigned long long ll = sum_lanes_mod4(sh_lo[threadIdx.x]);
+            const long long hh = static_cast<long long>(sum_lanes_mod4(static_cast<unsigned long long>(__double_as_longlong(sh_sum[threadIdx.x]))));
+            if (row == 0 && bin < n_bins) {
+                const bool far_bin = bin == 0 || bin == kBins - 1;
+                lut[bin] = mean_entry(fixed_bin_sum(cc, hh, ll, far_bin ? sh_far_n : 0ull, far_bin ? sh_far_s : 0.0, info.inv, bin), cc);
+                if (counts) counts[bin] = cc;
+            }
+        }
     } else {
+        // fp64 partials (rare: a zero or non-finite 1 / scale, or codes given by the caller): the 256 rows of a
+        // bin are added as a binary tree that pairs rows 128 apart first and neighbours last (row r += row r + h
+        // for h = 128, 64, ..., 1), a fixed order.  One barrier: the first wavefront, whose lane (r, bin) holds
+        // row r < 16, adds rows r + 16 w of the other wavefronts from LDS (the steps h = 128 .. 16), then the
+        // lanes are joined by exchanges at distances 32, 16, 8 and 4 (h = 8 .. 1).
         double s = 0.0;
 #pragma unroll
         for (int k = 0; k < kIters; ++k) s += part[k].sum;
+        sh_cnt[threadIdx.x] = c;
         sh_sum[threadIdx.x] = s;
-    }
-    __syncthreads();
-    // The 256 rows of a bin are added as a binary tree that pairs rows 128 apart first and neighbours last
-    // (row r += row r + h for h = 128, 64, ..., 1).  One barrier: the first wavefront, whose lane (r, bin) holds
-    // row r < 16, adds rows r + 16 w of the other wavefronts from LDS (the steps h = 128 .. 16), then the lanes
-    // are joined by exchanges at distances 32, 16, 8 and 4 (h = 8 .. 1); the operands of every addition are the
-    // ones the step-by-step tree would add, so fp64 partials give the same bits.
-    if (threadIdx.x < 64) {
-        unsigned long long cw[16], lw[16];
-        double sw[16];
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            unsigned long long cw[16];
+            double sw[16];
 #pragma unroll
-        for (int w = 0; w < 16; ++w) {
-            cw[w] = sh_cnt[threadIdx.x + 64 * w];
-            sw[w] = sh_sum[threadIdx.x + 64 * w];
-            lw[w] = fixed ? sh_lo[threadIdx.x + 64 * w] : 0ull;
-        }
-#pragma unroll
-        for (int h = 8; h > 0; h >>= 1) {
-#pragma unroll
-            for (int i = 0; i < h; ++i) {
-                cw[i] += cw[i + h];
-                lw[i] += lw[i + h];
-                sw[i] = fixed ? __longlong_as_double(__double_as_longlong(sw[i]) + __double_as_longlong(sw[i + h])) : sw[i] + sw[i + h];
+            for (int w = 0; w < 16; ++w) {
+                cw[w] = sh_cnt[threadIdx.x + 64 * w];
+                sw[w] = sh_sum[threadIdx.x + 64 * w];
             }
-        }
-        unsigned long long cc = cw[0], lo = lw[0];
-        double sum = sw[0];
 #pragma unroll
-        for (int d = 32; d >= kLutBinsPerBlock; d >>= 1) {
-            cc += __shfl_xor(cc, d, 64);
-            lo += __shfl_xor(lo, d, 64);
-            const double other = __shfl_xor(sum, d, 64);
-            sum = fixed ? __longlong_as_double(__double_as_longlong(sum) + __double_as_longlong(other)) : sum + other;
-        }
-        if (row == 0 && bin < n_bins) {
-            const bool far_bin = bin == 0 || bin == kBins - 1;
-            if (fixed) sum = fixed_bin_sum(cc, __double_as_longlong(sum), lo, far_bin ? sh_far_n : 0ull, far_bin ? sh_far_s : 0.0, info.inv, bin);
-            lut[bin] = mean_entry(sum, cc);
-            if (counts) counts[bin] = cc;
+            for (int h = 8; h > 0; h >>= 1) {
+#pragma unroll
+                for (int i = 0; i < h; ++i) {
+                    cw[i] += cw[i + h];
+                    sw[i] += sw[i + h];
+                }
+            }
+            unsigned long long cc = cw[0];
+            double sum = sw[0];
+#pragma unroll
+            for (int d = 32; d >= kLutBinsPerBlock; d >>= 1) {
+                cc += __shfl_xor(cc, d, 64);
+                sum += __shfl_xor(sum, d, 64);
+            }
+            if (row == 0 && bin < n_bins) {
+                lut[bin] = mean_entry(sum, cc);
+                if (counts) counts[bin] = cc;
+            }
         }
     }
     if (blockIdx.x == 0)
