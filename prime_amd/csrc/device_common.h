@@ -688,9 +688,9 @@ __device__ __forceinline__ void rhist_far_side(const H& h, int side, unsigned lo
     for (int c = 0; c < kFarCopies; ++c) far_s += h.far_sum[side][c];
 }
 
-// The sum of v over the sixteen lanes of the wavefront that share the lane's index modulo 4, in every lane:
-// two rotations within the rows of sixteen lanes (data-parallel moves), two exchanges between the rows.
-__device__ __forceinline__ unsigned long long sum_lanes_mod4(unsigned long long v) {
+// The sum of v over the four lanes of the lane's row of sixteen that share its index modulo 4, in every lane:
+// two rotations within the row (data-parallel moves).
+__device__ __forceinline__ unsigned long long sum_row_mod4(unsigned long long v) {
     auto rotated = [](unsigned long long x, auto ctrl_t) {
         constexpr int kCtrl = decltype(ctrl_t)::value;
         const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(x), kCtrl, 0xf, 0xf, false);
@@ -699,6 +699,12 @@ __device__ __forceinline__ unsigned long long sum_lanes_mod4(unsigned long long 
     };
     v += rotated(v, std::integral_constant<int, 0x128>{});      // row_ror:8
     v += rotated(v, std::integral_constant<int, 0x124>{});      // row_ror:4
+    return v;
+}
+
+// The same over the sixteen such lanes of the whole wavefront: then two exchanges between the rows.
+__device__ __forceinline__ unsigned long long sum_lanes_mod4(unsigned long long v) {
+    v = sum_row_mod4(v);
     v += __shfl_xor(v, 16, 64);
     v += __shfl_xor(v, 32, 64);
     return v;

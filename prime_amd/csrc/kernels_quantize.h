@@ -270,24 +270,32 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const flo
 }
 
 // Second stage of the lookup build.  Workgroup j owns bins 4j .. 4j+3 (64 contiguous bytes
-// of every partial): lane (row, bin) adds partials row, row + 256, ... in order, the 256
-// rows are then added by a tree of fixed shape.  Mean = fp64 sum / count rounded to float
-// once; an empty bin gives 0.0f (compression.cpp:100).  Entries >= 256 of a longer table
-// are 0.0f.  Fixed-point partials (BinPart) are added as integers, the far elements of the two
-// clip bins beside them, and converted once (fixed_bin_sum).
-__global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Workspace* __restrict__ ws, int nparts,
-                                                                      float* __restrict__ lut, int64_t n_bins,
-                                                                      unsigned long long* __restrict__ counts) {
-    constexpr int kRows = kFinalThreads / kLutBinsPerBlock;
-    __shared__ double sh_sum[kFinalThreads];                 // fixed-point partials: the upper halves' total, as an integer
-    __shared__ unsigned long long sh_lo[kFinalThreads];
-    __shared__ unsigned long long sh_cnt[kFinalThreads];
+// of every partial): lane (row, bin) adds partials row, row + THREADS / 4, ... and the rows are
+// then added up.  Mean = fp64 sum / count rounded to float once; an empty bin gives 0.0f
+// (compression.cpp:100).  Entries >= 256 of a longer table are 0.0f.  Fixed-point partials
+// (BinPart) are added as integers, the far elements of the two clip bins beside them, and
+// converted once (fixed_bin_sum).
+// Two shapes: 1024 lanes for up to kMaxGrid partials, 256 lanes for up to 256 (every launch of
+// the default options): with four wavefronts instead of sixteen, each on a SIMD of its own, the
+// chain from the partials' arrival to the table is shorter.  fp64 partials are added in one
+// order in both: as a binary tree over 256 rows that pairs rows 128 apart first and neighbours
+// last (row r += row r + h for h = 128, 64, ..., 1), row r being the sum of partials r, r + 256, ...
+template <int THREADS, int MAXPARTS>
+__global__ __launch_bounds__(THREADS) void lut_finalize_kernel(const Workspace* __restrict__ ws, int nparts,
+                                                                float* __restrict__ lut, int64_t n_bins,
+                                                                unsigned long long* __restrict__ counts) {
+    constexpr int kRows = THREADS / kLutBinsPerBlock;
+    constexpr int kWavesHere = THREADS / 64;
+    constexpr int kIters = MAXPARTS / kRows;
+    static_assert((THREADS == 1024 && MAXPARTS == kMaxGrid) || (THREADS == 256 && MAXPARTS == 256), "the two shapes");
+    __shared__ double sh_sum[THREADS];                       // fixed-point partials: the upper halves' total, as an integer
+    __shared__ unsigned long long sh_lo[THREADS];
+    __shared__ unsigned long long sh_cnt[THREADS];
     __shared__ double sh_far_s;
     __shared__ unsigned long long sh_far_n;
     const int bl = threadIdx.x % kLutBinsPerBlock;
     const int row = threadIdx.x / kLutBinsPerBlock;
     const int bin = blockIdx.x * kLutBinsPerBlock + bl;
-    constexpr int kIters = kMaxGrid / kRows;
     const HistInfo info = ws->hist_info;        // first of the loads: it is back when the partials are
     BinAcc part[kIters];
 #pragma unroll
@@ -298,20 +306,20 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
     // the far elements of bin 0 / 255 (fixed-point partials only; harmless to read otherwise): the last wavefront
     // of the workgroup that owns the bin adds them up, its loads in flight with everybody's
     const bool clip_block = blockIdx.x == 0 || blockIdx.x == kBins / kLutBinsPerBlock - 1;
-    if (clip_block && threadIdx.x >= kFinalThreads - 64) {
+    if (clip_block && threadIdx.x >= THREADS - 64) {
         double fs;
         unsigned long long fn;
         far_totals(ws, 0, nparts, blockIdx.x != 0, fs, fn);
-        if (threadIdx.x == kFinalThreads - 64) { sh_far_s = fs; sh_far_n = fn; }
+        if (threadIdx.x == THREADS - 64) { sh_far_s = fs; sh_far_n = fn; }
     }
     const bool fixed = info.mode == kHistFixed;
     unsigned long long c = 0;
 #pragma unroll
     for (int k = 0; k < kIters; ++k) c += part[k].cnt;
     if (fixed) {
-        // Integer partials: any order of addition gives the same totals.  Every wavefront adds its 16 rows of
-        // each bin by exchanges between lanes, the 16 wavefronts' totals meet in LDS (one barrier) and the
-        // first wavefront adds them the same way.
+        // Integer partials: any order of addition gives the same totals.  Every wavefront adds the four rows
+        // that share a row of sixteen lanes by data-parallel moves and leaves 16 totals (4 per bin) in LDS; one
+        // barrier; the first wavefront adds them.
         long long hi = 0;
         unsigned long long lo = 0;
 #pragma unroll
@@ -320,20 +328,28 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
             hi += units_hi(u);
             lo += units_lo(u);
         }
-        c = sum_lanes_mod4(c);
-        lo = sum_lanes_mod4(lo);
-        hi = static_cast<long long>(sum_lanes_mod4(static_cast<unsigned long long>(hi)));
-        if ((threadIdx.x & 63) < kLutBinsPerBlock) {
-            const int slot = (threadIdx.x >> 6) * kLutBinsPerBlock + bl;
+        c = sum_row_mod4(c);
+        lo = sum_row_mod4(lo);
+        hi = static_cast<long long>(sum_row_mod4(static_cast<unsigned long long>(hi)));
+        if ((threadIdx.x & 15) < kLutBinsPerBlock) {
+            const int slot = (threadIdx.x >> 4) * kLutBinsPerBlock + bl;      // (wavefront, row of lanes, bin)
             sh_cnt[slot] = c;
             sh_lo[slot] = lo;
             sh_sum[slot] = __longlong_as_double(hi);
         }
         __syncthreads();
         if (threadIdx.x < 64) {
-            const unsigned long long cc = sum_lanes_mod4(sh_cnt[threadIdx.x]);
-            const unsigned long long ll = sum_lanes_mod4(sh_lo[threadIdx.x]);
-            const long long hh = static_cast<long long>(sum_lanes_mod4(static_cast<unsigned long long>(__double_as_longlong(sh_sum[threadIdx.x]))));
+            unsigned long long cc = 0, ll = 0;
+            long long hh = 0;
+#pragma unroll
+            for (int k = 0; k < kWavesHere / 4; ++k) {        // kWavesHere * 16 slots, 64 per step; slot % 4 is the lane's bin
+                cc += sh_cnt[threadIdx.x + 64 * k];
+                ll += sh_lo[threadIdx.x + 64 * k];
+                hh += __double_as_longlong(sh_sum[threadIdx.x + 64 * k]);
+            }
+            cc = sum_lanes_mod4(cc);
+            ll = sum_lanes_mod4(ll);
+            hh = static_cast<long long>(sum_lanes_mod4(static_cast<unsigned long long>(hh)));
             if (row == 0 && bin < n_bins) {
                 const bool far_bin = bin == 0 || bin == kBins - 1;
                 lut[bin] = mean_entry(fixed_bin_sum(cc, hh, ll, far_bin ? sh_far_n : 0ull, far_bin ? sh_far_s : 0.0, info.inv, bin), cc);
@@ -341,27 +357,32 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
             }
         }
     } else {
-        // fp64 partials (rare: a zero or non-finite 1 / scale, or codes given by the caller): the 256 rows of a
-        // bin are added as a binary tree that pairs rows 128 apart first and neighbours last (row r += row r + h
-        // for h = 128, 64, ..., 1), a fixed order.  One barrier: the first wavefront, whose lane (r, bin) holds
-        // row r < 16, adds rows r + 16 w of the other wavefronts from LDS (the steps h = 128 .. 16), then the
-        // lanes are joined by exchanges at distances 32, 16, 8 and 4 (h = 8 .. 1).
-        double s = 0.0;
+        // fp64 partials (rare: a zero or non-finite 1 / scale, or codes given by the caller), the fixed tree.
+        // One barrier: the first wavefront, whose lane (r, bin) holds row r < 16, adds the rows r + 16 w of the
+        // other wavefronts from LDS (the steps down to h = 16), then the lanes are joined by exchanges at
+        // distances 32, 16, 8 and 4 (h = 8 .. 1).
+        double s;
+        if constexpr (THREADS == 1024) {
+            s = 0.0;
 #pragma unroll
-        for (int k = 0; k < kIters; ++k) s += part[k].sum;
+            for (int k = 0; k < kIters; ++k) s += part[k].sum;
+        } else {
+            // row r of the tree is partial r alone here; this lane holds rows row, row + 64, row + 128, row + 192
+            s = (part[0].sum + part[2].sum) + (part[1].sum + part[3].sum);      // h = 128, then h = 64
+        }
         sh_cnt[threadIdx.x] = c;
         sh_sum[threadIdx.x] = s;
         __syncthreads();
         if (threadIdx.x < 64) {
-            unsigned long long cw[16];
-            double sw[16];
+            unsigned long long cw[kWavesHere];
+            double sw[kWavesHere];
 #pragma unroll
-            for (int w = 0; w < 16; ++w) {
+            for (int w = 0; w < kWavesHere; ++w) {
                 cw[w] = sh_cnt[threadIdx.x + 64 * w];
                 sw[w] = sh_sum[threadIdx.x + 64 * w];
             }
 #pragma unroll
-            for (int h = 8; h > 0; h >>= 1) {
+            for (int h = kWavesHere / 2; h > 0; h >>= 1) {
 #pragma unroll
                 for (int i = 0; i < h; ++i) {
                     cw[i] += cw[i + h];
@@ -382,7 +403,7 @@ __global__ __launch_bounds__(kFinalThreads) void lut_finalize_kernel(const Works
         }
     }
     if (blockIdx.x == 0)
-        for (int64_t b = kBins + threadIdx.x; b < n_bins; b += kFinalThreads) lut[b] = 0.0f;
+        for (int64_t b = kBins + threadIdx.x; b < n_bins; b += THREADS) lut[b] = 0.0f;
 }
 
 __global__ void lut_zero_kernel(float* __restrict__ lut, int64_t n_bins, unsigned long long* __restrict__ counts) {

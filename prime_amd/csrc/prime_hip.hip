@@ -293,8 +293,12 @@ int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins
         launch(kIdLutFinalize, 0.0, lut_zero_kernel, 1, 256, st, lut, n_bins, reinterpret_cast<unsigned long long*>(counts));
         return launch_check("lut_zero_kernel");
     }
-    launch(kIdLutFinalize, 16.0 * kBins * nparts, lut_finalize_kernel, kBins / kLutBinsPerBlock, kFinalThreads, st, ws, nparts, lut,
-           n_bins, reinterpret_cast<unsigned long long*>(counts));
+    if (nparts <= 256)
+        launch(kIdLutFinalize, 16.0 * kBins * nparts, lut_finalize_kernel<256, 256>, kBins / kLutBinsPerBlock, 256, st, ws, nparts, lut, n_bins,
+               reinterpret_cast<unsigned long long*>(counts));
+    else
+        launch(kIdLutFinalize, 16.0 * kBins * nparts, lut_finalize_kernel<kFinalThreads, kMaxGrid>, kBins / kLutBinsPerBlock, kFinalThreads, st, ws,
+               nparts, lut, n_bins, reinterpret_cast<unsigned long long*>(counts));
     return launch_check("lut_finalize_kernel");
 }
 
