@@ -100,31 +100,37 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void seg_quantize_kernel(c
         quantize_block<true, true, true, true, POLICY, kUnroll>(job.x[t], n, inv, narrow, kZeroPoint, job.codes[t], out, copies_shift, p, P, hist_mem);
 }
 
-// The lookup tables of the job: one workgroup per tensor.  Lane (g, b) adds bin b of every fourth of
-// the tensor's partials (rows first[t] .. first[t + 1] of the quantize launch), several loads in
-// flight; the four groups are joined in LDS and the total converted once.
-constexpr int kSegFinalGroups = kFinalThreads / kBins;
-__global__ __launch_bounds__(kFinalThreads) void seg_lut_finalize_kernel(const SegJob job, const Workspace* __restrict__ ws, float* __restrict__ luts) {
-    __shared__ double sh_sum[kSegFinalGroups][kBins];            // fixed-point partials: the upper halves' total, as an integer
-    __shared__ unsigned long long sh_lo[kSegFinalGroups][kBins];
-    __shared__ unsigned long long sh_cnt[kSegFinalGroups][kBins];
-    __shared__ double sh_far_s[2];
-    __shared__ unsigned long long sh_far_n[2];
-    const int t = blockIdx.x;
-    const int b = threadIdx.x & (kBins - 1), g = threadIdx.x / kBins;
+// The lookup tables of the job: 64 workgroups of 256 lanes per tensor, each owning four bins, as in
+// lut_finalize_kernel; the tensor's partials are rows first[t] .. first[t + 1] of the quantize launch.
+// Lane (row, bin) adds partials row, row + 64, ... (four loads in flight); fp64 partials in that order,
+// then over the rows by a fixed tree.
+constexpr int kSegFinalThreads = 256;
+constexpr int kSegFinalBlocks = kBins / kLutBinsPerBlock;          // workgroups per tensor
+__global__ __launch_bounds__(kSegFinalThreads) void seg_lut_finalize_kernel(const SegJob job, const Workspace* __restrict__ ws, float* __restrict__ luts) {
+    constexpr int kRows = kSegFinalThreads / kLutBinsPerBlock;      // 64
+    constexpr int kWavesHere = kSegFinalThreads / 64;
+    constexpr int kInFlight = 4;
+    __shared__ double sh_sum[kSegFinalThreads];
+    __shared__ unsigned long long sh_lo[kSegFinalThreads];
+    __shared__ unsigned long long sh_cnt[kSegFinalThreads];
+    __shared__ double sh_far_s;
+    __shared__ unsigned long long sh_far_n;
+    const int t = blockIdx.x / kSegFinalBlocks, j = blockIdx.x % kSegFinalBlocks;
+    const int bl = threadIdx.x % kLutBinsPerBlock, row = threadIdx.x / kLutBinsPerBlock;
+    const int bin = j * kLutBinsPerBlock + bl;
     const int p0 = job.first[t], p1 = job.first[t + 1];
+    const HistInfo info = ws->seg[t].info;
     unsigned long long cnt = 0, lo = 0;
     long long hi = 0;
     double sum = 0.0;
-    constexpr int kInFlight = 8;
-    // both readings of a partial are added up (the integer one and the fp64 one); the record that says which
-    // one holds arrives with the first partials instead of ahead of them
-    for (int q0 = p0 + g; q0 < p1; q0 += kSegFinalGroups * kInFlight) {
+    // both readings of a partial are added up (the integer one and the fp64 one): which one holds is known
+    // when the record has arrived, with the first partials
+    for (int q0 = p0 + row; q0 < p1; q0 += kRows * kInFlight) {
         BinAcc e[kInFlight];
 #pragma unroll
         for (int k = 0; k < kInFlight; ++k) {
-            const int p = q0 + k * kSegFinalGroups;
-            e[k] = p < p1 ? ws->hist[p][b] : BinAcc{0.0, 0ull};
+            const int p = q0 + k * kRows;
+            e[k] = p < p1 ? ws->hist[p][bin] : BinAcc{0.0, 0ull};
         }
 #pragma unroll
         for (int k = 0; k < kInFlight; ++k) {
@@ -135,34 +141,66 @@ __global__ __launch_bounds__(kFinalThreads) void seg_lut_finalize_kernel(const S
             sum += e[k].sum;
         }
     }
-    // the far elements of bins 0 and 255: the last two wavefronts, one side each
-    if (threadIdx.x >= kFinalThreads - 128) {
-        const int side = threadIdx.x >= kFinalThreads - 64;
+    // the far elements of bins 0 and 255: the last wavefront of the workgroup that owns the bin
+    const bool clip_block = j == 0 || j == kSegFinalBlocks - 1;
+    if (clip_block && threadIdx.x >= kSegFinalThreads - 64) {
         double fs;
         unsigned long long fn;
-        far_totals(ws, p0, p1, side, fs, fn);
-        if ((threadIdx.x & 63) == 0) { sh_far_s[side] = fs; sh_far_n[side] = fn; }
+        far_totals(ws, p0, p1, j != 0, fs, fn);
+        if (threadIdx.x == kSegFinalThreads - 64) { sh_far_s = fs; sh_far_n = fn; }
     }
-    const HistInfo info = ws->seg[t].info;
     const bool fixed = info.mode == kHistFixed;
-    sh_cnt[g][b] = cnt;
-    sh_lo[g][b] = lo;
-    sh_sum[g][b] = fixed ? __longlong_as_double(hi) : sum;
-    __syncthreads();
-    if (g == 0) {
-#pragma unroll
-        for (int k = 1; k < kSegFinalGroups; ++k) {
-            cnt += sh_cnt[k][b];
-            if (fixed) {
-                hi += __double_as_longlong(sh_sum[k][b]);
-                lo += sh_lo[k][b];
-            } else {
-                sum += sh_sum[k][b];
+    float* lut = luts + static_cast<int64_t>(t) * kBins;
+    if (fixed) {
+        cnt = sum_row_mod4(cnt);
+        lo = sum_row_mod4(lo);
+        hi = static_cast<long long>(sum_row_mod4(static_cast<unsigned long long>(hi)));
+        if ((threadIdx.x & 15) < kLutBinsPerBlock) {
+            const int slot = (threadIdx.x >> 4) * kLutBinsPerBlock + bl;
+            sh_cnt[slot] = cnt;
+            sh_lo[slot] = lo;
+            sh_sum[slot] = __longlong_as_double(hi);
+        }
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            static_assert(kWavesHere * 16 == 64, "one slot per lane of the first wavefront");
+            const unsigned long long cc = sum_lanes_mod4(sh_cnt[threadIdx.x]);
+            const unsigned long long ll = sum_lanes_mod4(sh_lo[threadIdx.x]);
+            const long long hh = static_cast<long long>(sum_lanes_mod4(static_cast<unsigned long long>(__double_as_longlong(sh_sum[threadIdx.x]))));
+            if (row == 0) {
+                const bool far_bin = bin == 0 || bin == kBins - 1;
+                lut[bin] = mean_entry(fixed_bin_sum(cc, hh, ll, far_bin ? sh_far_n : 0ull, far_bin ? sh_far_s : 0.0, info.inv, bin), cc);
             }
         }
-        const bool far_bin = b == 0 || b == kBins - 1;
-        if (fixed) sum = fixed_bin_sum(cnt, hi, lo, far_bin ? sh_far_n[b != 0] : 0ull, far_bin ? sh_far_s[b != 0] : 0.0, info.inv, b);
-        luts[static_cast<int64_t>(t) * kBins + b] = mean_entry(sum, cnt);
+    } else {
+        sh_cnt[threadIdx.x] = cnt;
+        sh_sum[threadIdx.x] = sum;
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            unsigned long long cw[kWavesHere];
+            double sw[kWavesHere];
+#pragma unroll
+            for (int w = 0; w < kWavesHere; ++w) {
+                cw[w] = sh_cnt[threadIdx.x + 64 * w];
+                sw[w] = sh_sum[threadIdx.x + 64 * w];
+            }
+#pragma unroll
+            for (int h = kWavesHere / 2; h > 0; h >>= 1) {
+#pragma unroll
+                for (int i = 0; i < h; ++i) {
+                    cw[i] += cw[i + h];
+                    sw[i] += sw[i + h];
+                }
+            }
+            unsigned long long cc = cw[0];
+            double s = sw[0];
+#pragma unroll
+            for (int d = 32; d >= kLutBinsPerBlock; d >>= 1) {
+                cc += __shfl_xor(cc, d, 64);
+                s += __shfl_xor(s, d, 64);
+            }
+            if (row == 0) lut[bin] = mean_entry(s, cc);
+        }
     }
 }
 

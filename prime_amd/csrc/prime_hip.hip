@@ -879,7 +879,7 @@ int run_segment_group(SegKind kind, int count, float* const* xs, const int64_t* 
     while ((1 << (shift + 1)) <= g_opt.hist_replicas) ++shift;
     launch(kIdSegQuantize, bytes_q, seg_quantize_kernel<kStoreNt>, first, kThreads, st, job, qps, w, shift);
     if (int rc = launch_check("seg_quantize_kernel")) return rc;
-    launch(kIdSegLutFinalize, 16.0 * kBins * first, seg_lut_finalize_kernel, count, kFinalThreads, st, job, w, luts);
+    launch(kIdSegLutFinalize, 16.0 * kBins * first, seg_lut_finalize_kernel, count * kSegFinalBlocks, kSegFinalThreads, st, job, w, luts);
     return launch_check("seg_lut_finalize_kernel");
 }
 
