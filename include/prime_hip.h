@@ -62,7 +62,8 @@ const char* prime_hip_last_error(void);
  * 1024 elements instead of two on tensors of at most this many Mi elements; 0: never),
  * "dynamic_tail_percent" / "dynamic_tail_min_mi_elems" (the fused quantize + lookup pass hands out this
  * share of its tiles, the last ones, on demand instead of round-robin, on tensors of at least that many
- * Mi elements; 0: never), "segment_blocks_per_cu" (workgroups per compute unit that the quantize pass of
+ * Mi elements; 0: never; the counter it deals them through lives in the workspace and is left at zero by
+ * prime_workspace_init and by every call that uses it), "segment_blocks_per_cu" (workgroups per compute unit that the quantize pass of
  * a segmented launch shares out among its tensors), "grid_cap" (upper bound on the workgroups of a looping kernel, for
  * experiments; 0: none).
  * Cache policies, load hints, the one-workgroup-per-tile and one-launch variants, the number of LDS

@@ -281,9 +281,12 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void hist_kernel(const flo
 // order in both: as a binary tree over 256 rows that pairs rows 128 apart first and neighbours
 // last (row r += row r + h for h = 128, 64, ..., 1), row r being the sum of partials r, r + 256, ...
 template <int THREADS, int MAXPARTS>
-__global__ __launch_bounds__(THREADS) void lut_finalize_kernel(const Workspace* __restrict__ ws, int nparts,
+__global__ __launch_bounds__(THREADS) void lut_finalize_kernel(Workspace* __restrict__ ws, int nparts,
                                                                 float* __restrict__ lut, int64_t n_bins,
                                                                 unsigned long long* __restrict__ counts) {
+    // the fused pass of this call may have dealt tiles through the workspace's counter: left at zero for the next
+    // call's (the passes that write statistics partials reset it as well)
+    if (blockIdx.x == 0 && threadIdx.x == 0) ws->tile_counter = 0u;
     constexpr int kRows = THREADS / kLutBinsPerBlock;
     constexpr int kWavesHere = THREADS / 64;
     constexpr int kIters = MAXPARTS / kRows;

@@ -234,9 +234,9 @@ void launch_quantize_p(bool al, bool two, int grid, hipStream_t st, const float*
     const int id = HIST ? kIdQuantizeHist : kIdQuantize;
     int shift = 0;
     while ((1 << (shift + 1)) <= g_opt.hist_replicas) ++shift;
-    // tiles on demand only where the kernel before this one, in the same call, has reset the workspace's tile counter
-    // (the passes that leave statistics partials do)
-    const int dyn = HIST && stats_parts > 0 && n >= g_opt.dynamic_tail_min_elems ? g_opt.dynamic_tail_percent : 0;
+    // tiles on demand need the workspace's tile counter at zero: the lookup finalize that ends every call with a
+    // fused pass leaves it so (as do the passes that write statistics partials, and prime_workspace_init)
+    const int dyn = HIST && n >= g_opt.dynamic_tail_min_elems ? g_opt.dynamic_tail_percent : 0;
     if (!al)
         launch(id, 5.0 * n, quantize_kernel<false, false, HIST, REVERSE, kStorePlain>, grid, kThreads, st, x, n, scale, stats_parts, qp_out, zp, codes, ws, shift, dyn);
     else if ((n >> 18) >= g_opt.nt_second_min_mib)      // the quantize pass is always the last reader of the tensor
@@ -288,7 +288,7 @@ int run_quantize(const float* x, int64_t n, float scale, int stats_parts, prime_
     return launch_check("quantize_kernel");
 }
 
-int run_lut_finalize(const Workspace* ws, int nparts, float* lut, int64_t n_bins, uint64_t* counts, hipStream_t st) {
+int run_lut_finalize(Workspace* ws, int nparts, float* lut, int64_t n_bins, uint64_t* counts, hipStream_t st) {
     if (nparts == 0) {
         launch(kIdLutFinalize, 0.0, lut_zero_kernel, 1, 256, st, lut, n_bins, reinterpret_cast<unsigned long long*>(counts));
         return launch_check("lut_zero_kernel");
@@ -562,10 +562,12 @@ int prime_workspace_init(void* ws, int64_t ws_bytes, prime_stream_t stream) {
     if (!ws) return fail(PRIME_EWORKSPACE, "workspace is null");
     if (ws_bytes < static_cast<int64_t>(sizeof(Workspace))) return fail(PRIME_EWORKSPACE, "workspace too small");
     if (!aligned_to(ws, 16)) return fail(PRIME_EWORKSPACE, "workspace must be 16-byte aligned");
-    // Only the scale record is ever read before it is written by the same call sequence;
-    // clear it so that a stray read is defined.
+    // Read before the same call sequence writes them: the scale record (cleared so that a stray read is
+    // defined) and the tile counter of the fused pass, which must start at zero.  The head of the workspace
+    // up to the counter is cleared.
+    static_assert(offsetof(Workspace, tile_counter) % 4 == 0 && offsetof(Workspace, tile_counter) < 16384, "the counter sits in the head");
     launch(kIdFill, 0.0, fill_zero_kernel, 1, 64, static_cast<hipStream_t>(stream), static_cast<uint32_t*>(ws),
-           static_cast<int64_t>(sizeof(prime_qparams) / 4));
+           static_cast<int64_t>(offsetof(Workspace, tile_counter) / 4 + 1));
     return launch_check("fill_zero_kernel");
 }
 

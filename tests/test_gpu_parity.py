@@ -501,7 +501,7 @@ def test_tiles_dealt_on_demand_give_the_results_of_the_round_robin_deal_bit_for_
     # the fused pass may hand out its last tiles through a counter: which workgroup sees which tile then changes
     # from run to run, the integer histogram partials add up to the same totals, the codes depend on the element
     # alone.  Tensors with several rounds of tiles (two- and four-row), ordinary data and values beyond the
-    # fixed-point range, through uniform_8bit_quantize and a ring step.
+    # fixed-point range, through uniform_8bit_quantize, a ring step and quantize + lookup with a given scale.
     rng = np.random.default_rng(77)
     saved = {k: _lib.get_option(k) for k in ("dynamic_tail_percent", "dynamic_tail_min_mi_elems", "two_row_below_mi_elems")}
     try:
@@ -520,9 +520,15 @@ def test_tiles_dealt_on_demand_give_the_results_of_the_round_robin_deal_bit_for_
                 codes, lut, qp = abi.uniform(xt)
                 acc = abi.to_dev(acc0)
                 c2, l2, q2 = abi.ring_step(acc, codes, lut)
+                # the pass with a given scale has no statistics kernel ahead of it: the counter it deals tiles through
+                # is the one the call before left at zero; twice in a row
+                c3, l3 = abi.quantize_lookup(xt, 2.5e-5)
+                c4, l4 = abi.quantize_lookup(xt, 2.5e-5)
                 torch.cuda.synchronize()
+                assert torch.equal(c3, c4) and torch.equal(l3[1:255], l4[1:255])
                 got = [codes.cpu().numpy(), lut.cpu().numpy().view(np.uint32), qp.cpu().numpy().view(np.uint64),
-                       c2.cpu().numpy(), l2.cpu().numpy().view(np.uint32), q2.cpu().numpy().view(np.uint64), acc.cpu().numpy().view(np.uint32)]
+                       c2.cpu().numpy(), l2.cpu().numpy().view(np.uint32), q2.cpu().numpy().view(np.uint64), acc.cpu().numpy().view(np.uint32),
+                       c4.cpu().numpy(), l4.cpu().numpy().view(np.uint32)]
                 if want is None:
                     want = got
                     q = abi.qparams(qp)
@@ -533,7 +539,7 @@ def test_tiles_dealt_on_demand_give_the_results_of_the_round_robin_deal_bit_for_
                     continue
                 for k, (a, b) in enumerate(zip(got, want)):
                     # entries 0 and 255 of a table with far elements are fp64 sums in arrival order: compared by value
-                    if k in (1, 4):
+                    if k in (1, 4, 8):
                         assert np.array_equal(a[1:255], b[1:255]), (percent, k)
                         assert np.allclose(a.view(np.float32)[[0, 255]], b.view(np.float32)[[0, 255]], rtol=1e-6, atol=0), (percent, k)
                     else:
