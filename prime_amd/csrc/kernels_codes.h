@@ -72,7 +72,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_count_kernel(con
 
 // Between the passes, first kernel: total population of each code.  Workgroup j owns codes
 // 4j .. 4j+3 (16 contiguous bytes of every partial); lane (row, code) adds partials row,
-// row + 256, ..., then the rows are added by a tree of fixed shape.
+// row + 256, ..., then the rows are added up.
 __global__ __launch_bounds__(kFinalThreads) void code_total_kernel(Workspace* ws, int nparts) {
     constexpr int kRows = kFinalThreads / kLutBinsPerBlock;
     __shared__ unsigned long long sh_cnt[kFinalThreads];
@@ -89,13 +89,18 @@ __global__ __launch_bounds__(kFinalThreads) void code_total_kernel(Workspace* ws
     unsigned long long c = 0;
 #pragma unroll
     for (int k = 0; k < kIters; ++k) c += part[k];
-    sh_cnt[threadIdx.x] = c;
+    // integers: every wavefront joins the rows that share a row of sixteen lanes, the totals meet in LDS
+    // behind one barrier and the first wavefront adds them
+    c = sum_row_mod4(c);
+    if ((threadIdx.x & 15) < kLutBinsPerBlock) sh_cnt[(threadIdx.x >> 4) * kLutBinsPerBlock + bl] = c;
     __syncthreads();
-    for (int half = kRows / 2; half > 0; half >>= 1) {
-        if (row < half) sh_cnt[threadIdx.x] += sh_cnt[threadIdx.x + half * kLutBinsPerBlock];
-        __syncthreads();
+    if (threadIdx.x < 64) {
+        unsigned long long t = 0;
+#pragma unroll
+        for (int k = 0; k < kFinalThreads / 256; ++k) t += sh_cnt[threadIdx.x + 64 * k];
+        t = sum_lanes_mod4(t);
+        if (row == 0) ws->code_total[bin] = t;
     }
-    if (row == 0) ws->code_total[bin] = sh_cnt[threadIdx.x];
 }
 
 // Between the passes, second kernel, one workgroup: the statistics
@@ -235,14 +240,18 @@ __device__ __forceinline__ void dequant_block(float* __restrict__ out, const flo
     static_assert(!(ONESHOT && STATS), "statistics partials need the small grid of the looping sweep");
     using M = Mem<ALIGNED, NT>;
     constexpr int T = ONESHOT ? SHOT_THREADS : kThreads;
-    // The table goes to LDS once per workgroup, first thing.  A workgroup of the plain set that lives
-    // for one tile issues the tile's loads before that, so that the table's trip to L2 runs beside the
-    // codes' trip to memory instead of in front of it (2^28 elements: 210 instead of 233 us; with the
-    // accumulator's loads in flight as well the order makes no difference or costs 1 %).
-    constexpr bool kLateFill = ONESHOT && !ADD;
+    // The table goes to LDS once per workgroup.  A workgroup of the plain set that lives for one tile
+    // issues the tile's loads before that, so that the table's trip to L2 runs beside the codes' trip
+    // to memory instead of in front of it (2^28 elements: 210 instead of 233 us; with the accumulator's
+    // loads in flight as well the order makes no difference or costs 1 % there).  The looping passes do
+    // the same with their first tile: on a tensor of a few million elements the table's trip would
+    // otherwise stand alone at the head of the kernel.
+    constexpr bool kLateFill = (ONESHOT && !ADD) || !ONESHOT;
+    bool filled = false;                 // uniform over the workgroup
     auto fill_lut = [&] {
         for (int b = threadIdx.x; b < kBins; b += T) s_lut[b] = lut[b];
         __syncthreads();
+        filled = true;
     };
     if (!kLateFill) fill_lut();
     const int64_t nvec = n >> 2;
@@ -261,7 +270,7 @@ __device__ __forceinline__ void dequant_block(float* __restrict__ out, const flo
             c[j] = ok ? Mem<ALIGNED, true>::ldu32(codes, i) : 0u;      // a message is read once: never kept in cache
             if (ADD) a[j] = ok ? M::ldf4(out, i) : f4a{0.f, 0.f, 0.f, 0.f};
         }
-        if (kLateFill) fill_lut();        // every workgroup of such a launch has a tile: the barrier is uniform
+        if (kLateFill && !filled) fill_lut();        // the workgroup's first tile: the barrier is uniform
 #pragma unroll
         for (int j = 0; j < U; ++j) {
             const int64_t i = i0 + j * stride;
@@ -281,6 +290,7 @@ __device__ __forceinline__ void dequant_block(float* __restrict__ out, const flo
             }
         }
     });
+    if (slot == 0 && (n & 3) && !filled) fill_lut();      // a tensor of fewer than four elements: no tile at all
     if (slot == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (nvec << 2) + threadIdx.x;
         float v = s_lut[codes[i]];
