@@ -94,10 +94,12 @@ int prime_hip_profile_begin(void);
 int prime_hip_profile_end(prime_kernel_time* out, int capacity, int* count);
 
 /* Workspace: a fixed-size block of device memory (about 10 MiB) that holds every workgroup's
- * partial sums and partial 256-bin histogram between a kernel and its second stage.  It
- * carries no state from one call to the next; prime_workspace_init only validates it and
- * clears the scale record (a fill kernel, safe under stream capture).  Two calls that share a
- * workspace must be ordered on one stream. */
+ * partial sums and partial 256-bin histogram between a kernel and its second stage.  The one
+ * thing it carries from call to call is a tile counter that every call leaves at zero;
+ * prime_workspace_init validates the block and clears its head, the scale record and that
+ * counter (a fill kernel, safe under stream capture): call it once on a new workspace before
+ * any other entry point sees it.  Two calls that share a workspace must be ordered on one
+ * stream. */
 int64_t prime_workspace_bytes(void);
 int prime_workspace_init(void* ws, int64_t ws_bytes, prime_stream_t stream);
 
