@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <vector>
 
+#include <cstring>
 #include "prime_hip.h"
 
 extern "C" {
@@ -167,6 +168,70 @@ int main() {
         for (void* p : {(void*)d_x, (void*)d_acc, (void*)d_c1, (void*)d_c2, (void*)d_c3, (void*)d_l1, (void*)d_l2, (void*)d_l3,
                         (void*)d_out, (void*)d_qp})
             HIP_OK(hipFree(p));
+    }
+
+    // several tensors in one segmented call: every tensor's results are those of the one-tensor entry point
+    {
+        const std::vector<int64_t> ns = {int64_t(3) << 18, 0, 70001, (int64_t(1) << 20) + 1, 5, 300000};
+        const int64_t count = static_cast<int64_t>(ns.size());
+        std::vector<float*> xs(ns.size()), accs(ns.size());
+        std::vector<uint8_t*> cs(ns.size()), cs1(ns.size()), cs2(ns.size());
+        std::vector<const float*> xs_c(ns.size()), luts_in(ns.size());
+        std::vector<const uint8_t*> codes_in(ns.size());
+        float *d_luts, *d_luts2, *d_lut1;
+        prime_qparams *d_qps, *d_qp1;
+        HIP_OK(hipMalloc(&d_luts, ns.size() * 1024));
+        HIP_OK(hipMalloc(&d_luts2, ns.size() * 1024));
+        HIP_OK(hipMalloc(&d_lut1, 1024));
+        HIP_OK(hipMalloc(&d_qps, ns.size() * sizeof(prime_qparams)));
+        HIP_OK(hipMalloc(&d_qp1, sizeof(prime_qparams)));
+        for (size_t t = 0; t < ns.size(); ++t) {
+            xs[t] = to_device(make_input(ns[t] ? ns[t] : 1, 10 + static_cast<int>(t), 1e-3f));
+            accs[t] = to_device(make_input(ns[t] ? ns[t] : 1, 30 + static_cast<int>(t), 1e-3f));
+            xs_c[t] = xs[t];
+            HIP_OK(hipMalloc(&cs[t], ns[t] + 16));
+            HIP_OK(hipMalloc(&cs1[t], ns[t] + 16));
+            HIP_OK(hipMalloc(&cs2[t], ns[t] + 16));
+        }
+        PRIME_OK(prime_uniform_8bit_quantize_segmented(xs_c.data(), ns.data(), count, cs.data(), d_luts, d_qps, ws, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        const auto seg_luts = to_host(d_luts, 256 * count);
+        const auto seg_qps = to_host(d_qps, count);
+        for (size_t t = 0; t < ns.size(); ++t) {
+            if (ns[t] == 0) continue;
+            PRIME_OK(prime_uniform_8bit_quantize(xs[t], ns[t], cs1[t], d_lut1, d_qp1, ws, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            expect(to_host(cs[t], ns[t]) == to_host(cs1[t], ns[t]), "segmented call: codes of the one-tensor call");
+            const auto l1 = to_host(d_lut1, 256);
+            expect(std::memcmp(l1.data(), seg_luts.data() + 256 * t, 1024) == 0, "segmented call: lookup table of the one-tensor call, bit for bit");
+            const auto q1 = to_host(d_qp1, 1);
+            expect(std::memcmp(&q1[0], &seg_qps[t], sizeof(prime_qparams)) == 0, "segmented call: statistics record of the one-tensor call");
+            codes_in[t] = cs[t];
+            luts_in[t] = d_luts + 256 * t;
+        }
+        codes_in[1] = cs[1];
+        luts_in[1] = d_luts + 256;
+        // a ring step on every accumulator with its tensor's message, in one call; then one by one on copies
+        std::vector<std::vector<float>> acc_before(ns.size());
+        for (size_t t = 0; t < ns.size(); ++t) acc_before[t] = to_host(accs[t], ns[t]);
+        PRIME_OK(prime_ring_reduce_step_segmented(accs.data(), codes_in.data(), luts_in.data(), ns.data(), count, cs2.data(), d_luts2, nullptr, ws,
+                                                  stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        const auto seg_luts2 = to_host(d_luts2, 256 * count);
+        for (size_t t = 0; t < ns.size(); ++t) {
+            if (ns[t] == 0) continue;
+            float* d_acc = to_device(acc_before[t]);
+            PRIME_OK(prime_ring_reduce_step(d_acc, cs[t], d_luts + 256 * t, ns[t], cs1[t], d_lut1, nullptr, ws, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            expect(to_host(d_acc, ns[t]) == to_host(accs[t], ns[t]), "segmented ring step: accumulator of the one-tensor call");
+            expect(to_host(cs2[t], ns[t]) == to_host(cs1[t], ns[t]), "segmented ring step: codes of the one-tensor call");
+            const auto l1 = to_host(d_lut1, 256);
+            expect(std::memcmp(l1.data(), seg_luts2.data() + 256 * t, 1024) == 0, "segmented ring step: lookup table of the one-tensor call");
+            HIP_OK(hipFree(d_acc));
+        }
+        for (size_t t = 0; t < ns.size(); ++t)
+            for (void* p : {(void*)xs[t], (void*)accs[t], (void*)cs[t], (void*)cs1[t], (void*)cs2[t]}) HIP_OK(hipFree(p));
+        for (void* p : {(void*)d_luts, (void*)d_luts2, (void*)d_lut1, (void*)d_qps, (void*)d_qp1}) HIP_OK(hipFree(p));
     }
 
     // error behaviour: rejected arguments return non-zero with a message, and launch nothing
