@@ -13,8 +13,11 @@ side of the compressed all-reduce:
 The reference keeps the outer copy, the gradient and the optimizer state in host memory and
 pays a device-to-host copy of every parameter per outer step; with 288 GB of HBM they stay on
 the device: the pseudo-gradient is one fused launch per 64 parameters, and the optimizer step
-and the copy back to the model are one more.  Elastic membership, retries and the barrier of
-the reference (:84,:92-126) belong to its control plane and are not here.
+and the copy back to the model are one more.  The retry loop around the all-reduce (:92-126) is
+kept, with what it falls back to when every attempt fails (the worker's own pseudo-gradient,
+not divided: :127-132); elastic membership and the barrier (:84, :103) belong to the reference's
+control plane and are not here: a caller that can rebuild its process group hands
+``sync_pseudo_gradient`` a ``regroup`` callable for the retries (:121).
 
 With ``flat_inner=True`` the model's own parameters are moved into a fourth flat buffer laid
 out like the other three (each ``param.data`` becomes a view of it).  The pseudo-gradient and
@@ -52,6 +55,7 @@ class Diloco:
         self.outer_lr = float(outer_lr)
         self.compression = compression
         self._first_step = True
+        self.last_all_reduce_error: Optional[BaseException] = None
         self.inner_flat: Optional[torch.Tensor] = None
         self._init_outer_state(model)
         if flat_inner:
@@ -134,6 +138,30 @@ class Diloco:
             all_reduce(self.compression, bucket, dist.ReduceOp.SUM, group)
 
     @torch.no_grad()
+    def sync_pseudo_gradient(self, model: nn.Module, group: Optional[object], world_size: int, fake: bool = False,
+                             retry_all_reduce: int = 1, regroup=None) -> bool:
+        """Pseudo-gradient, then the all-reduce of every bucket, tried up to ``retry_all_reduce`` times
+        (diloco.py:92-126: the gradient is formed afresh for every attempt, because a failed all-reduce
+        leaves the buckets half reduced).  After an attempt that raised, ``regroup()`` (if given) returns the
+        group for the next one (:121).  When every attempt has failed the worker keeps its own pseudo-gradient,
+        outer - inner, not divided by the world size (:127-132).  Returns whether an all-reduce went through."""
+        if retry_all_reduce < 1:
+            raise ValueError("retry_all_reduce must be at least 1")
+        last = None
+        for attempt in range(retry_all_reduce):
+            self.compute_pseudo_gradient(model, world_size, fake=fake)
+            try:
+                self.all_reduce_buckets(group)
+                return True
+            except Exception as e:      # the reference catches everything here (:119)
+                last = e
+                if regroup is not None and attempt + 1 < retry_all_reduce:
+                    group = regroup()
+        self.compute_pseudo_gradient(model, 1, fake=fake)
+        self.last_all_reduce_error = last
+        return False
+
+    @torch.no_grad()
     def outer_step(self, model: nn.Module) -> None:
         """outer_optimizer.step() and sync_inner_model (diloco.py:212-215), one launch per 64 parameters
         (one for the whole model when the inner parameters are flat)."""
@@ -148,12 +176,17 @@ class Diloco:
         self._first_step = False
 
     @torch.no_grad()
-    def step(self, model: nn.Module, group: Optional[object] = None, world_size: Optional[int] = None, fake: bool = False) -> None:
-        """The whole outer step of one worker (diloco.py:203-215)."""
+    def step(self, model: nn.Module, group: Optional[object] = None, world_size: Optional[int] = None, fake: bool = False,
+             retry_all_reduce: int = 1, regroup=None) -> None:
+        """The whole outer step of one worker (diloco.py:203-215).  With ``retry_all_reduce`` > 1 a failing
+        all-reduce is tried again as the reference tries it; with the default an exception propagates."""
         if world_size is None:
             world_size = group.size() if group is not None else dist.get_world_size()
-        self.compute_pseudo_gradient(model, world_size, fake=fake)
-        self.all_reduce_buckets(group)
+        if retry_all_reduce > 1 or regroup is not None:
+            self.sync_pseudo_gradient(model, group, world_size, fake=fake, retry_all_reduce=retry_all_reduce, regroup=regroup)
+        else:
+            self.compute_pseudo_gradient(model, world_size, fake=fake)
+            self.all_reduce_buckets(group)
         self.outer_step(model)
 
 

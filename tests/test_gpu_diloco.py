@@ -386,6 +386,50 @@ def test_uncompressed_simulated_all_reduce_and_fake_step(dev):
         assert torch.equal(p.detach(), q)
 
 
+def test_all_reduce_is_retried_and_falls_back_to_the_unreduced_pseudo_gradient(dev):
+    # diloco.py:92-132: every attempt forms the pseudo-gradient afresh and all-reduces the buckets; an attempt that
+    # raises is followed by another on the group regroup() returns; when all have failed the worker keeps
+    # outer - inner, not divided by the world size
+    from prime_amd.C.collectives import SimulatedRing
+    from prime_amd.collectives import Compression
+    from prime_amd.diloco import Diloco
+
+    class Broken:
+        """A group whose all-reduce cannot run: prime_amd.collectives.all_reduce raises on it."""
+
+    torch.manual_seed(5)
+    model = TinyLlama().to(dev)
+    d = Diloco(0.7, model, compression=Compression.NO)
+    for p in model.parameters():
+        p.data.add_(torch.randn_like(p) * 1e-3)
+    inner = torch.cat([p.detach().reshape(-1) for p in model.parameters()])
+    want = d.outer_data_flat - inner
+
+    # every attempt fails: the fallback
+    calls = []
+    ok = d.sync_pseudo_gradient(model, Broken(), world_size=4, retry_all_reduce=3, regroup=lambda: calls.append(1) or Broken())
+    assert ok is False and len(calls) == 2 and d.last_all_reduce_error is not None
+    assert torch.equal(d.grad_flat, want)                                   # not divided by 4
+
+    # the second attempt succeeds on the group regroup() hands over: SUM over one simulated rank of grad / 4
+    ok = d.sync_pseudo_gradient(model, Broken(), world_size=4, retry_all_reduce=3, regroup=lambda: SimulatedRing([d.grad_flat]))
+    assert ok is True
+    assert torch.equal(d.grad_flat, want / 4.0)
+
+    # without retries the exception reaches the caller, as before
+    with pytest.raises(Exception):
+        d.step(model, group=Broken(), world_size=4)
+    with pytest.raises(ValueError, match="at least 1"):
+        d.sync_pseudo_gradient(model, Broken(), world_size=4, retry_all_reduce=0)
+
+    # step() with retries applies the outer optimizer to the fallback gradient
+    before = d.outer_data_flat.clone()
+    d.step(model, group=Broken(), world_size=4, retry_all_reduce=2)
+    torch.cuda.synchronize()
+    # first Nesterov step: p -= lr (1 + mu) g; the difference of two fp32 parameters of size ~1 carries ~1e-7
+    assert torch.allclose(before - d.outer_data_flat, 0.7 * 1.9 * want, rtol=1e-4, atol=1e-6)
+
+
 def test_outer_step_with_a_real_process_group_of_one_rank(dev, oracle, tmp_path):
     # the reference's call site unchanged: all_reduce(Compression.UINT8, bucket, SUM, group) on the default
     # process group; with one rank no message is sent, but every bucket's two chunks still take the lossy
