@@ -298,7 +298,7 @@ def test_reference_import_paths_reach_the_hip_kernels(dev):
             del sys.modules[k]
 
 
-@pytest.mark.parametrize("W", [1, 2, 3, 4, 8])
+@pytest.mark.parametrize("W", [1, 2, 3, 4, 5, 7, 8])
 @pytest.mark.parametrize("avg", [False, True])
 @pytest.mark.parametrize("code_domain", [False, True])
 def test_ring_closed_form_on_chunkwise_constant_inputs(dev, W, avg, code_domain):
