@@ -189,8 +189,9 @@ __global__ __launch_bounds__(kFinalThreads) void requant_plan_kernel(Workspace* 
     }
 }
 
-// Pass 2: codes_out[i] = map[codes_in[i]].  2 bytes per element.
-template <bool ALIGNED>
+// Pass 2: codes_out[i] = map[codes_in[i]].  2 bytes per element.  REVERSE: from the end of the codes, where the
+// last-level cache still holds what the counting pass read last.
+template <bool ALIGNED, bool REVERSE = false>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_remap_kernel(const uint8_t* __restrict__ in, uint8_t* __restrict__ out,
                                                                               int64_t n, const Workspace* __restrict__ ws) {
     __shared__ uint32_t map_words[kBins / 4];
@@ -202,7 +203,8 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void code_remap_kernel(con
                (static_cast<uint32_t>(map[(w >> 16) & 255]) << 16) | (static_cast<uint32_t>(map[w >> 24]) << 24);
     };
     const int64_t nvec = n >> 4;
-    sweep(nvec, [&](int64_t i0, int64_t stride, auto full_t) {
+    sweep_tiles<kUnroll, REVERSE>(nvec, [&](int64_t base, int64_t stride, auto full_t) {
+        const int64_t i0 = base + threadIdx.x;
         constexpr bool full = decltype(full_t)::value;
         u4a v[kUnroll];
 #pragma unroll

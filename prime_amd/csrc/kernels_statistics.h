@@ -12,19 +12,36 @@ __global__ __launch_bounds__(kFinalThreads) void stats_finalize_kernel(Workspace
 
 // The statistics partial of workgroup `slot` of a grid of G, computed by the calling workgroup and
 // stored in the workspace: fp64 sum and sum of squares of the rows that workgroup owns.
+//
+// With NT the loads carry the non-temporal hint, except from vector `keep_from` on: what a hinted load
+// brings in does not stay in the last-level cache, and the pass that re-reads the tensor from its end
+// finds there what this pass read last without the hint.
+constexpr int64_t kKeepNothing = INT64_MAX;
 template <bool ALIGNED, bool NT, int U = kUnroll>
-__device__ __forceinline__ void stats_partial(const float* __restrict__ x, int64_t n, int slot, int G, double* part_sum, double* part_sq) {
+__device__ __forceinline__ void stats_partial(const float* __restrict__ x, int64_t n, int slot, int G, double* part_sum, double* part_sq,
+                                              int64_t keep_from = kKeepNothing) {
     using M = Mem<ALIGNED, NT>;
+    using Kept = Mem<ALIGNED, false>;
     const int64_t nvec = n >> 2;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
     sweep_tiles_of<U, false>(nvec, slot, G, [&](int64_t base, int64_t stride, auto full_t) {
         constexpr bool full = decltype(full_t)::value;
         const int64_t i0 = base + threadIdx.x;
         f4a v[U];
+        if (NT && base >= keep_from) {
+            asm volatile("" ::: "memory");        // keeps the two sets of loads apart: merged, they would lose the hint
 #pragma unroll
-        for (int j = 0; j < U; ++j) {
-            const int64_t i = i0 + j * stride;
-            v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            for (int j = 0; j < U; ++j) {
+                const int64_t i = i0 + j * stride;
+                v[j] = (full || i < nvec) ? Kept::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            }
+            asm volatile("" ::: "memory");
+        } else {
+#pragma unroll
+            for (int j = 0; j < U; ++j) {
+                const int64_t i = i0 + j * stride;
+                v[j] = (full || i < nvec) ? M::ldf4(x, i) : f4a{0.f, 0.f, 0.f, 0.f};
+            }
         }
 #pragma unroll
         for (int j = 0; j < U; ++j) {
@@ -101,9 +118,10 @@ __device__ __forceinline__ void stats_partial_short(const float* __restrict__ x,
 // K1: sum and sum of squares in fp64.  4 bytes per element.
 // U = rows per tile: 4 from 2^27 elements up, 2 below (a 51 M-element bucket: 33.3 against 34.4 us).
 template <bool ALIGNED, bool NT, int U = kUnroll>
-__global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws) {
+__global__ __launch_bounds__(kThreads, kWavesPerSimd) void stats_kernel(const float* __restrict__ x, int64_t n, Workspace* ws,
+                                                                                int64_t keep_from) {
     if (blockIdx.x == 0 && threadIdx.x == 0) ws->tile_counter = 0u;      // for the quantize pass that follows (sweep_tiles_dynamic)
-    stats_partial<ALIGNED, NT, U>(x, n, blockIdx.x, gridDim.x, ws->part_sum, ws->part_sq);
+    stats_partial<ALIGNED, NT, U>(x, n, blockIdx.x, gridDim.x, ws->part_sum, ws->part_sq, keep_from);
 }
 
 // The norm as libtorch's CPU kernel accumulates it (the value compression.cpp:113 actually

@@ -451,7 +451,7 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
 
 
 @pytest.mark.parametrize("option,values", [("hist_replicas", (1, 2, 4, 8)), ("average_replicas", (1, 2, 4, 8, 16)), ("blocks_per_cu", (1, 2, 3, 4)),
-                                           ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20)),
+                                           ("nt_load_min_mib", (0, 1 << 20)), ("nt_second_min_mib", (0, 1 << 20)), ("stats_keep_mib", (0, 1, 256)),
                                            ("code_store_policy", (0, 2, 16)), ("f32_reread_store_policy", (0, 2, 16)),
                                            ("reverse_second_pass", (0, 1)), ("one_shot", (0, 1)),
                                            ("one_shot_store_policy", (0, 2, 16)), ("two_row_below_mi_elems", (0, 128)),
