@@ -44,6 +44,7 @@ const char* prime_hip_last_error(void);
 /* Tuning knobs: "blocks_per_cu" (workgroups per compute unit of a streaming kernel),
  * "large_read_grid_eighths" / "large_read_min_mi_elems" (kernels that read at least as much as they
  * write use this many eighths of the compute units on tensors of at least that many Mi elements),
+ * "stats_grid_eighths" (the statistics pass on such tensors: at most this many eighths; 0: the same as the others),
  * "code_store_policy", "f32_store_policy", "f32_reread_store_policy", "copy_store_policy" (cache
  * policy of the stores of codes, of fp32 outputs, of fp32 outputs the next kernel reads back, of
  * the plain copy: 0 write-back, 2 non-temporal, 16 write-through), "reverse_second_pass" (the pass
@@ -71,7 +72,7 @@ const char* prime_hip_last_error(void);
  * experiments; 0: none).
  * Cache policies, load hints, the one-workgroup-per-tile and one-launch variants, the number of LDS
  * copies, the dynamic tail and segment_blocks_per_cu never change a result.  The options that change the number of
- * workgroups of the statistics pass or its tile shape (blocks_per_cu, grid_cap, large_read_*,
+ * workgroups of the statistics pass or its tile shape (blocks_per_cu, grid_cap, large_read_*, stats_grid_eighths,
  * two_row_below_mi_elems) change the order in which the fp64 sums are added: codes and scale have been
  * equal on all tested data, but a sum may move in its last bit and, rarely, a scale with it.
  * Returns 0 if the name is known.  The

@@ -54,6 +54,7 @@ struct Options {
     int blocks_per_cu = 1;          // workgroups per compute unit a streaming kernel is launched with
     int large_read_grid_eighths = 7;   // read-heavy kernels on large tensors: workgroups = this many eighths of the compute units
     int64_t large_read_min_elems = int64_t(1) << 27;
+    int stats_grid_eighths = 6;        // the statistics pass on such tensors: at most this many eighths (0: as the line above)
     int nt_load_min_mib = 512;      // tensors of at least this many MiB are loaded with the non-temporal hint
     int stats_keep_mib = 256;       // the statistics pass of uniform_8bit_quantize: all but the last this many MiB hinted (0: as the line above)
     int nt_second_min_mib = 0;      // the same for the quantize pass that re-reads a tensor: its last use, always hinted
@@ -110,7 +111,9 @@ constexpr int64_t kRowElems = static_cast<int64_t>(kThreads) * 4;
 // per compute unit is at least as fast as two from 4 Mi elements up (fewer concurrent streams into
 // HBM), and with `reads` (a kernel that reads at least as much as it writes) tensors of 2^27 elements
 // or more do best on seven eighths of the compute units: at 2^28 elements the statistics pass goes
-// from 158 to 152 us and the quantize pass from 241 to 218 us.  A kernel that mostly writes
+// from 158 to 152 us and the quantize pass from 241 to 218 us; the statistics pass, which only reads, does
+// better still on six eighths (2^27: 79.9 -> 77.2 us, 2^28: 156 -> 151 us, 2^29: 307 -> 299 us; below 2^27
+// elements every compute unit stays ahead for both).  A kernel that mostly writes
 // (dequantize set) wants every compute unit.
 int grid_for(int64_t n, bool reads = false) {
     int64_t tiles = (n + kRowElems - 1) / kRowElems;
@@ -123,6 +126,15 @@ int grid_for(int64_t n, bool reads = false) {
     if (cap > kMaxGrid) cap = kMaxGrid;
     if (g_opt.grid_cap > 0 && cap > g_opt.grid_cap) cap = g_opt.grid_cap;
     return static_cast<int>(tiles < cap ? tiles : cap);
+}
+
+// Workgroups (= partials) of the statistics pass over a tensor: every path that stands in for that pass takes its
+// slots from here, so that the fp64 sums are added in one order whichever entry point runs.
+int stats_grid_for(int64_t n) {
+    int grid = grid_for(n, true);
+    if (n >= g_opt.large_read_min_elems && g_opt.stats_grid_eighths > 0)
+        grid = std::min(grid, std::max(8, cu_count() / 8 * g_opt.stats_grid_eighths));
+    return grid;
 }
 
 // One workgroup per tile for a kernel launched ONESHOT.
@@ -215,7 +227,7 @@ int run_stats_finalize(Workspace* ws, int nparts, int64_t n, prime_qparams* out,
 // rest with it: 2^28 elements 364 instead of 377 us for the whole call (the quantize pass 202 instead of 217 us),
 // 2^27 185 instead of 196 us; up to 256 MiB nothing is hinted, as before.
 int run_stats_partials(const float* x, int64_t n, Workspace* ws, hipStream_t st, int* parts, bool reread = false) {
-    const int grid = grid_for(n, true);
+    const int grid = stats_grid_for(n);
     const bool two = two_row_tiles(n);
     const bool keep_end = reread && g_opt.reverse_second_pass && g_opt.stats_keep_mib > 0;
     const bool nt = keep_end ? (n >> 18) > g_opt.stats_keep_mib : use_nt(n);
@@ -448,6 +460,9 @@ int prime_hip_set_option(const char* name, int value) {
     } else if (!strcmp(name, "large_read_grid_eighths")) {
         if (value < 0 || value > 16) return fail(PRIME_EINVAL, "large_read_grid_eighths must be 0 (off) .. 16");
         g_opt.large_read_grid_eighths = value;
+    } else if (!strcmp(name, "stats_grid_eighths")) {
+        if (value < 0 || value > 16) return fail(PRIME_EINVAL, "stats_grid_eighths must be 0 (off) .. 16");
+        g_opt.stats_grid_eighths = value;
     } else if (!strcmp(name, "large_read_min_mi_elems")) {
         if (value < 0) return fail(PRIME_EINVAL, "large_read_min_mi_elems must be >= 0");
         g_opt.large_read_min_elems = static_cast<int64_t>(value) << 20;
@@ -524,6 +539,7 @@ int prime_hip_get_option(const char* name, int* value) {
     else if (!strcmp(name, "nt_load_min_mib")) *value = g_opt.nt_load_min_mib;
     else if (!strcmp(name, "nt_second_min_mib")) *value = g_opt.nt_second_min_mib;
     else if (!strcmp(name, "stats_keep_mib")) *value = g_opt.stats_keep_mib;
+    else if (!strcmp(name, "stats_grid_eighths")) *value = g_opt.stats_grid_eighths;
     else if (!strcmp(name, "unroll")) *value = kUnroll;
     else if (!strcmp(name, "threads")) *value = kThreads;
     else return fail(PRIME_EINVAL, "unknown option");
@@ -847,7 +863,7 @@ int run_segment_group(SegKind kind, int count, float* const* xs, const int64_t* 
         job.codes_in[t] = codes_in ? codes_in[t] : nullptr;
         job.lut_in[t] = luts_in ? luts_in[t] : nullptr;
         // the statistics slots: the grid the one-tensor entry point launches for its first pass
-        job.parts[t] = kind == kSegUniform ? grid_for(ns[t], true) : grid_for(ns[t], add);
+        job.parts[t] = kind == kSegUniform ? stats_grid_for(ns[t]) : grid_for(ns[t], add);
         if (kind == kSegUniform && two_row_tiles(ns[t])) job.two_row |= 1ull << t;
         total += ns[t];
         bytes_a += (kind == kSegUniform ? 4.0 : add ? 9.0 : 5.0) * ns[t];

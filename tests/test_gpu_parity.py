@@ -456,7 +456,7 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
                                            ("reverse_second_pass", (0, 1)), ("one_shot", (0, 1)),
                                            ("one_shot_store_policy", (0, 2, 16)), ("two_row_below_mi_elems", (0, 128)),
                                            ("set_four_rows_max_mi_elems", (0, 32)), ("grid_cap", (0, 7, 64)),
-                                           ("large_read_grid_eighths", (0, 3, 7)), ("large_read_min_mi_elems", (0, 128)),
+                                           ("large_read_grid_eighths", (0, 3, 7)), ("large_read_min_mi_elems", (0, 128)), ("stats_grid_eighths", (0, 3, 6)),
                                            ("f32_store_policy", (0, 2, 16)), ("copy_store_policy", (0, 2, 16)),
                                            ("dynamic_tail_percent", (0, 5, 100)), ("dynamic_tail_min_mi_elems", (0, 128)),
                                            ("segment_blocks_per_cu", (1, 2, 4))])
@@ -468,7 +468,10 @@ def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle,
     inputs = {"normal": (rng.standard_normal(n) * 1e-3).astype(np.float32),
               "near one": (1 + rng.standard_normal(n) * 1e-2).astype(np.float32)}
     old = _lib.get_option(option)
+    old_large = _lib.get_option("large_read_min_mi_elems")
     try:
+        if option == "stats_grid_eighths":
+            _lib.set_option("large_read_min_mi_elems", 0)        # the option acts on "large" tensors only: make these large
         for value in values:
             _lib.set_option(option, value)
             for label, x in inputs.items():
@@ -495,6 +498,8 @@ def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle,
             assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
     finally:
         _lib.set_option(option, old)
+        if option == "stats_grid_eighths":
+            _lib.set_option("large_read_min_mi_elems", old_large)
 
 
 def test_tiles_dealt_on_demand_give_the_results_of_the_round_robin_deal_bit_for_bit(abi, oracle):
