@@ -521,11 +521,12 @@ def main() -> int:
         out["roofline"] = {
             "bound": "hbm",
             "kernel": "quantize_kernel<aligned, nt loads, hist, walked from the end, non-temporal code stores, four-row tiles> "
-                      "(quantize + 256-bin count / fixed-point sum histogram, the last 5 % of the tiles dealt on demand)",
+                      "(quantize + 256-bin count / fixed-point sum histogram; 256 workgroups, the tiles of the tensor's cached end "
+                      "visited spread among the others, the last 5 % of the tiles dealt on demand)",
             "workload": "inside uniform_8bit_quantize on 2^28-element tensors (1 GiB each; inputs and code buffers three in rotation: "
                         "nothing of either is left in the 256 MB last-level cache when the call starts).  Cache-assisted by the "
                         "call's own statistics pass, which reads the tensor's last 256 MiB without the non-temporal hint: this "
-                        "pass walks the tensor from its end and takes that quarter of its reads from the last-level cache; "
+                        "pass takes that quarter of its reads from the last-level cache, interleaved with the three quarters from HBM; "
                         "input_cold is the same kernel with the scale given and nothing cached",
             "achieved": round(dom_bytes / dom_us / 1e3, 1),
             "peak": HBM_PEAK_GBS,

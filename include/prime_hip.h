@@ -54,7 +54,10 @@ const char* prime_hip_last_error(void);
  * are read with non-temporal loads in their first pass), "stats_keep_mib" (the statistics pass of
  * uniform_8bit_quantize reads the last this many MiB of the tensor without that hint and all before them with it,
  * whatever the size: what a hinted load fetches does not stay in the last-level cache, and the quantize pass
- * starts at the tensor's end; 0: nt_load_min_mib decides for the whole tensor), "nt_second_min_mib" (the same for the
+ * starts at the tensor's end; 0: nt_load_min_mib decides for the whole tensor), "mix_cached" (on tensors of at least
+ * twice that size the quantize pass visits the tiles of that cached end spread evenly among the others instead of
+ * first, so that cache and memory deliver side by side) and "mixed_grid_eighths" (eighths of the compute units it then
+ * runs on), "nt_second_min_mib" (the same for the
  * quantize pass that reads a tensor for the last time), "one_shot" (kernels that keep nothing from
  * tile to tile - dequantize, plain quantize, divide, pseudo-gradient, outer step, copy - run as one
  * 256-lane workgroup per tile from 65536 elements up instead of a loop) and "one_shot_store_policy"

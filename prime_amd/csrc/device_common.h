@@ -412,8 +412,13 @@ __device__ __forceinline__ void sweep_tiles_of(int64_t nvec, int64_t slot, int64
 // gets which of these tiles differs from run to run: only for passes whose per-workgroup results add
 // up to the same totals in any order (integer histogram partials; codes depend on nothing but the
 // element).  Every workgroup of the launch must call this (it uses barriers while tiles are left).
+//
+// mix_rounds (REVERSE only): the last that many rounds of the tensor are in the last-level cache (the pass before
+// left them there).  Instead of first, they are visited spread evenly among the rounds of the part that comes
+// from memory, so that cache and memory deliver side by side for the whole pass instead of one after the other.
 template <int U, bool REVERSE, typename Body>
-__device__ __forceinline__ void sweep_tiles_dynamic(int64_t nvec, int64_t slot, int64_t G, unsigned* counter, int dyn_percent, Body&& body) {
+__device__ __forceinline__ void sweep_tiles_dynamic(int64_t nvec, int64_t slot, int64_t G, unsigned* counter, int dyn_percent, Body&& body,
+                                                    int64_t mix_rounds = 0) {
     __shared__ unsigned sh_next[2];
     const int64_t rows = (nvec + kThreads - 1) / kThreads;
     const int64_t rounds = (nvec / kThreads) / (G * U);
@@ -424,8 +429,14 @@ __device__ __forceinline__ void sweep_tiles_dynamic(int64_t nvec, int64_t slot, 
     // forward: static tiles [0, static_rounds * G), then the dynamic ones, then the ragged rows;
     // reverse: the ragged rows, static tiles from the end down to dyn_tiles, then the dynamic ones [0, dyn_tiles) downwards
     if (REVERSE && r0 < rows) body(r0 * kThreads, G * kThreads, std::false_type{});
+    const bool mixed = REVERSE && mix_rounds > 0 && mix_rounds < static_rounds;
     for (int64_t kk = 0; kk < static_rounds; ++kk) {
-        const int64_t k = REVERSE ? rounds - 1 - kk : kk;
+        int64_t k = REVERSE ? rounds - 1 - kk : kk;
+        if (mixed) {
+            // the cached rounds spread evenly over the walk: position kk takes one when the running share crosses an integer
+            const int64_t before = kk * mix_rounds / static_rounds, after = (kk + 1) * mix_rounds / static_rounds;
+            k = after > before ? rounds - 1 - before : rounds - 1 - mix_rounds - (kk - before);
+        }
         body(((k * G + slot) * U) * kThreads, static_cast<int64_t>(kThreads), std::true_type{});
     }
     if (dyn_tiles > 0) {

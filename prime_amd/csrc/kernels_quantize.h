@@ -39,6 +39,7 @@ struct HistOut {
     bool first;
     unsigned* tile_counter;     // deals the last part of the tiles on demand (sweep_tiles_dynamic); null: all round-robin
     int dyn_percent;
+    int mix_rounds = 0;         // rounds of tiles at the tensor's end that the last-level cache holds (sweep_tiles_dynamic)
     bool cleared = false;       // the caller has zeroed the fixed-point histogram (all copies) ahead of a barrier
 };
 __device__ __forceinline__ HistOut hist_out_of(Workspace* ws, int slot, int dyn_percent) {
@@ -133,7 +134,7 @@ __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int6
             }
         };
         // the fixed-point histogram's partials are integers: its tiles may go to any workgroup
-        if constexpr (kMode == kFixed) sweep_tiles_dynamic<U, REVERSE>(nvec, slot, G, out_part.tile_counter, out_part.dyn_percent, body);
+        if constexpr (kMode == kFixed) sweep_tiles_dynamic<U, REVERSE>(nvec, slot, G, out_part.tile_counter, out_part.dyn_percent, body, out_part.mix_rounds);
         else sweep_tiles_of<U, REVERSE>(nvec, slot, G, body);
         if (slot == 0 && threadIdx.x < (n & 3)) {
             const int64_t i = (nvec << 2) + threadIdx.x;
@@ -173,7 +174,8 @@ __device__ __forceinline__ void quantize_block(const float* __restrict__ x, int6
 template <bool ALIGNED, bool NT, bool HIST, bool REVERSE, int POLICY, int U = kUnroll>
 __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const float* __restrict__ x, int64_t n, float scale_val,
                                                             int stats_parts, prime_qparams* qp_out, int zero_point,
-                                                            uint8_t* __restrict__ codes, Workspace* ws, int copies_shift, int dyn_percent) {
+                                                            uint8_t* __restrict__ codes, Workspace* ws, int copies_shift, int dyn_percent,
+                                                            int mix_rounds) {
     // the scale: given by value, or derived here from the statistics partials of the pass before
     // (stats_parts < 0: the record a preceding kernel left in the workspace)
     int narrow = INT_MIN;                // set when the statistics show a tensor crowded into a few codes
@@ -188,6 +190,7 @@ __global__ __launch_bounds__(kThreads, kWavesPerSimd) void quantize_kernel(const
                                         : 1.0f / scale_val;
     HistOut out = hist_out_of(HIST ? ws : nullptr, blockIdx.x, dyn_percent);
     out.cleared = HIST && stats_parts > 0;
+    out.mix_rounds = mix_rounds;
     quantize_block<ALIGNED, NT, HIST, REVERSE, POLICY, U>(x, n, inv, narrow, zero_point, codes, out, copies_shift, blockIdx.x, gridDim.x,
                                                        reinterpret_cast<QuantHist&>(hist_mem));
 }

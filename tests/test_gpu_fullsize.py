@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 import torch
 
+from prime_amd import _lib
 from tests.conftest import tables_agree
 from tests.gpu_util import Abi, announce
 
@@ -53,6 +54,22 @@ def test_uniform_8bit_quantize_2p28_properties(abi):
     assert torch.equal(out, lut[codes.long()])
     inside = (codes > 0) & (codes < 255)
     assert float((out - x)[inside].abs().max()) <= float(q["scale"])
+    del out, inside
+    # the default walk spreads the cached end of the tensor among the other tiles and keeps that end out of the
+    # statistics pass's load hint: without either, the same codes, table and statistics record bit for bit
+    saved = {k: _lib.get_option(k) for k in ("mix_cached", "stats_keep_mib")}
+    try:
+        for mix, keep in ((0, saved["stats_keep_mib"]), (0, 0)):
+            _lib.set_option("mix_cached", mix)
+            _lib.set_option("stats_keep_mib", keep)
+            announce(f"2^28 uniform mix_cached={mix} stats_keep_mib={keep}")
+            c2, l2, q2 = abi.uniform(x)
+            torch.cuda.synchronize()
+            assert torch.equal(c2, codes) and torch.equal(l2.view(torch.int32), lut.view(torch.int32))
+            assert torch.equal(q2.view(torch.int64), qp.view(torch.int64))
+    finally:
+        for k, v in saved.items():
+            _lib.set_option(k, v)
 
 
 def test_ring_reduce_step_2p26_chunks(abi):

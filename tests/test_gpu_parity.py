@@ -456,7 +456,7 @@ def test_literal_path_matches_the_large_digests_of_the_compiled_reference(abi, n
                                            ("reverse_second_pass", (0, 1)), ("one_shot", (0, 1)),
                                            ("one_shot_store_policy", (0, 2, 16)), ("two_row_below_mi_elems", (0, 128)),
                                            ("set_four_rows_max_mi_elems", (0, 32)), ("grid_cap", (0, 7, 64)),
-                                           ("large_read_grid_eighths", (0, 3, 7)), ("large_read_min_mi_elems", (0, 128)), ("stats_grid_eighths", (0, 3, 6)),
+                                           ("large_read_grid_eighths", (0, 3, 7)), ("large_read_min_mi_elems", (0, 128)), ("stats_grid_eighths", (0, 3, 6)), ("mix_cached", (0, 1)), ("mixed_grid_eighths", (0, 7, 8)),
                                            ("f32_store_policy", (0, 2, 16)), ("copy_store_policy", (0, 2, 16)),
                                            ("dynamic_tail_percent", (0, 5, 100)), ("dynamic_tail_min_mi_elems", (0, 128)),
                                            ("segment_blocks_per_cu", (1, 2, 4))])
@@ -500,6 +500,49 @@ def test_every_setting_of_the_tuning_options_gives_the_same_results(abi, oracle,
         _lib.set_option(option, old)
         if option == "stats_grid_eighths":
             _lib.set_option("large_read_min_mi_elems", old_large)
+
+
+def test_the_walk_that_spreads_the_cached_end_among_the_rest_gives_the_same_results_bit_for_bit(abi, oracle):
+    # From twice the kept size up, the quantize pass of uniform_8bit_quantize visits the end of the tensor (which the
+    # statistics pass left in the last-level cache) spread among its other tiles.  The order of the tiles changes
+    # nothing: made to act on small tensors (1 MiB kept, a grid of 7 so that there are many rounds of tiles), with
+    # and without tiles dealt on demand, two- and four-row tiles, against the plain walk and the oracle.
+    rng = np.random.default_rng(78)
+    names = ("stats_keep_mib", "mix_cached", "grid_cap", "dynamic_tail_percent", "dynamic_tail_min_mi_elems", "two_row_below_mi_elems")
+    saved = {k: _lib.get_option(k) for k in names}
+    try:
+        _lib.set_option("stats_keep_mib", 1)
+        _lib.set_option("grid_cap", 7)
+        _lib.set_option("dynamic_tail_min_mi_elems", 0)
+        for two_row in (128, 0):
+            _lib.set_option("two_row_below_mi_elems", two_row)
+            for n in (524_288 + 4096, 1_000_003, 3_300_001):          # just over twice the kept size; ragged; many rounds
+                x = (rng.standard_normal(n) * 1e-3).astype(np.float32)
+                x[rng.integers(0, n, 10)] = np.float32(0.9)
+                xt = abi.to_dev(x)
+                want = None
+                for mix, percent in ((0, 0), (1, 0), (1, 5), (1, 50), (0, 50)):
+                    _lib.set_option("mix_cached", mix)
+                    _lib.set_option("dynamic_tail_percent", percent)
+                    announce(f"mixed walk {mix} dynamic {percent} % n={n} two_row_below={two_row}")
+                    codes, lut, qp = abi.uniform(xt)
+                    torch.cuda.synchronize()
+                    got = [codes.cpu().numpy(), lut.cpu().numpy().view(np.uint32), qp.cpu().numpy().view(np.uint64)]
+                    if want is None:
+                        want = got
+                        q = abi.qparams(qp)
+                        oc, _, _ = oracle.uniform_8bit_quantize(x, "given", scale=float(q["scale"]))
+                        assert q["scale"] == oracle.scale_exact(x) and np.array_equal(got[0], oc)
+                        mean, _ = oracle.average_buckets_f64(x, oc)
+                        assert lut_rel_err(lut.cpu().numpy(), mean, float(q["scale"])) <= LUT_TOL
+                        continue
+                    assert np.array_equal(got[0], want[0]) and np.array_equal(got[2], want[2]), (n, mix, percent)
+                    # entries 0 and 255 may hold elements beyond the fixed-point range, added as fp64 in arrival order
+                    assert np.array_equal(got[1][1:255], want[1][1:255]), (n, mix, percent)
+                    assert np.allclose(got[1][[0, 255]].view(np.float32), want[1][[0, 255]].view(np.float32), rtol=1e-6, atol=0)
+    finally:
+        for k, v in saved.items():
+            _lib.set_option(k, v)
 
 
 def test_tiles_dealt_on_demand_give_the_results_of_the_round_robin_deal_bit_for_bit(abi, oracle):
