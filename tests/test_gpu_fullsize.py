@@ -103,6 +103,47 @@ def test_ring_reduce_step_2p26_chunks(abi):
         del want, acc
 
 
+def test_ring_reduce_step_2p28_all_three_kinds(abi):
+    # the ring steps at the size the second headline figure is quoted on (1 GiB accumulators: hinted loads in the
+    # accumulate pass, four-row tiles and tiles on demand in the quantize pass that follows a writer): reduce,
+    # reduce with the division of AVG, gather; accumulator bit for bit against torch, codes recomputed from the
+    # derived scale, table against the bin means
+    n = 1 << 28
+    msg = torch.randn(n, device=abi.dev, generator=torch.Generator(device=abi.dev).manual_seed(40)) * 1e-3
+    mc, ml, _ = abi.uniform(msg)
+    del msg
+    for kind, divisor in (("reduce", None), ("reduce_div", 8.0), ("gather", None)):
+        acc = torch.randn(n, device=abi.dev, generator=torch.Generator(device=abi.dev).manual_seed(41)) * 1e-3
+        if kind == "gather":
+            want = ml[mc.long()]
+        else:
+            want = acc + ml[mc.long()]
+            if divisor:
+                want = want / divisor
+        announce(f"2^28 ring step {kind}")
+        codes, lut, qp = abi.ring_step(acc, mc, ml, gather=(kind == "gather"), divisor=divisor)
+        torch.cuda.synchronize()
+        assert torch.equal(acc.view(torch.int32), want.view(torch.int32))
+        del acc
+        q = abi.qparams(qp)
+        sumsq = float((want.double() ** 2).sum())
+        assert abs(q["sumsq"] - sumsq) <= 1e-12 * sumsq
+        exact = np.float32(6.0 * (float(np.float32(np.sqrt(sumsq))) / np.sqrt(n - 1)) / 256.0)
+        assert abs(float(q["scale"]) - float(exact)) <= 1e-6 * float(exact)
+        inv = float(torch.tensor(1.0, dtype=torch.float32) / torch.tensor(float(q["scale"]), dtype=torch.float32))
+        p = want * inv
+        r = torch.where((p - torch.trunc(p)).abs() == 0.5, torch.trunc(p) + torch.sign(p), torch.round(p))
+        assert torch.equal(codes, (r.clamp(-128, 127) + 128).to(torch.uint8))
+        del p, r
+        cnt = torch.bincount(codes.int(), minlength=256)
+        assert int(cnt.sum()) == n
+        sums = torch.bincount(codes.int(), weights=want.double(), minlength=256)
+        mean = torch.where(cnt > 0, sums / cnt.clamp(min=1).double(), torch.zeros_like(sums))
+        floor = torch.tensor(float(q["scale"]), device=abi.dev, dtype=torch.float64)
+        assert float(((lut.double() - mean).abs() / torch.maximum(mean.abs(), floor)).max()) <= 1e-6
+        del want, codes
+
+
 def test_config2_all_22_layer_buckets(abi):
     # benchmark configuration 2 in full: 22 per-layer buckets of 51,380,224 elements, Student-t(3) * 1e-4
     # (heavy tails: the clip bins fill), quantized bucket by bucket; every bucket is checked on the
