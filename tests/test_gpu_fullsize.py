@@ -72,6 +72,45 @@ def test_uniform_8bit_quantize_2p28_properties(abi):
             _lib.set_option(k, v)
 
 
+@pytest.mark.parametrize("n", [70_000_001, (1 << 27), (1 << 27) + 4096 * 3 + 5, 200_000_003])
+def test_large_tensors_around_the_cache_thresholds(abi, n):
+    # 267 MiB (the end kept, walked from the end), 512 MiB (exactly twice the kept size: the mixed walk begins), a ragged
+    # size just above, 763 MiB with an odd element count: codes against the formula, counts, and the same call with the
+    # cache-aware paths switched off bit for bit
+    x = torch.randn(n, device=abi.dev, generator=torch.Generator(device=abi.dev).manual_seed(n % 1000)) * 1e-3
+    x[n // 3] = 0.9                                         # beyond the fixed-point range: the fp64 side sums
+    announce(f"large uniform n={n}")
+    codes, lut, qp = abi.uniform(x)
+    torch.cuda.synchronize()
+    q = abi.qparams(qp)
+    sumsq = float((x.double() ** 2).sum())
+    assert abs(q["sumsq"] - sumsq) <= 1e-12 * sumsq
+    inv = float(torch.tensor(1.0, dtype=torch.float32) / torch.tensor(float(q["scale"]), dtype=torch.float32))
+    p = x * inv
+    r = torch.where((p - torch.trunc(p)).abs() == 0.5, torch.trunc(p) + torch.sign(p), torch.round(p))
+    assert torch.equal(codes, (r.clamp(-128, 127) + 128).to(torch.uint8))
+    del p, r
+    cnt = torch.bincount(codes.int(), minlength=256)
+    assert int(cnt.sum()) == n
+    sums = torch.bincount(codes.int(), weights=x.double(), minlength=256)
+    mean = torch.where(cnt > 0, sums / cnt.clamp(min=1).double(), torch.zeros_like(sums))
+    floor = torch.tensor(float(q["scale"]), device=abi.dev, dtype=torch.float64)
+    assert float(((lut.double() - mean).abs() / torch.maximum(mean.abs(), floor)).max()) <= 1e-6
+    saved = {k: _lib.get_option(k) for k in ("mix_cached", "stats_keep_mib")}
+    try:
+        _lib.set_option("mix_cached", 0)
+        _lib.set_option("stats_keep_mib", 0)
+        announce(f"large uniform n={n}, plain walk")
+        c2, l2, q2 = abi.uniform(x)
+        torch.cuda.synchronize()
+        assert torch.equal(c2, codes) and torch.equal(q2.view(torch.int64), qp.view(torch.int64))
+        assert torch.equal(l2.view(torch.int32)[1:255], lut.view(torch.int32)[1:255])        # one far element, in entry 255
+        assert torch.allclose(l2[[0, 255]], lut[[0, 255]], rtol=1e-6, atol=0)
+    finally:
+        for k, v in saved.items():
+            _lib.set_option(k, v)
+
+
 def test_ring_reduce_step_2p26_chunks(abi):
     # benchmark configuration 3 in full: W = 8 ranks' 2^26-element chunks N(0, 1e-3), seed = rank; chunk 0 is
     # quantized, then all 7 hops of dequantize-add + requantize, each checked through properties
