@@ -169,7 +169,9 @@ int prime_uniform_8bit_quantize_literal(const float* x, int64_t n, uint8_t* code
 /* Large buckets, pipelined: bucket i is quantized as prime_uniform_8bit_quantize would, on
  * streams[i % n_streams] with workspaces[i % n_streams], so that the statistics pass of one
  * bucket overlaps the quantize pass and the launch ramps of its neighbours (two streams
- * give +5 % on 205 MB buckets, more of them less).  This is the loop over per-layer buckets of
+ * give +5 % on 205 MB buckets, more of them less; a set that holds a bucket of 2^27 elements or more runs on
+ * streams[0] alone: such a bucket fills the device by itself, and a neighbour on another stream would displace what
+ * it keeps in the last-level cache between its passes).  This is the loop over per-layer buckets of
  * Diloco.sync_pseudo_gradient (src/zeroband/diloco.py:108-110) without the network in between.
  * xs, ns, codes, workspaces and streams are host arrays; luts is count x 256 on the device and
  * qparams_out (optional) count records.  The caller orders the streams against its own work. */

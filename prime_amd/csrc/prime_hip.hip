@@ -783,6 +783,12 @@ int prime_uniform_8bit_quantize_buckets(const float* const* xs, const int64_t* n
         return fail(PRIME_EINVAL, "prime_uniform_8bit_quantize_buckets: bad argument");
     for (int k = 0; k < n_streams; ++k)
         if (!workspaces[k]) return fail(PRIME_EWORKSPACE, "prime_uniform_8bit_quantize_buckets: a workspace is null");
+    // Several streams pay off while a bucket leaves part of the device idle at its ramps.  A bucket of 2^27 elements or
+    // more fills the device on its own and keeps its end in the last-level cache between its two passes, which a
+    // neighbour on another stream would displace (8 x 2^27 elements: 1.47 ms on one stream, 1.54 ms on two; 6 x 2^28:
+    // 2.12 against 2.40 ms): with such a bucket in the set everything goes to the first stream.
+    for (int64_t i = 0; i < count; ++i)
+        if (ns[i] >= g_opt.large_read_min_elems) n_streams = 1;
     for (int64_t i = 0; i < count; ++i) {
         const int k = static_cast<int>(i % n_streams);
         if (int rc = uniform_checked(xs[i], ns[i], codes[i], luts + i * kBins, qparams_out ? qparams_out + i : nullptr,

@@ -1285,6 +1285,17 @@ def test_pipelined_buckets_equal_one_by_one(abi, oracle, n_streams):
     for i in range(len(xs)):
         c1, l1, q1 = abi.uniform(xs[i])
         assert torch.equal(codes[i], c1) and torch.equal(luts[i], l1)
+    # a set that holds a "large" bucket goes to the first stream alone (made to apply here by calling these buckets large)
+    saved = _lib.get_option("large_read_min_mi_elems")
+    try:
+        _lib.set_option("large_read_min_mi_elems", 1)
+        plan.run()
+        torch.cuda.synchronize()
+        for i in range(len(xs)):
+            c1, l1, q1 = abi.uniform(xs[i])
+            assert torch.equal(codes[i], c1) and torch.equal(luts[i], l1) and torch.equal(qps[i], q1)
+    finally:
+        _lib.set_option("large_read_min_mi_elems", saved)
 
 
 def test_fused_pass_codes_for_every_float_within_and_around_the_fixed_point_range(abi, oracle):
